@@ -1,0 +1,521 @@
+// Mixed INT4 / FP6-e3m2 weight-only GEMM for gfx950 (MI355X):  C[m,n] = A[m,k] . deq(B)[k,n] * s
+//
+// Replaces the device kernel and host dispatcher of liuchuan22/FP6-Marlin
+// (fp6_marlin/fp6_marlin_cuda_kernel.cu:288-951).  Same packed operands, a different machine mapping:
+//
+//  * One wavefront (64 lanes) owns a 128-column tile (two 64-column groups of the packed layout) and a
+//    contiguous range of k.  It streams the packed words with linear, fully coalesced 16-byte-per-lane
+//    loads (1 KiB per k-block and tile), turns them through a wave-private LDS slab so that the
+//    fragment owner's k-pair index becomes the high lane bits, dequantises in registers and feeds
+//    v_mfma_f32_16x16x32_f16 with the *weights as the 16-row operand* (C^T = W^T A^T), so a single
+//    MFMA covers 16 columns x 32 k for up to 16 rows of A.  No workgroup barrier in the main loop.
+//  * A workgroup is four such waves splitting k; they are summed through LDS.  `ksplit` workgroups may
+//    share a tile; each writes its fp32 partial tile to a per-device scratch, and the workgroup that
+//    arrives last (one atomic counter per tile in `workspace`) sums the partials in a fixed order,
+//    applies the scales and writes fp16 C.  Nobody spins, so there is nothing to deadlock on, and the
+//    counters are zero again when the launch drains.
+//  * INT4 and FP6 tiles are entries of one tile list handled by the same launch.
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+#include <mutex>
+
+#include "fp6m.h"
+#include "fp6m_layout.h"
+
+namespace fp6m {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;        // four wavefronts
+constexpr int kWaves = 4;
+constexpr int kTileN = 128;          // columns per tile
+constexpr int kRedStride = kTileN + 4;                       // floats per row of the reduction slab
+constexpr int kRedBytes = kWaves * 16 * kRedStride * 4;      // one 16-row block from every wave
+constexpr int kSlabBytes = 3072;                             // per wave: 2 x 1 KiB (4-bit) + 2 x 512 B (2-bit)
+constexpr size_t kScratchBytes = size_t(64) << 20;           // per-device partial-sum scratch
+
+struct GemmArgs {
+    const uint16_t* A;
+    const uint32_t* b_int4;   // INT4 words
+    const uint32_t* b_fp6_2;  // FP6 2-bit plane
+    const uint32_t* b_fp6_4;  // FP6 4-bit plane
+    uint16_t* C;
+    const uint16_t* s_int4;   // per-column (permuted order) or [k/128][n4] group scales
+    const uint16_t* s_fp6;    // per-column (permuted order)
+    float* scratch;
+    int* counters;
+    int m, n, k;
+    int n4, qc;               // columns in the INT4 / FP6 region
+    int tiles6;               // FP6 tiles come first in the tile list
+    int tiles;                // all tiles
+    int ksplit;               // workgroups per (tile, m-tile)
+};
+
+// ------------------------------------------------------------------------------------------------ bit tricks
+
+__device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
+
+// Eight INT4 weights of one packed word -> (e0,e1) (e2,e3) (e4,e5) (e6,e7), value = nibble - 8.
+// 0x6400 | u is the half 1024 + u;  0x6400 | (u << 4) is 1024 + 16 u.
+__device__ __forceinline__ void dequant_int4(uint32_t q, h2 (&r)[4])
+{
+    const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+    const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+    r[0] = as_h2((q & 0x000f000fu) | 0x64006400u) - bias_lo;
+    r[1] = __builtin_elementwise_fma(as_h2((q & 0x00f000f0u) | 0x64006400u), mul_hi, bias_hi);
+    const uint32_t q8 = q >> 8;
+    r[2] = as_h2((q8 & 0x000f000fu) | 0x64006400u) - bias_lo;
+    r[3] = __builtin_elementwise_fma(as_h2((q8 & 0x00f000f0u) | 0x64006400u), mul_hi, bias_hi);
+}
+
+// Eight FP6 weights from the tile's 2-bit word (already shifted so the tile's fields are the top two
+// bits of every byte) and its 4-bit word.  A byte `s eee mm 00` moved to s 00eee mm 0000 0000 is the
+// half value * 2^-12 (sub-normal codes become half sub-normals); the multiply by 4096 is exact.
+__device__ __forceinline__ void dequant_fp6(uint32_t q2, uint32_t q4, h2 (&r)[4])
+{
+    const h2 unbias = {(_Float16)4096.0f, (_Float16)4096.0f};
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const uint32_t p = (q2 & 0xc0c0c0c0u) | ((q4 & 0xf0f0f0f0u) >> 2);  // bytes, MSB first: e1 e3 e0 e2 (then e5 e7 e4 e6)
+        const uint32_t a = (p & 0x80008000u) | ((p & 0x7c007c00u) >> 2);
+        const uint32_t p8 = p << 8;
+        const uint32_t b = (p8 & 0x80008000u) | ((p8 & 0x7c007c00u) >> 2);
+        r[2 * half + 0] = as_h2(a) * unbias;
+        r[2 * half + 1] = as_h2(b) * unbias;
+        q2 <<= 2;
+        q4 <<= 4;
+    }
+}
+
+__device__ __forceinline__ h8 join(h2 a, h2 b, h2 c, h2 d)
+{
+    h8 v;
+    v[0] = a[0]; v[1] = a[1]; v[2] = b[0]; v[3] = b[1];
+    v[4] = c[0]; v[5] = c[1]; v[6] = d[0]; v[7] = d[1];
+    return v;
+}
+
+// Orders this wave's LDS writes before its LDS reads (and the reverse) for the compiler.  The LDS
+// unit executes one wave's instructions in order, so no hardware wait is needed.
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup b of a 1-D grid runs on XCD b % 8.  Renumber so that every XCD sees a contiguous range of
+// logical ids: workgroups that share a tile (adjacent logical ids) then share an L2.
+__device__ __forceinline__ int xcd_contiguous_id(int b, int total)
+{
+    const int q = total >> 3, r = total & 7, x = b & 7;
+    return x * q + (x < r ? x : r) + (b >> 3);
+}
+
+// ------------------------------------------------------------------------------------------------ kernel
+
+template <int MB>
+struct Stage {
+    u4 w4[2];            // 4-bit plane / INT4 words of k-blocks 2s, 2s+1 (this lane's linear 16 bytes)
+    u2 w2[2];            // FP6 2-bit plane (this lane's linear 8 bytes)
+    uint32_t a[MB][4];   // activations, already in MFMA operand order
+};
+
+template <int MB, bool G128>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes];
+    __shared__ int s_is_last;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int tile = logical / p.ksplit;
+    const int part = logical - tile * p.ksplit;
+    const int mtile = blockIdx.y;
+    const bool fp6 = tile < p.tiles6;
+    const int tcol = fp6 ? tile : tile - p.tiles6;          // tile index inside its region
+    const int region_n = fp6 ? p.qc : p.n4;
+    const int col0 = (fp6 ? p.n4 : 0) + tcol * kTileN;      // first column of the tile in C
+
+    // k range of this wave, in steps of 32 (two k-blocks); group-aligned when scales are per group.
+    const int unit_steps = G128 ? 4 : 1;
+    const int units = p.k / (32 * unit_steps);
+    const int nwaves = p.ksplit * kWaves;
+    const int wv = part * kWaves + wave;
+    const int step_begin = (int)((long long)units * wv / nwaves) * unit_steps;
+    const int step_end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
+
+    // MFMA-side identity of this lane: k-pair index i, column slot c = 8*sigma + l.
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+    const int owner = 32 * sigma + 4 * l + i;               // linear 16-byte granule of (group sigma, owner 4l+i)
+    unsigned char* slab = smem + wave * kSlabBytes;
+    const int wr4 = (lane ^ ((lane >> 4) & 3)) * 16;        // swizzled so both sides are bank-conflict free
+    const int rd4 = (owner ^ ((owner >> 4) & 3)) * 16;
+    const int wr2 = (lane ^ ((lane >> 5) << 1)) * 8;
+    const int rd2 = (owner ^ ((owner >> 5) << 1)) * 8;
+
+    // Global pointers.  A k-block of a region is one row of region_n*8 bytes (4-bit) / region_n*4 (2-bit).
+    const size_t row4 = (size_t)region_n * 8, row2 = (size_t)region_n * 4;
+    const unsigned char* g4 = reinterpret_cast<const unsigned char*>(fp6 ? p.b_fp6_4 : p.b_int4) +
+                              (size_t)tcol * 1024 + lane * 16;
+    const unsigned char* g2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)tcol * 512 + lane * 8;
+
+    const uint16_t* a_row[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        int row = mtile * 16 * MB + 16 * mb + c;
+        row = row < p.m ? row : p.m - 1;
+        a_row[mb] = p.A + (size_t)row * p.k + 2 * i;
+    }
+
+    auto load = [&](Stage<MB>& st, int s) {
+        const unsigned char* src4 = g4 + (size_t)(2 * s) * row4;
+        st.w4[0] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4));
+        st.w4[1] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4 + row4));
+        if (fp6) {
+            const unsigned char* src2 = g2 + (size_t)(2 * s) * row2;
+            st.w2[0] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2));
+            st.w2[1] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2 + row2));
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                st.a[mb][d] = *reinterpret_cast<const uint32_t*>(a_row[mb] + 32 * s + 8 * d);
+    };
+
+    f4 acc[MB][8];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
+
+    h2 gscale[8];  // G128, INT4 tiles: scale of column (j, half) duplicated into both halves
+    auto load_group_scales = [&](int s) {
+        const uint16_t* srow = p.s_int4 + (size_t)(s >> 2) * p.n4 + tcol * kTileN + 64 * sigma + l;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint16_t v = srow[16 * (t >> 1) + 8 * (t & 1)];
+            gscale[t] = as_h2((uint32_t)v | ((uint32_t)v << 16));
+        }
+    };
+
+    auto consume = [&](Stage<MB>& st, int s) {
+        wave_lds_fence();
+        *reinterpret_cast<u4*>(slab + wr4) = st.w4[0];
+        *reinterpret_cast<u4*>(slab + 1024 + wr4) = st.w4[1];
+        if (fp6) {
+            *reinterpret_cast<u2*>(slab + 2048 + wr2) = st.w2[0];
+            *reinterpret_cast<u2*>(slab + 2560 + wr2) = st.w2[1];
+        }
+        wave_lds_fence();
+        const u4 q0 = *reinterpret_cast<const u4*>(slab + rd4);
+        const u4 q1 = *reinterpret_cast<const u4*>(slab + 1024 + rd4);
+        u2 t0 = {0, 0}, t1 = {0, 0};
+        if (fp6) {
+            t0 = *reinterpret_cast<const u2*>(slab + 2048 + rd2);
+            t1 = *reinterpret_cast<const u2*>(slab + 2560 + rd2);
+        }
+        if (G128 && !fp6 && (s & 3) == 0) load_group_scales(s);
+
+        h8 av[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            u4 raw = {st.a[mb][0], st.a[mb][1], st.a[mb][2], st.a[mb][3]};
+            av[mb] = __builtin_bit_cast(h8, raw);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h2 r0[4], r1[4];
+            if (fp6) {
+                dequant_fp6(t0[j >> 1] << (4 * (j & 1)), q0[j], r0);
+                dequant_fp6(t1[j >> 1] << (4 * (j & 1)), q1[j], r1);
+            } else {
+                dequant_int4(q0[j], r0);
+                dequant_int4(q1[j], r1);
+                if (G128) {
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        r0[x] = r0[x] * gscale[2 * j + (x >> 1)];
+                        r1[x] = r1[x] * gscale[2 * j + (x >> 1)];
+                    }
+                }
+            }
+            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
+            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                acc[mb][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av[mb], acc[mb][2 * j + 0], 0, 0, 0);
+                acc[mb][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av[mb], acc[mb][2 * j + 1], 0, 0, 0);
+            }
+        }
+    };
+
+    // Two stages of loads stay in flight in registers while the current one is consumed.
+    Stage<MB> st0, st1;
+    int s = step_begin;
+    if (s < step_end) load(st0, s);
+    if (s + 1 < step_end) load(st1, s + 1);
+    for (; s < step_end; s += 2) {
+        consume(st0, s);
+        if (s + 2 < step_end) load(st0, s + 2);
+        if (s + 1 < step_end) {
+            consume(st1, s + 1);
+            if (s + 3 < step_end) load(st1, s + 3);
+        }
+    }
+
+    // ---- epilogue: sum the four waves through LDS, then either finish or hand over a partial tile.
+    // MFMA result layout: lane (m = lane & 15, q = lane >> 4) holds column slots 4q .. 4q+3.
+    const int q = lane >> 4;
+    float* red = reinterpret_cast<float*>(smem);
+    const int out_m = threadIdx.x >> 4;          // row inside the 16-row block
+    const int out_n = (threadIdx.x & 15) * 8;    // first of eight consecutive columns
+    const size_t tile_floats = (size_t)MB * 16 * kTileN;
+    float* my_partial = p.scratch + ((size_t)(mtile * p.tiles + tile) * p.ksplit + part) * tile_floats;
+
+    const bool per_column_scale = fp6 || !G128;
+    float sc[8];
+    if (per_column_scale) {
+        const uint16_t* sp = (fp6 ? p.s_fp6 : p.s_int4);
+        const int nr = tcol * kTileN + out_n;    // column inside the region, multiple of 8
+        const int base = (nr & ~31) + 4 * ((nr >> 4) & 1) + 2 * ((nr >> 3) & 1);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint16_t v = sp[base + 8 * (e >> 1) + (e & 1)];
+            sc[e] = (float)__builtin_bit_cast(_Float16, v);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) sc[e] = 1.0f;
+    }
+
+    auto store_row = [&](int row, const float (&v)[8]) {
+        h8 o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = (_Float16)(v[e] * sc[e]);
+        *reinterpret_cast<h8*>(p.C + (size_t)row * p.n + col0 + out_n) = o;
+    };
+
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        __syncthreads();
+        float* mine = red + wave * 16 * kRedStride + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[mb][t];
+        __syncthreads();
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) {
+            const float* src = red + w * 16 * kRedStride + out_m * kRedStride + out_n;
+            const f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) { v[e] += lo[e]; v[4 + e] += hi[e]; }
+        }
+        const int row = mtile * 16 * MB + 16 * mb + out_m;
+        if (row < p.m) {
+            if (p.ksplit == 1) {
+                store_row(row, v);
+            } else {
+                float* dst = my_partial + (size_t)(16 * mb + out_m) * kTileN + out_n;
+                *reinterpret_cast<f4*>(dst) = f4{v[0], v[1], v[2], v[3]};
+                *reinterpret_cast<f4*>(dst + 4) = f4{v[4], v[5], v[6], v[7]};
+            }
+        }
+    }
+    if (p.ksplit == 1) return;
+
+    // Publish the partial, then count arrivals; the last workgroup of the tile finishes it.
+    __threadfence();
+    __syncthreads();
+    int* counter = p.counters + mtile * p.tiles + tile;
+    if (threadIdx.x == 0) {
+        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_is_last = (seen == p.ksplit - 1);
+    }
+    __syncthreads();
+    if (!s_is_last) return;
+    __threadfence();
+    const float* first = p.scratch + (size_t)(mtile * p.tiles + tile) * p.ksplit * tile_floats;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        const int row = mtile * 16 * MB + 16 * mb + out_m;
+        if (row >= p.m) continue;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = 0.f;
+        for (int pp = 0; pp < p.ksplit; pp++) {
+            const float* src = first + (size_t)pp * tile_floats + (size_t)(16 * mb + out_m) * kTileN + out_n;
+            const f4 lo = __builtin_nontemporal_load(reinterpret_cast<const f4*>(src));
+            const f4 hi = __builtin_nontemporal_load(reinterpret_cast<const f4*>(src + 4));
+#pragma unroll
+            for (int e = 0; e < 4; e++) { v[e] += lo[e]; v[4 + e] += hi[e]; }
+        }
+        store_row(row, v);
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ------------------------------------------------------------------------------------------------ host
+
+thread_local int g_last_hip_error = 0;
+
+struct DeviceScratch {
+    float* ptr = nullptr;
+    int cus = 0;
+};
+constexpr int kMaxDevices = 64;
+DeviceScratch g_scratch[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+int hip_fail(hipError_t e)
+{
+    g_last_hip_error = (int)e;
+    return FP6M_ERR_HIP;
+}
+
+int ensure_scratch(int dev, DeviceScratch** out)
+{
+    if (dev < 0 || dev >= kMaxDevices) return FP6M_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    DeviceScratch& d = g_scratch[dev];
+    if (!d.ptr) {
+        int prev = 0;
+        hipError_t e = hipGetDevice(&prev);
+        if (e != hipSuccess) return hip_fail(e);
+        if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) return hip_fail(e);
+        void* mem = nullptr;
+        e = hipMalloc(&mem, kScratchBytes);
+        int cus = 0;
+        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (prev != dev) (void)hipSetDevice(prev);
+        if (e != hipSuccess) return hip_fail(e);
+        d.ptr = static_cast<float*>(mem);
+        d.cus = cus > 0 ? cus : 256;
+    }
+    *out = &d;
+    return FP6M_OK;
+}
+
+template <int MB>
+void launch(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
+{
+    if (g128)
+        hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
+}
+
+}  // namespace fp6m
+
+extern "C" {
+
+int fp6m_last_hip_error(void) { return fp6m::g_last_hip_error; }
+
+int fp6m_init(int dev)
+{
+    fp6m::DeviceScratch* d = nullptr;
+    return fp6m::ensure_scratch(dev, &d);
+}
+
+int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+             void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
+             int quant_cols, int group_size)
+{
+    using namespace fp6m;
+    if (prob_m < 0 || prob_n < 0 || prob_k < 0) return FP6M_ERR_ARG;
+
+    // Tile-shape arguments are validated the way the reference does it
+    // (fp6_marlin_cuda_kernel.cu:890-905, 933-944) even though they do not pick a kernel here.
+    if (thread_k == -1 || thread_n == -1) {
+        thread_k = prob_m <= 16 ? 128 : 64;
+        thread_n = prob_m <= 16 ? 128 : 256;
+    }
+    if (thread_k <= 0 || thread_n <= 0) return FP6M_ERR_KERN_SHAPE;
+    if (prob_n % thread_n != 0 || prob_k % thread_k != 0) return FP6M_ERR_PROB_SHAPE;
+    if (prob_m == 0 || prob_n == 0 || prob_k == 0) return FP6M_OK;
+    const bool small_tile = thread_k == 128 && thread_n == 128;
+    const bool large_tile = thread_k == 64 && thread_n == 256;
+    if (!(large_tile || (small_tile && prob_m <= 16))) return FP6M_ERR_KERN_SHAPE;
+
+    if (!A || !B || !C || !s || !workspace) return FP6M_ERR_ARG;
+    if (max_par <= 0) return FP6M_ERR_ARG;
+    int qc = quant_cols <= 0 ? 0 : quant_cols;
+    if (quant_cols < -1 || qc > prob_n) return FP6M_ERR_ARG;
+    const int n4 = prob_n - qc;
+    if (n4 % kTileN || qc % kTileN) return FP6M_ERR_PROB_SHAPE;
+    if (group_size != -1 && group_size != 128) return FP6M_ERR_ARG;
+    const bool g128 = group_size == 128 && n4 > 0;
+    if (g128 && prob_k % 128) return FP6M_ERR_PROB_SHAPE;
+
+    DeviceScratch* scratch = nullptr;
+    if (int rc = ensure_scratch(dev, &scratch)) return rc;
+
+    GemmArgs a;
+    a.b_int4 = static_cast<const uint32_t*>(B);
+    a.b_fp6_2 = a.b_int4 + (size_t)prob_k * n4 / 8;
+    a.b_fp6_4 = a.b_fp6_2 + (size_t)prob_k * qc / 16;
+    a.s_int4 = static_cast<const uint16_t*>(s);
+    a.s_fp6 = a.s_int4 + (g128 ? (size_t)(prob_k / 128) * n4 : (size_t)n4);
+    a.scratch = scratch->ptr;
+    a.counters = static_cast<int*>(workspace);
+    a.n = prob_n;
+    a.k = prob_k;
+    a.n4 = n4;
+    a.qc = qc;
+    a.tiles6 = qc / kTileN;
+    a.tiles = prob_n / kTileN;
+
+    const int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
+    const int rows_per_tile = 16 * mb;
+    const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
+    const int units = g128 ? prob_k / 128 : prob_k / 32;
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int mt0 = 0; mt0 < mtiles_total; mt0 += max_par) {
+        const int mtiles = mtiles_total - mt0 < max_par ? mtiles_total - mt0 : max_par;
+        const int rows0 = mt0 * rows_per_tile;
+        a.A = static_cast<const uint16_t*>(A) + (size_t)rows0 * prob_k;
+        a.C = static_cast<uint16_t*>(C) + (size_t)rows0 * prob_n;
+        a.m = prob_m - rows0 < mtiles * rows_per_tile ? prob_m - rows0 : mtiles * rows_per_tile;
+
+        // How many workgroups share one tile's k range: enough to put several workgroups on every CU,
+        // never so many that a wave gets less than one unit of k, that the partial tiles outgrow the
+        // scratch, or that partial-sum traffic rivals the weight stream.
+        const long long base = (long long)a.tiles * mtiles;
+        const long long want_wgs = (long long)scratch->cus * 4;
+        long long ks = (want_wgs + base - 1) / base;
+        const long long ks_k = units / (kWaves * 2) > 0 ? units / (kWaves * 2) : 1;
+        if (ks > ks_k) ks = ks_k;
+        const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
+        if (ks > traffic_cap) ks = traffic_cap;
+        if (sms > 0 && ks > sms) ks = sms;
+        const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
+        while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
+        if (const char* e = getenv("FP6M_KSPLIT")) {
+            const int v = atoi(e);
+            if (v >= 1 && (size_t)base * v * tile_bytes <= kScratchBytes && v * kWaves <= units) ks = v;
+        }
+        if (ks < 1) ks = 1;
+        a.ksplit = (int)ks;
+
+        dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
+        if (mb == 1) launch<1>(a, g128, grid, st);
+        else if (mb == 2) launch<2>(a, g128, grid, st);
+        else launch<4>(a, g128, grid, st);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return hip_fail(e);
+    }
+    return FP6M_OK;
+}
+
+}  // extern "C"

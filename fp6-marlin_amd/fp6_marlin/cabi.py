@@ -1,0 +1,195 @@
+"""ctypes binding of the C ABI declared in include/fp6m.h (libfp6m.so, built by fp6-marlin_amd/build.py).
+
+Nothing here computes anything: every function checks shapes/dtypes, hands raw pointers to the shared
+library and maps its return code to the exception the reference raises for the same condition
+(std::invalid_argument -> ValueError for the CPU helpers, AT_ERROR -> RuntimeError for `mul`).
+There is no Python fallback: if the library is missing, importing this module fails.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfp6m.so")
+
+OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_RANGE, ERR_SHAPE, ERR_ARG, ERR_HIP, ERR_NO_GPU_CODE = range(8)
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} is missing: build it with `python fp6-marlin_amd/build.py` "
+        "(hipcc --offload-arch=gfx950); there is no fallback implementation")
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_vp, _sz, _int = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+lib.fp6m_strerror.restype = ctypes.c_char_p
+lib.fp6m_strerror.argtypes = [_int]
+lib.fp6m_last_hip_error.restype = _int
+lib.fp6m_abi_version.restype = _int
+lib.fp6m_workspace_elems.restype = _sz
+lib.fp6m_workspace_elems.argtypes = [_int, _int]
+lib.fp6m_init.argtypes = [_int]
+lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
+lib.fp6m_fp6_quantize.argtypes = [_vp, _vp, _sz, _sz]
+lib.fp6m_fp6_prepack.argtypes = [_vp, _vp, _sz, _sz]
+lib.fp6m_fp6_dequant.argtypes = [_vp, _vp, _sz, _sz, _vp]
+lib.fp6m_int4_quantize.argtypes = [_vp, _sz, _sz, _int, _vp, _vp, _vp]
+lib.fp6m_int4_pack.argtypes = [_vp, _vp, _sz, _sz]
+lib.fp6m_permute_scales.argtypes = [_vp, _vp, _sz]
+lib.fp6m_unpack_to_fp16.argtypes = [_vp, _vp, _vp, _sz, _sz, _int, _int]
+for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
+           lib.fp6m_int4_quantize, lib.fp6m_int4_pack, lib.fp6m_permute_scales, lib.fp6m_unpack_to_fp16):
+    _f.restype = _int
+
+
+def strerror(code):
+    return lib.fp6m_strerror(code).decode()
+
+
+def _raise_cpu(code):
+    if code != OK:
+        raise ValueError(strerror(code))
+
+
+def _cpu(t, dtype, name):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} should be of type {dtype}.")
+    if t.device.type != "cpu":
+        raise ValueError(f"{name} must be a CPU tensor")
+    return t.contiguous()
+
+
+# ------------------------------------------------------------------------------------------ host routines
+
+def fp6_quantize(w):
+    """float16 [OC, IC] -> int32 [IC, OC*3/16].  The flat row-major buffer is quantised as IC rows of OC
+    values and *labelled* transposed, exactly as fp6_marlin/pybind.cpp:42-59 does."""
+    w = _cpu(w, torch.float16, "Input tensor")
+    if w.dim() != 2 or w.shape[0] % 256 or w.shape[1] % 256:
+        raise ValueError("quantize expects a 2-D tensor with both dimensions multiples of 256")
+    oc, ic = w.shape
+    out = torch.empty((ic, oc // 16 * 3), dtype=torch.int32)
+    _raise_cpu(lib.fp6m_fp6_quantize(w.data_ptr(), out.data_ptr(), ic, oc))
+    return out
+
+
+def fp6_prepack(q):
+    """int32 [OC, IC*3/16] -> int32 [IC*3/32, OC*2] (2-bit plane then 4-bit plane), fp6_marlin/pybind.cpp:18-31."""
+    q = _cpu(q, torch.int32, "fp6 tensor")
+    if q.dim() != 2 or q.shape[1] % 3:
+        raise ValueError("prepacking expects int32 [OC, IC*3/16]")
+    oc, ic = q.shape[0], q.shape[1] * 16 // 3
+    if oc % 256 or ic % 256:
+        raise ValueError("prepacking expects OC and IC to be multiples of 256")
+    out = torch.empty((ic // 32 * 3, oc * 2), dtype=torch.int32)
+    _raise_cpu(lib.fp6m_fp6_prepack(out.data_ptr(), q.data_ptr(), oc, ic))
+    return out
+
+
+def fp6_dequant(q, scale):
+    """int32 [OC, IC*3/16], float16 [OC] -> float16 [OC, IC], fp6_marlin/pybind.cpp:70-87."""
+    q = _cpu(q, torch.int32, "fp6 tensor")
+    scale = _cpu(scale, torch.float16, "scales")
+    if q.dim() != 2 or q.shape[1] % 3 or scale.numel() != q.shape[0]:
+        raise ValueError("dequantize expects int32 [OC, IC*3/16] and float16 [OC]")
+    oc, ic = q.shape[0], q.shape[1] // 3 * 16
+    out = torch.empty((oc, ic), dtype=torch.float16)
+    _raise_cpu(lib.fp6m_fp6_dequant(out.data_ptr(), q.data_ptr(), oc, ic, scale.data_ptr()))
+    return out
+
+
+def int4_quantize(w, group_size=-1):
+    """float16 [k, n] -> (codes uint8 [k, n], scales float16 [k/group, n], w_ref float16 [k, n]); test.py:85-101."""
+    w = _cpu(w, torch.float16, "weight")
+    k, n = w.shape
+    g = k if group_size == -1 else group_size
+    if g <= 0 or k % g:
+        raise ValueError("group_size must be -1 or divide k")
+    codes = torch.empty((k, n), dtype=torch.uint8)
+    scales = torch.empty((k // g, n), dtype=torch.float16)
+    ref = torch.empty((k, n), dtype=torch.float16)
+    _raise_cpu(lib.fp6m_int4_quantize(w.data_ptr(), k, n, group_size, codes.data_ptr(), scales.data_ptr(), ref.data_ptr()))
+    return codes, scales, ref
+
+
+def int4_pack(codes):
+    """uint8 [k, n] in 0..15 -> int32 [k/16, n*2]; test.py:106-113."""
+    codes = _cpu(codes, torch.uint8, "codes")
+    k, n = codes.shape
+    out = torch.empty((k // 16, n * 2), dtype=torch.int32)
+    _raise_cpu(lib.fp6m_int4_pack(codes.data_ptr(), out.data_ptr(), k, n))
+    return out
+
+
+def permute_scales(s):
+    """float16 [..., n] -> same shape with the reference's 32-column scale permutation; test.py:80-83."""
+    s = _cpu(s, torch.float16, "scales")
+    out = torch.empty_like(s)
+    rows = s.numel() // s.shape[-1] if s.numel() else 0
+    for r in range(rows):
+        off = r * s.shape[-1] * 2
+        _raise_cpu(lib.fp6m_permute_scales(s.data_ptr() + off, out.data_ptr() + off, s.shape[-1]))
+    return out
+
+
+def unpack_to_fp16(B, s, k, n, quant_cols=-1, group_size=-1):
+    """Packed B / s (CPU tensors) -> dequantised float16 [k, n]."""
+    B = _cpu(B, torch.int32, "B")
+    s = _cpu(s, torch.float16, "s")
+    out = torch.empty((k, n), dtype=torch.float16)
+    _raise_cpu(lib.fp6m_unpack_to_fp16(B.data_ptr(), s.data_ptr(), out.data_ptr(), k, n, quant_cols, group_size))
+    return out
+
+
+# ------------------------------------------------------------------------------------------ the GEMM
+
+def workspace_elems(n, max_par=16):
+    return int(lib.fp6m_workspace_elems(n, max_par))
+
+
+def init(device=0):
+    code = lib.fp6m_init(int(device))
+    if code != OK:
+        raise RuntimeError(f"fp6m_init: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+
+
+def mul(A, B, C, s, workspace, quant_cols=-1, thread_k=-1, thread_n=-1, sms=-1, max_par=16, group_size=-1):
+    """C = A @ dequant(B) * s on the current HIP stream.  Argument order of fp6_marlin/__init__.py:39-40
+    (reference: fp6_marlin/fp6_marlin_cuda.cpp:47-92), plus `group_size`."""
+    for name, t in (("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise RuntimeError(f"{name} must be a tensor on the GPU")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+        if t.device != A.device:
+            raise RuntimeError("all operands must live on the same device")
+    if A.dtype != torch.float16 or C.dtype != torch.float16 or s.dtype != torch.float16:
+        raise RuntimeError("A, C and s must be float16")
+    if B.element_size() != 4 or workspace.element_size() != 4:
+        raise RuntimeError("B must be int32 (or another 4-byte type) and workspace a 4-byte type")
+    m, k = A.shape
+    n = C.shape[1]
+    if C.shape[0] != m:
+        raise RuntimeError("C must be [m, n]")
+    if workspace.numel() < n // 128 * max_par:                       # fp6_marlin_cuda.cpp:62-63
+        raise RuntimeError(f"workspace must be of size at least {n // 128 * max_par}.")
+    qc = 0 if quant_cols in (-1, 0) else quant_cols
+    n4 = n - qc
+    if k % 32 == 0 and 0 <= qc <= n:
+        need_b = k * n4 // 8 + k * qc * 3 // 16
+        need_s = (n4 if group_size == -1 else (k // 128) * n4) + qc
+        if B.numel() < need_b or s.numel() != need_s:                # a (2, n) scale tensor fails here, test.py:219-226
+            raise RuntimeError(f"B must hold {need_b} words and s {need_s} scales for this problem")
+    dev = A.device.index
+    stream = torch.cuda.current_stream(A.device).cuda_stream
+    code = lib.fp6m_mul(A.data_ptr(), B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k, workspace.data_ptr(),
+                        dev, stream, thread_k, thread_n, sms, max_par, quant_cols, group_size)
+    if code == ERR_PROB_SHAPE:
+        raise RuntimeError(f"Problem (m={m}, n={n}, k={k}) not compatible with thread_k={thread_k}, thread_n={thread_n}.")
+    if code == ERR_KERN_SHAPE:
+        raise RuntimeError(f"No kernel implementation for thread_k={thread_k}, thread_n={thread_n}.")
+    if code != OK:
+        raise RuntimeError(f"fp6m_mul: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")

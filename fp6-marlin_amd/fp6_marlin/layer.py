@@ -1,0 +1,126 @@
+"""Weight preparation and the ``Layer`` module.
+
+The reference keeps INT4 packing, the scale permutation and the mixed-weight concatenation in its test
+harness (test.py:13-152) and has no ``Layer``; here they are library functions backed by the C ABI.
+"""
+import torch
+import torch.nn as nn
+
+from . import cabi
+
+int4_quantize = cabi.int4_quantize
+int4_pack = cabi.int4_pack
+permute_scales = cabi.permute_scales
+unpack_to_fp16 = cabi.unpack_to_fp16
+
+FP6_MAX = 28.0
+FP6_MIN = 0.0625
+
+
+def _fp6_region(w):
+    """test.py:13-58 on a [k, nq] float16 slice whose storage is [k, nq] row-major.
+    Returns (B int32 [k*3/32, nq*2], s float16 [nq] permuted, w_ref float16 [k, nq])."""
+    k, nq = w.shape
+    s = torch.max(torch.abs(w), 0, keepdim=True)[0]
+    s *= 1.0 / FP6_MAX
+    s = s.reshape(-1, nq).contiguous().squeeze(0)
+    w = w / s
+    w = torch.where(torch.abs(w) < FP6_MIN, torch.zeros_like(w), w)
+    w = torch.clamp(w, -FP6_MAX, FP6_MAX)
+    q = cabi.fp6_quantize(w)                       # int32 [nq, k*3/16]: rows of the *flat* buffer
+    w_ref = cabi.fp6_dequant(q, s).transpose(0, 1).contiguous()
+    return cabi.fp6_prepack(q), cabi.permute_scales(s), w_ref
+
+
+def pack_mixed_weight(w, quant_cols=-1, group_size=-1, harness_layout=True):
+    """Quantise and pack a float16 weight ``w`` [k, n] into the operands of ``mul``.
+
+    The last ``quant_cols`` columns go to FP6 with one scale per column, the others to symmetric INT4
+    with one scale per column (``group_size=-1``) or per 128 rows and column (``group_size=128``).
+    Returns ``(B, s, w_ref)``: int32 1-D, float16 1-D, and the dequantised float16 [k, n] weight that
+    ``mul`` multiplies by (the reference's check weight, test.py:37-38, 98).
+
+    ``harness_layout=True`` reproduces the reference harness bit for bit, including the fact that its
+    FP6 path quantises the [k, nq] buffer as if it were [nq, k] (no transpose, pybind.cpp:52-57), so the
+    FP6 part of ``w_ref`` is a reshuffle of ``w``.  ``harness_layout=False`` transposes first, so that
+    ``w_ref`` approximates ``w`` column for column: use that for real models (``Layer.pack`` does).
+    """
+    if w.dtype != torch.float16 or w.dim() != 2:
+        raise ValueError("w must be a 2-D float16 tensor")
+    w = w.detach().cpu().contiguous()
+    k, n = w.shape
+    qc = 0 if quant_cols in (-1, 0) else quant_cols
+    if qc < 0 or qc > n or qc % 64:
+        raise ValueError("quant_cols must be -1 or a multiple of 64 not above n")
+    parts_b, parts_s, parts_ref = [], [], []
+    if n - qc:
+        w4 = w[:, : n - qc].contiguous()
+        codes, scales, ref = cabi.int4_quantize(w4, group_size)
+        parts_b.append(cabi.int4_pack(codes).reshape(-1))
+        parts_s.append((cabi.permute_scales(scales) if group_size == -1 else scales).reshape(-1))
+        parts_ref.append(ref)
+    if qc:
+        w6 = w[:, n - qc:].contiguous()
+        if harness_layout:
+            b6, s6, ref6 = _fp6_region(w6)
+        else:
+            # quantise the true transpose: feed quantize() a buffer whose flat view is [nq, k]
+            s6 = torch.max(torch.abs(w6), 0)[0] * (1.0 / FP6_MAX)
+            s6 = torch.where(s6 == 0, torch.ones_like(s6), s6)
+            t = (w6 / s6).transpose(0, 1).contiguous()            # [nq, k]
+            t = torch.where(torch.abs(t) < FP6_MIN, torch.zeros_like(t), t).clamp(-FP6_MAX, FP6_MAX)
+            q = cabi.fp6_quantize(t.reshape(k, qc))               # flat view read as [nq, k]
+            ref6 = cabi.fp6_dequant(q, s6).transpose(0, 1).contiguous()
+            b6, s6 = cabi.fp6_prepack(q), cabi.permute_scales(s6)
+        parts_b.append(b6.reshape(-1))
+        parts_s.append(s6.reshape(-1))
+        parts_ref.append(ref6)
+    return (torch.cat(parts_b).contiguous(), torch.cat(parts_s).contiguous(),
+            torch.cat(parts_ref, dim=1).contiguous())
+
+
+class Layer(nn.Module):
+    """Linear layer ``y = x @ W`` with W [infeatures, outfeatures] stored as mixed INT4 / FP6.
+
+    Buffers (all on the module's device):
+      ``B``          int32 1-D, the wire format of ``mul``
+      ``s``          float16 1-D: INT4 scales (per column in the reference's permuted order, or
+                     [infeatures/128, outfeatures-quant_cols] in natural column order when
+                     ``groupsize=128``) followed by the FP6 per-column scales (permuted order)
+      ``workspace``  int32 zeros, outfeatures // 128 * 16
+
+    ``quant_cols`` output features, the *last* ones, are kept in FP6.  To protect arbitrary "significant"
+    output channels, permute the columns of W so they come last (and un-permute y).
+    """
+
+    def __init__(self, infeatures, outfeatures, groupsize=-1, quant_cols=-1):
+        super().__init__()
+        if groupsize not in (-1, 128):
+            raise ValueError("Only groupsize -1 and 128 are supported.")
+        qc = 0 if quant_cols in (-1, 0) else quant_cols
+        if infeatures % 128 or outfeatures % 128 or qc % 128 or qc > outfeatures:
+            raise ValueError("infeatures, outfeatures and quant_cols must be multiples of 128")
+        self.k, self.n, self.groupsize, self.quant_cols = infeatures, outfeatures, groupsize, quant_cols
+        n4 = outfeatures - qc
+        words = infeatures * n4 // 8 + infeatures * qc * 3 // 16
+        nscale = (n4 if groupsize == -1 else infeatures // 128 * n4) + qc
+        self.register_buffer("B", torch.empty(words, dtype=torch.int32))
+        self.register_buffer("s", torch.empty(nscale, dtype=torch.float16))
+        self.register_buffer("workspace", torch.zeros(outfeatures // 128 * 16, dtype=torch.int32), persistent=False)
+
+    def pack(self, linear):
+        """Quantise and pack ``linear`` (an ``nn.Linear`` or a float16 weight [outfeatures, infeatures])."""
+        w = linear.weight.data if isinstance(linear, nn.Module) else linear
+        w = w.detach().to(torch.float16).cpu().t().contiguous()      # [k, n]
+        if tuple(w.shape) != (self.k, self.n):
+            raise ValueError("weight shape does not match the layer")
+        B, s, w_ref = pack_mixed_weight(w, self.quant_cols, self.groupsize, harness_layout=False)
+        self.B.copy_(B)
+        self.s.copy_(s)
+        return w_ref
+
+    def forward(self, x):
+        x2 = x.reshape(-1, x.shape[-1]).to(torch.float16).contiguous()
+        out = torch.empty((x2.shape[0], self.n), dtype=torch.float16, device=x2.device)
+        cabi.mul(x2, self.B, out, self.s, self.workspace, self.quant_cols, -1, -1, -1, 16, self.groupsize)
+        return out.reshape(x.shape[:-1] + (self.n,))

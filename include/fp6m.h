@@ -1,0 +1,142 @@
+/*
+ * fp6m.h -- C ABI of the MI355X (gfx950) mixed INT4 / FP6-e3m2 weight-only GEMM.
+ *
+ * Plain pointers and sizes only; no torch, no HIP types (a stream is passed as
+ * the opaque `hipStream_t` pointer value).  Every entry point cites the
+ * interface of liuchuan22/FP6-Marlin it replaces (paths relative to that
+ * repository).  All functions return FP6M_OK (0) or one of the codes below and
+ * never throw across the boundary.
+ *
+ * Matrix conventions (identical to the reference):
+ *   A  [m, k] fp16 row-major, device
+ *   C  [m, n] fp16 row-major, device, fully overwritten
+ *   B  1-D int32, device:  INT4 words of columns [0, n-quant_cols)       (k * (n-quant_cols) / 8  words)
+ *                       || FP6 "2-bit" words of the last quant_cols columns  (k * quant_cols / 16      words)
+ *                       || FP6 "4-bit" words of the same columns             (k * quant_cols / 8       words)
+ *      exactly what test.py:123-152 (gen_mixed_weight) concatenates.
+ *   s  fp16, device: INT4 scales || FP6 scales.  Per-column scales are stored
+ *      in the reference's permuted order (test.py:80-83); INT4 group scales
+ *      (group_size = 128) are [k/128, n-quant_cols] in natural column order.
+ */
+#ifndef FP6M_H_
+#define FP6M_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP6M_OK              0
+#define FP6M_ERR_PROB_SHAPE  1 /* fp6_marlin_cuda_kernel.cu:861  n or k not divisible by the tile   */
+#define FP6M_ERR_KERN_SHAPE  2 /* fp6_marlin_cuda_kernel.cu:862  no kernel for (thread_k, thread_n) */
+#define FP6M_ERR_RANGE       3 /* weight_quant.cpp:48-53 throws std::invalid_argument                */
+#define FP6M_ERR_SHAPE       4 /* weight_quant.cpp:112, weight_prepacking.cpp:124-125,182-183, pybind.cpp:22-24,50 */
+#define FP6M_ERR_ARG         5 /* null pointer, unsupported group_size / quant_cols                  */
+#define FP6M_ERR_HIP         6 /* a HIP runtime call failed; fp6m_last_hip_error() has the code      */
+#define FP6M_ERR_NO_GPU_CODE 7 /* the library was built without its gfx950 kernels                   */
+
+/* Human-readable text for a return code (static storage). */
+const char* fp6m_strerror(int code);
+/* hipError_t of the most recent failing HIP call on this thread (0 if none). */
+int fp6m_last_hip_error(void);
+/* ABI version of this header: bumped on any incompatible change. */
+int fp6m_abi_version(void);
+
+/*
+ * The GEMM.  Replaces
+ *   int fp6_marlin_cuda(const void* A, const void* B, void* C, void* s, int prob_m, int prob_n,
+ *                       int prob_k, void* workspace, int dev, cudaStream_t stream, int thread_k,
+ *                       int thread_n, int sms, int max_par, int quant_cols)
+ *   (fp6_marlin/fp6_marlin_cuda_kernel.cu:864-951, declared again fp6_marlin/fp6_marlin_cuda.cpp:26-42).
+ *
+ * Same argument order and meaning, plus `group_size` at the end:
+ *   workspace   >= fp6m_workspace_elems(prob_n, max_par) 4-byte elements of device memory, all zero
+ *               on entry; it is all zero again when the call's work has finished (same contract as
+ *               the reference's lock array, fp6_marlin_cuda_kernel.cu:90-92).
+ *   dev, stream device ordinal and hipStream_t; the call is asynchronous on `stream`.
+ *   thread_k, thread_n  -1/-1 = automatic.  Otherwise validated exactly like the reference:
+ *               (128,128) only for prob_m <= 16, (64,256) for any m; anything else -> ERR_KERN_SHAPE;
+ *               prob_n % thread_n or prob_k % thread_k -> ERR_PROB_SHAPE.  They do not select a
+ *               different kernel here (tile shapes are chosen for 256 CUs / wave64).
+ *   sms         -1 = automatic; otherwise an upper bound on the number of workgroups that cooperate
+ *               on one column tile's reduction (debug/testing knob, like the reference's).
+ *   max_par     as in the reference: bounds how many 64-row blocks of A one launch covers.
+ *   quant_cols  -1 (or 0) = all INT4; n = all FP6; otherwise the last quant_cols columns are FP6.
+ *               Must be a multiple of 128, as must n - quant_cols.
+ *   group_size  -1 = one INT4 scale per column (what the reference kernel supports);
+ *               128 = one INT4 scale per 128 rows of k per column.  FP6 scales are always per column.
+ * Zero-sized problems return FP6M_OK without launching (fp6_marlin_cuda_kernel.cu:906-907).
+ */
+int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+             void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
+             int quant_cols, int group_size);
+
+/* Minimum workspace length in 4-byte elements: n / 128 * max_par (fp6_marlin/fp6_marlin_cuda.cpp:62-63). */
+size_t fp6m_workspace_elems(int prob_n, int max_par);
+
+/*
+ * Device-memory scratch the GEMM keeps per GPU for cross-workgroup partial sums.  It is allocated
+ * on the first fp6m_mul on a device, or eagerly here (call once per device outside any region that
+ * must not allocate).  No counterpart in the reference (which reduces through C in fp16).
+ */
+int fp6m_init(int dev);
+
+/*
+ * FP16 -> FP6 (e3m2) row quantiser.  Replaces
+ *   void weight_prepacking_fp16_to_fp6(uint16_t* weight_16bit, uint8_t* weight_6bit_packed, size_t K, size_t N)
+ *   (fp6_marlin/weight_quant.cpp:106-124, declared fp6_marlin/pybind.cpp:7).
+ * `w`: rows x cols binary16 bit patterns, `out`: rows x cols*6/8 bytes, four codes per three bytes, MSB
+ * first.  Truncating cast; values with 0 < |x| < 0.0625, |x| > 28 or NaN -> FP6M_ERR_RANGE (the reference
+ * throws); cols*6 % 8 != 0 -> FP6M_ERR_SHAPE.
+ */
+int fp6m_fp6_quantize(const uint16_t* w, uint8_t* out, size_t rows, size_t cols);
+
+/*
+ * FP6 2+4-bit prepacker, bit-exact with
+ *   void weight_matrix_prepacking(int* packed_weights, int* FP6Weights, size_t K, size_t N)
+ *   (fp6_marlin/weight_prepacking.cpp:123-177, declared fp6_marlin/pybind.cpp:6).
+ * `fp6`: oc rows (output channels) x ic*6/8 bytes of row-packed codes; `packed`: oc*ic*6/8 bytes, the
+ * 2-bit plane followed by the 4-bit plane.  oc % 64 or ic % 64 -> FP6M_ERR_SHAPE (the reference asserts).
+ */
+int fp6m_fp6_prepack(int32_t* packed, const int32_t* fp6, size_t oc, size_t ic);
+
+/*
+ * FP6 -> FP16 dequantiser.  Replaces
+ *   void dequantMatrix_fp6_to_fp16(half* A_16bit_h, unsigned char* A_x_bit_h, size_t M, size_t K, half* scale)
+ *   (fp6_marlin/weight_prepacking.cpp:180-217, declared fp6_marlin/pybind.cpp:5).
+ * out[r][c] = fp16(value(code[r][c]) * scale[r]), one rounding.
+ */
+int fp6m_fp6_dequant(uint16_t* out, const uint8_t* fp6, size_t rows, size_t cols, const uint16_t* scale);
+
+/*
+ * Symmetric INT4 quantiser of the reference's harness (test.py:85-101, gen_int4_weight up to the
+ * fake-quantised reference).  `w`: k x n binary16, row-major.  group_size -1 (per column) or a divisor
+ * of k.  Outputs: codes k x n bytes in 0..15, scales (k/group) x n binary16 in natural column order,
+ * w_ref k x n binary16 = (code - 8) * scale.  Any output pointer may be NULL.
+ */
+int fp6m_int4_quantize(const uint16_t* w, size_t k, size_t n, int group_size, uint8_t* codes,
+                       uint16_t* scales, uint16_t* w_ref);
+
+/*
+ * Marlin INT4 packer, bit-exact with the packing half of gen_int4_weight (test.py:106-113 with the
+ * permutation of test.py:60-79).  codes k x n bytes in 0..15 -> packed int32 [k/16, n*2].
+ * k % 16 or n % 64 -> FP6M_ERR_SHAPE.
+ */
+int fp6m_int4_pack(const uint8_t* codes, int32_t* packed, size_t k, size_t n);
+
+/* Scale permutation of test.py:80-83 applied per group of 32 (test.py:49-53, 102-105). n % 32 -> ERR_SHAPE. */
+int fp6m_permute_scales(const uint16_t* in, uint16_t* out, size_t n);
+
+/*
+ * Host inverse of both packers: the dequantised fp16 weight W_ref [k, n] that `B`/`s` encode -- the
+ * left operand of the reference's dequantise-then-matmul check (test.py:37-38, 98, 165-167).
+ */
+int fp6m_unpack_to_fp16(const int32_t* B, const uint16_t* s, uint16_t* w_ref, size_t k, size_t n,
+                        int quant_cols, int group_size);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP6M_H_ */
