@@ -64,26 +64,28 @@ def _cpu(t, dtype, name):
 
 # ------------------------------------------------------------------------------------------ host routines
 
-def fp6_quantize(w):
+def fp6_quantize(w, strict=True):
     """float16 [OC, IC] -> int32 [IC, OC*3/16].  The flat row-major buffer is quantised as IC rows of OC
     values and *labelled* transposed, exactly as fp6_marlin/pybind.cpp:42-59 does."""
     w = _cpu(w, torch.float16, "Input tensor")
-    if w.dim() != 2 or w.shape[0] % 256 or w.shape[1] % 256:
-        raise ValueError("quantize expects a 2-D tensor with both dimensions multiples of 256")
+    mult = 256 if strict else 64        # the reference's wrapper asserts 256 (pybind.cpp:50), its C routine needs less
+    if w.dim() != 2 or w.shape[0] % mult or w.shape[1] % mult:
+        raise ValueError(f"quantize expects a 2-D tensor with both dimensions multiples of {mult}")
     oc, ic = w.shape
     out = torch.empty((ic, oc // 16 * 3), dtype=torch.int32)
     _raise_cpu(lib.fp6m_fp6_quantize(w.data_ptr(), out.data_ptr(), ic, oc))
     return out
 
 
-def fp6_prepack(q):
+def fp6_prepack(q, strict=True):
     """int32 [OC, IC*3/16] -> int32 [IC*3/32, OC*2] (2-bit plane then 4-bit plane), fp6_marlin/pybind.cpp:18-31."""
     q = _cpu(q, torch.int32, "fp6 tensor")
     if q.dim() != 2 or q.shape[1] % 3:
         raise ValueError("prepacking expects int32 [OC, IC*3/16]")
     oc, ic = q.shape[0], q.shape[1] * 16 // 3
-    if oc % 256 or ic % 256:
-        raise ValueError("prepacking expects OC and IC to be multiples of 256")
+    mult = 256 if strict else 64        # pybind.cpp:24 asserts 256, weight_prepacking.cpp:124-125 asserts 64
+    if oc % mult or ic % mult:
+        raise ValueError(f"prepacking expects OC and IC to be multiples of {mult}")
     out = torch.empty((ic // 32 * 3, oc * 2), dtype=torch.int32)
     _raise_cpu(lib.fp6m_fp6_prepack(out.data_ptr(), q.data_ptr(), oc, ic))
     return out

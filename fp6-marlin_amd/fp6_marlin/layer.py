@@ -27,9 +27,9 @@ def _fp6_region(w):
     w = w / s
     w = torch.where(torch.abs(w) < FP6_MIN, torch.zeros_like(w), w)
     w = torch.clamp(w, -FP6_MAX, FP6_MAX)
-    q = cabi.fp6_quantize(w)                       # int32 [nq, k*3/16]: rows of the *flat* buffer
+    q = cabi.fp6_quantize(w, strict=False)         # int32 [nq, k*3/16]: rows of the *flat* buffer
     w_ref = cabi.fp6_dequant(q, s).transpose(0, 1).contiguous()
-    return cabi.fp6_prepack(q), cabi.permute_scales(s), w_ref
+    return cabi.fp6_prepack(q, strict=False), cabi.permute_scales(s), w_ref
 
 
 def pack_mixed_weight(w, quant_cols=-1, group_size=-1, harness_layout=True):
@@ -69,9 +69,9 @@ def pack_mixed_weight(w, quant_cols=-1, group_size=-1, harness_layout=True):
             s6 = torch.where(s6 == 0, torch.ones_like(s6), s6)
             t = (w6 / s6).transpose(0, 1).contiguous()            # [nq, k]
             t = torch.where(torch.abs(t) < FP6_MIN, torch.zeros_like(t), t).clamp(-FP6_MAX, FP6_MAX)
-            q = cabi.fp6_quantize(t.reshape(k, qc))               # flat view read as [nq, k]
+            q = cabi.fp6_quantize(t.reshape(k, qc), strict=False)  # flat view read as [nq, k]
             ref6 = cabi.fp6_dequant(q, s6).transpose(0, 1).contiguous()
-            b6, s6 = cabi.fp6_prepack(q), cabi.permute_scales(s6)
+            b6, s6 = cabi.fp6_prepack(q, strict=False), cabi.permute_scales(s6)
         parts_b.append(b6.reshape(-1))
         parts_s.append(s6.reshape(-1))
         parts_ref.append(ref6)

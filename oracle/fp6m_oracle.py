@@ -104,7 +104,7 @@ def fp6_quantize_flat(w_bits, rows, cols):
     return dst
 
 
-def fp6_quantize(w):
+def fp6_quantize(w, strict=True):
     """pybind.cpp:42-59.  `w`: float16 [OC, IC]; returns int32 [IC, OC*3/16].
 
     The reference labels its result "transposed" but hands the *untransposed*
@@ -114,7 +114,7 @@ def fp6_quantize(w):
     w = np.ascontiguousarray(w)
     assert w.dtype == np.float16 and w.ndim == 2
     oc, ic = w.shape
-    if oc % 256 or ic % 256:  # pybind.cpp:50
+    if strict and (oc % 256 or ic % 256):  # pybind.cpp:50 (strict=False: only what the C routines need)
         raise OracleError("shape not supported")
     q = fp6_quantize_flat(w.view(np.uint16), ic, oc)
     return q.view(np.int32).reshape(ic, oc * 3 // 16)
@@ -227,7 +227,7 @@ def gen_int4_weight(w, group_size=-1):
     return ref, int4_pack(codes), np.ascontiguousarray(s)
 
 
-def gen_fp6_weight(w):
+def gen_fp6_weight(w, strict=True):
     """test.py:13-58.  w (k,n) f16 -> (w_ref (k,n) f16, B int32 [k*3/32, n*2], s (n,) f16 permuted)."""
     w = torch.as_tensor(np.ascontiguousarray(w)).clone()
     k, n = w.shape
@@ -237,28 +237,30 @@ def gen_fp6_weight(w):
     w = w / s                                                # :24
     w = torch.where(torch.abs(w) < 0.0625, torch.zeros_like(w), w)  # :26
     w = torch.clamp(w, -28.0, 28.0)                          # :27
-    q = fp6_quantize(w.numpy())                              # :32  int32 [n, k*3/16]
+    q = fp6_quantize(w.numpy(), strict)                      # :32  int32 [n, k*3/16]
     w_ref = fp6_dequant(q, s.numpy()).T                      # :37-38
-    packed = fp6_prepack(q)                                  # :43
+    packed = fp6_prepack(q, strict)                          # :43
     return np.ascontiguousarray(w_ref), packed, permute_scales(s.numpy())
 
 
-def gen_mixed_weight(w, quant_cols=-1, group_size=-1):
+def gen_mixed_weight(w, quant_cols=-1, group_size=-1, strict=True):
     """test.py:123-152.  w (k,n) f16.  Returns (w_ref (k,n) f16, B int32 1-D, s f16 1-D).
 
     B = INT4 words of columns [0, n-qc)  ||  FP6 2-bit words  ||  FP6 4-bit words
-    s = INT4 scales || FP6 scales        (test.py:139, 143-147)."""
+    s = INT4 scales || FP6 scales        (test.py:139, 143-147).
+    strict=False drops the multiple-of-256 asserts of the Python wrappers (pybind.cpp:24,50) and keeps
+    the multiple-of-64 ones of the C routines, for FP6 regions of 128 columns."""
     k, n = w.shape
     if quant_cols == -1:
         ref, b, s = gen_int4_weight(w, group_size)
         return ref, b.reshape(-1), s.reshape(-1)
     if quant_cols == n:
-        ref, b, s = gen_fp6_weight(w)
+        ref, b, s = gen_fp6_weight(w, strict)
         return ref, b.reshape(-1), s.reshape(-1)
     assert quant_cols % 64 == 0                               # :129
     w1, w2 = w[:, : n - quant_cols], w[:, n - quant_cols:]    # :130
     r1, b1, s1 = gen_int4_weight(np.ascontiguousarray(w1), group_size)
-    r2, b2, s2 = gen_fp6_weight(np.ascontiguousarray(w2))
+    r2, b2, s2 = gen_fp6_weight(np.ascontiguousarray(w2), strict)
     return (np.ascontiguousarray(np.concatenate([r1, r2], axis=1)),
             np.concatenate([b1.reshape(-1), b2.reshape(-1)]),
             np.concatenate([s1.reshape(-1), s2.reshape(-1)]))
