@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the mixed INT4/FP6 weight-only GEMM on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]          one JSON line (the driver's contract)
+    python bench.py --sweep gpurun_out/sweep.json                per-shape table for all BASELINE configs
+
+Workload of the JSON line: decode (M=1) through Llama-2-7B layer shapes (K x N) 4096x12288, 4096x4096,
+4096x22016, 11008x4096; INT4 with group-128 scales plus 256 FP6 columns.  A *step* is one layer: those four
+GEMMs.  Eight distinct layers (8 x 105.7 MB of packed weights) are cycled so that neither the L2 nor the
+256 MB Infinity Cache can serve the weight stream.  Packed words are random bits, scales random positive
+fp16, activations N(0,1) fp16 (the reference's own bench does the same, bench.py:26-34).
+
+value        packed-weight GB/s over the timed steps: algorithmic weight bytes / wall time, where
+             weight bytes = K(N-qc)/2 + K*qc*3/4 + scale bytes.
+roofline     the GEMM kernel against the 8 TB/s HBM peak: algorithmic bytes per launch / mean time per
+             launch, measured with HIP events on the launch stream over the same timed region.
+cpu_baseline the oracle's CPU path (quantise + prepack + dequantise-then-matmul) on one bounded sample
+             shape, single-threaded like the reference, on this box's host cores.
+Also reported: a fp16 torch.matmul (hipBLASLt/rocBLAS) over the same shapes and rotation, and the speed-up.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "fp6-marlin_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+LLAMA7B = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
+LLAMA70B = [(8192, 10240), (8192, 8192), (8192, 57344), (28672, 8192)]
+
+
+def weight_bytes(k, n, qc, gs):
+    n4 = n - qc
+    scale = 2 * n if gs == -1 else 2 * (k // gs) * n4 + 2 * qc
+    return k * n4 // 2 + k * qc * 3 // 4 + scale
+
+
+class Problem:
+    """Device operands of one (m, k, n) GEMM with random packed words."""
+
+    def __init__(self, torch, m, k, n, qc, gs, gen, fp16_ref=False):
+        dev = torch.device("cuda:0")
+        n4 = n - qc
+        words = k * n4 // 8 + k * qc * 3 // 16
+        self.m, self.k, self.n, self.qc, self.gs = m, k, n, qc, gs
+        self.B = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
+        ns = (n4 if gs == -1 else (k // gs) * n4) + qc
+        self.s = (torch.rand(ns, generator=gen) * 0.01 + 0.001).half().to(dev)
+        self.A = torch.randn((m, k), generator=gen).half().to(dev)
+        self.C = torch.zeros((m, n), dtype=torch.half, device=dev)
+        self.ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev)
+        self.W16 = (torch.randn((k, n), generator=gen) * 0.02).half().to(dev) if fp16_ref else None
+        self.bytes = weight_bytes(k, n, qc, gs)
+        self.flops = 2 * m * k * n
+
+    def run(self, mul):
+        mul(self.A, self.B, self.C, self.s, self.ws, self.qc if self.qc else -1, -1, -1, -1, 16, self.gs)
+
+    def run_fp16(self, torch):
+        torch.matmul(self.A, self.W16, out=self.C)
+
+
+def time_region(torch, fn, iters):
+    """Wall clock (synchronised on both sides) and HIP-event time of `iters` calls of fn(i)."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(iters):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, start.elapsed_time(stop) * 1e-3
+
+
+def cpu_baseline(torch):
+    """Oracle path on the host: quantise + prepack, then dequantise-then-matmul, single thread."""
+    import numpy as np
+    from oracle import fp6m_oracle as oracle
+    m, k, n, qc, gs = 1, 4096, 4096, 256, 128
+    threads = torch.get_num_threads()
+    torch.set_num_threads(1)
+    try:
+        rng = np.random.default_rng(0)
+        w = rng.normal(0, 0.02, (k, n)).astype(np.float16)
+        a = rng.normal(0, 1, (m, k)).astype(np.float16)
+        t0 = time.perf_counter()
+        w_ref, b, s = oracle.gen_mixed_weight(w, qc, gs)        # quantise, dequantise (w_ref), pack, prepack
+        t1 = time.perf_counter()
+        c = torch.matmul(torch.from_numpy(a).float(), torch.from_numpy(w_ref).float())
+        t2 = time.perf_counter()
+        del c, b, s
+    finally:
+        torch.set_num_threads(threads)
+    nbytes = weight_bytes(k, n, qc, gs)
+    return {"value": nbytes / (t2 - t0) / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"one GEMM m={m} k={k} n={n} (Llama-2-7B o_proj), INT4 g128 + 256 FP6 cols: "
+                      f"quantise+prepack+dequantise {t1 - t0:.2f} s, fp32 matmul {t2 - t1:.4f} s, "
+                      f"{nbytes} weight bytes; host has {os.cpu_count()} logical cores"}
+
+
+def headline(args):
+    import torch
+    import fp6_marlin
+    gen = torch.Generator().manual_seed(0)
+    qc, gs, m, layers = 256, 128, 1, 8
+    fp6_marlin.init(0)
+    model = [[Problem(torch, m, k, n, qc, gs, gen, fp16_ref=True) for (k, n) in LLAMA7B] for _ in range(layers)]
+    step_bytes = sum(p.bytes for p in model[0])
+    launches_per_step = len(LLAMA7B)
+
+    def step(i):
+        for p in model[i % layers]:
+            p.run(fp6_marlin.mul)
+
+    def step_fp16(i):
+        for p in model[i % layers]:
+            p.run_fp16(torch)
+
+    for i in range(args.warmup):
+        step(i)
+    wall, ev = time_region(torch, step, args.steps)
+    for i in range(max(2, args.warmup // 4)):
+        step_fp16(i)
+    wall16, _ = time_region(torch, step_fp16, args.steps)
+
+    gbs = step_bytes * args.steps / wall / 1e9
+    per_launch = ev / (args.steps * launches_per_step)
+    achieved = step_bytes / launches_per_step / per_launch / 1e9
+    out = {
+        "metric": "weight-stream GB/s (M=1-16), TFLOP/s (M=128), speedup vs fp16 hipBLASLt",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "decode M=1, Llama-2-7B layer shapes 4096x12288 4096x4096 4096x22016 11008x4096, "
+                               "INT4 g128 + 256 FP6 columns, one step = one layer (4 GEMMs), 8 layers cycled",
+                   "m": m, "quant_cols": qc, "group_size": gs, "weight_bytes_per_step": step_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "fp6m::gemm_kernel<1, true>", "us_per_launch": round(per_launch * 1e6, 3),
+                     "bytes_per_launch": step_bytes // launches_per_step},
+        "cpu_baseline": cpu_baseline(torch),
+        "fp16_hipblaslt": {"ms_per_step": round(wall16 / args.steps * 1e3, 5),
+                           "speedup": round(wall16 / wall, 3)},
+    }
+    print(json.dumps(out), flush=True)
+
+
+def sweep(args):
+    """Per-shape numbers for every BASELINE configuration; written as JSON rows."""
+    import torch
+    import fp6_marlin
+    gen = torch.Generator().manual_seed(0)
+    fp6_marlin.init(0)
+    rows = []
+    cases = []
+    cases += [("cfg0", 16, 4096, 4096, 256, 128)]
+    cases += [("cfg1-7B", 1, k, n, 256, 128) for k, n in LLAMA7B]
+    cases += [("cfg1-7B-m16", 16, k, n, 256, 128) for k, n in LLAMA7B]
+    cases += [("cfg2-70B", m, k, n, 256, 128) for m in (1, 16) for k, n in LLAMA70B]
+    cases += [("cfg3-msweep", m, 8192, 8192, 256, 128) for m in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024)]
+    cases += [("cfg4-13B", 33, 5120, 13824, 512, -1), ("cfg4-13B", 33, 13824, 5120, 512, -1)]
+    cases += [("all-int4-g-1", 16, 8192, 8192, 0, -1), ("all-int4-g128", 16, 8192, 8192, 0, 128)]
+    for tag, m, k, n, qc, gs in cases:
+        nbytes = weight_bytes(k, n, qc, gs)
+        copies = max(2, min(24, int(640e6 // nbytes) + 1))           # rotate over > 512 MB of weights
+        probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
+        w16 = [(torch.randn((k, n), generator=gen) * 0.02).half().cuda() for _ in range(max(2, min(copies, int(640e6 // (2 * k * n)) + 1)))]
+        iters = 100
+
+        def f(i):
+            probs[i % copies].run(fp6_marlin.mul)
+
+        def f16(i):
+            torch.matmul(probs[0].A, w16[i % len(w16)], out=probs[0].C)
+
+        for i in range(10):
+            f(i)
+            f16(i)
+        _, ev = time_region(torch, f, iters)
+        _, ev16 = time_region(torch, f16, iters)
+        t, t16 = ev / iters, ev16 / iters
+        row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "us": round(t * 1e6, 2),
+               "weight_GBs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
+               "TFLOPs": round(2 * m * k * n / t / 1e12, 2), "mfma_frac": round(2 * m * k * n / t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+               "fp16_us": round(t16 * 1e6, 2), "speedup_vs_fp16": round(t16 / t, 2)}
+        rows.append(row)
+        print(json.dumps(row), flush=True)
+        del probs, w16
+        torch.cuda.empty_cache()
+    os.makedirs(os.path.dirname(os.path.abspath(args.sweep)), exist_ok=True)
+    with open(args.sweep, "w") as fh:
+        json.dump(rows, fh, indent=1)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the op shards along N without any exchange); "
+                 "run with --gpus 1")
+    if args.sweep:
+        sweep(args)
+    else:
+        headline(args)
+
+
+if __name__ == "__main__":
+    main()

@@ -118,174 +118,63 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int total)
     return x * q + (x < r ? x : r) + (b >> 3);
 }
 
-// ------------------------------------------------------------------------------------------------ kernel
+// ------------------------------------------------------------------------------------------------ tile bookkeeping
 
-template <int MB>
-struct Stage {
-    u4 w4[2];            // 4-bit plane / INT4 words of k-blocks 2s, 2s+1 (this lane's linear 16 bytes)
-    u2 w2[2];            // FP6 2-bit plane (this lane's linear 8 bytes)
-    uint32_t a[MB][4];   // activations, already in MFMA operand order
+struct TileInfo {
+    int tile, part, mtile;   // tile in the [FP6 | INT4] tile list, k partner index, m-tile
+    bool fp6;
+    int tcol;                // tile index inside its region
+    int region_n;            // columns of the region
+    int col0;                // first column of the tile in C
 };
 
-template <int MB, bool G128>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
+__device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes];
-    __shared__ int s_is_last;
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    TileInfo t;
     const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    const int tile = logical / p.ksplit;
-    const int part = logical - tile * p.ksplit;
-    const int mtile = blockIdx.y;
-    const bool fp6 = tile < p.tiles6;
-    const int tcol = fp6 ? tile : tile - p.tiles6;          // tile index inside its region
-    const int region_n = fp6 ? p.qc : p.n4;
-    const int col0 = (fp6 ? p.n4 : 0) + tcol * kTileN;      // first column of the tile in C
+    t.tile = logical / p.ksplit;
+    t.part = logical - t.tile * p.ksplit;
+    t.mtile = blockIdx.y;
+    t.fp6 = t.tile < p.tiles6;
+    t.tcol = t.fp6 ? t.tile : t.tile - p.tiles6;
+    t.region_n = t.fp6 ? p.qc : p.n4;
+    t.col0 = (t.fp6 ? p.n4 : 0) + t.tcol * kTileN;
+    return t;
+}
 
-    // k range of this wave, in steps of 32 (two k-blocks); group-aligned when scales are per group.
-    const int unit_steps = G128 ? 4 : 1;
+// k range of one wave in steps of 32 (two k-blocks).  Units of two steps (four with group scales) keep
+// every wave's step count even and group-aligned.
+template <bool G128>
+__device__ __forceinline__ void wave_k_range(const GemmArgs& p, int part, int wave, int& begin, int& end)
+{
+    constexpr int unit_steps = G128 ? 4 : 2;
     const int units = p.k / (32 * unit_steps);
     const int nwaves = p.ksplit * kWaves;
     const int wv = part * kWaves + wave;
-    const int step_begin = (int)((long long)units * wv / nwaves) * unit_steps;
-    const int step_end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
+    begin = (int)((long long)units * wv / nwaves) * unit_steps;
+    end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
+}
 
-    // MFMA-side identity of this lane: k-pair index i, column slot c = 8*sigma + l.
-    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
-    const int owner = 32 * sigma + 4 * l + i;               // linear 16-byte granule of (group sigma, owner 4l+i)
-    unsigned char* slab = smem + wave * kSlabBytes;
-    const int wr4 = (lane ^ ((lane >> 4) & 3)) * 16;        // swizzled so both sides are bank-conflict free
-    const int rd4 = (owner ^ ((owner >> 4) & 3)) * 16;
-    const int wr2 = (lane ^ ((lane >> 5) << 1)) * 8;
-    const int rd2 = (owner ^ ((owner >> 5) << 1)) * 8;
-
-    // Global pointers.  A k-block of a region is one row of region_n*8 bytes (4-bit) / region_n*4 (2-bit).
-    const size_t row4 = (size_t)region_n * 8, row2 = (size_t)region_n * 4;
-    const unsigned char* g4 = reinterpret_cast<const unsigned char*>(fp6 ? p.b_fp6_4 : p.b_int4) +
-                              (size_t)tcol * 1024 + lane * 16;
-    const unsigned char* g2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)tcol * 512 + lane * 8;
-
-    const uint16_t* a_row[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        int row = mtile * 16 * MB + 16 * mb + c;
-        row = row < p.m ? row : p.m - 1;
-        a_row[mb] = p.A + (size_t)row * p.k + 2 * i;
-    }
-
-    auto load = [&](Stage<MB>& st, int s) {
-        const unsigned char* src4 = g4 + (size_t)(2 * s) * row4;
-        st.w4[0] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4));
-        st.w4[1] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4 + row4));
-        if (fp6) {
-            const unsigned char* src2 = g2 + (size_t)(2 * s) * row2;
-            st.w2[0] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2));
-            st.w2[1] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2 + row2));
-        }
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-                st.a[mb][d] = *reinterpret_cast<const uint32_t*>(a_row[mb] + 32 * s + 8 * d);
-    };
-
-    f4 acc[MB][8];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
-
-    h2 gscale[8];  // G128, INT4 tiles: scale of column (j, half) duplicated into both halves
-    auto load_group_scales = [&](int s) {
-        const uint16_t* srow = p.s_int4 + (size_t)(s >> 2) * p.n4 + tcol * kTileN + 64 * sigma + l;
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            const uint16_t v = srow[16 * (t >> 1) + 8 * (t & 1)];
-            gscale[t] = as_h2((uint32_t)v | ((uint32_t)v << 16));
-        }
-    };
-
-    auto consume = [&](Stage<MB>& st, int s) {
-        wave_lds_fence();
-        *reinterpret_cast<u4*>(slab + wr4) = st.w4[0];
-        *reinterpret_cast<u4*>(slab + 1024 + wr4) = st.w4[1];
-        if (fp6) {
-            *reinterpret_cast<u2*>(slab + 2048 + wr2) = st.w2[0];
-            *reinterpret_cast<u2*>(slab + 2560 + wr2) = st.w2[1];
-        }
-        wave_lds_fence();
-        const u4 q0 = *reinterpret_cast<const u4*>(slab + rd4);
-        const u4 q1 = *reinterpret_cast<const u4*>(slab + 1024 + rd4);
-        u2 t0 = {0, 0}, t1 = {0, 0};
-        if (fp6) {
-            t0 = *reinterpret_cast<const u2*>(slab + 2048 + rd2);
-            t1 = *reinterpret_cast<const u2*>(slab + 2560 + rd2);
-        }
-        if (G128 && !fp6 && (s & 3) == 0) load_group_scales(s);
-
-        h8 av[MB];
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-            u4 raw = {st.a[mb][0], st.a[mb][1], st.a[mb][2], st.a[mb][3]};
-            av[mb] = __builtin_bit_cast(h8, raw);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            h2 r0[4], r1[4];
-            if (fp6) {
-                dequant_fp6(t0[j >> 1] << (4 * (j & 1)), q0[j], r0);
-                dequant_fp6(t1[j >> 1] << (4 * (j & 1)), q1[j], r1);
-            } else {
-                dequant_int4(q0[j], r0);
-                dequant_int4(q1[j], r1);
-                if (G128) {
-#pragma unroll
-                    for (int x = 0; x < 4; x++) {
-                        r0[x] = r0[x] * gscale[2 * j + (x >> 1)];
-                        r1[x] = r1[x] * gscale[2 * j + (x >> 1)];
-                    }
-                }
-            }
-            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
-            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                acc[mb][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av[mb], acc[mb][2 * j + 0], 0, 0, 0);
-                acc[mb][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av[mb], acc[mb][2 * j + 1], 0, 0, 0);
-            }
-        }
-    };
-
-    // Two stages of loads stay in flight in registers while the current one is consumed.
-    Stage<MB> st0, st1;
-    int s = step_begin;
-    if (s < step_end) load(st0, s);
-    if (s + 1 < step_end) load(st1, s + 1);
-    for (; s < step_end; s += 2) {
-        consume(st0, s);
-        if (s + 2 < step_end) load(st0, s + 2);
-        if (s + 1 < step_end) {
-            consume(st1, s + 1);
-            if (s + 3 < step_end) load(st1, s + 3);
-        }
-    }
-
-    // ---- epilogue: sum the four waves through LDS, then either finish or hand over a partial tile.
-    // MFMA result layout: lane (m = lane & 15, q = lane >> 4) holds column slots 4q .. 4q+3.
-    const int q = lane >> 4;
+// Epilogue shared by both kernels: sum the four waves of the workgroup through LDS, then either write
+// C (scaled, fp16) or publish an fp32 partial tile and let the last-arriving partner finish.
+// MFMA result layout: lane (m = lane & 15, q = lane >> 4) holds column slots 4q .. 4q+3 of each of the
+// eight 16-column accumulators (t = 2*j + half): column = 64*(q >> 1) + 16*j + 8*half + 4*(q & 1) + r.
+template <int MB>
+__device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& ti, f4 (&acc)[MB][8],
+                                            bool per_column_scale, unsigned char* smem, int* s_is_last)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, q = lane >> 4;
     float* red = reinterpret_cast<float*>(smem);
     const int out_m = threadIdx.x >> 4;          // row inside the 16-row block
     const int out_n = (threadIdx.x & 15) * 8;    // first of eight consecutive columns
     const size_t tile_floats = (size_t)MB * 16 * kTileN;
-    float* my_partial = p.scratch + ((size_t)(mtile * p.tiles + tile) * p.ksplit + part) * tile_floats;
+    float* my_partial = p.scratch + ((size_t)(ti.mtile * p.tiles + ti.tile) * p.ksplit + ti.part) * tile_floats;
 
-    const bool per_column_scale = fp6 || !G128;
     float sc[8];
     if (per_column_scale) {
-        const uint16_t* sp = (fp6 ? p.s_fp6 : p.s_int4);
-        const int nr = tcol * kTileN + out_n;    // column inside the region, multiple of 8
+        const uint16_t* sp = (ti.fp6 ? p.s_fp6 : p.s_int4);
+        const int nr = ti.tcol * kTileN + out_n;    // column inside the region, multiple of 8
         const int base = (nr & ~31) + 4 * ((nr >> 4) & 1) + 2 * ((nr >> 3) & 1);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -301,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
         h8 o;
 #pragma unroll
         for (int e = 0; e < 8; e++) o[e] = (_Float16)(v[e] * sc[e]);
-        *reinterpret_cast<h8*>(p.C + (size_t)row * p.n + col0 + out_n) = o;
+        *reinterpret_cast<h8*>(p.C + (size_t)row * p.n + ti.col0 + out_n) = o;
     };
 
 #pragma unroll
@@ -321,7 +210,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
 #pragma unroll
             for (int e = 0; e < 4; e++) { v[e] += lo[e]; v[4 + e] += hi[e]; }
         }
-        const int row = mtile * 16 * MB + 16 * mb + out_m;
+        const int row = ti.mtile * 16 * MB + 16 * mb + out_m;
         if (row < p.m) {
             if (p.ksplit == 1) {
                 store_row(row, v);
@@ -337,18 +226,18 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
     // Publish the partial, then count arrivals; the last workgroup of the tile finishes it.
     __threadfence();
     __syncthreads();
-    int* counter = p.counters + mtile * p.tiles + tile;
+    int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
     if (threadIdx.x == 0) {
         const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_is_last = (seen == p.ksplit - 1);
+        *s_is_last = (seen == p.ksplit - 1);
     }
     __syncthreads();
-    if (!s_is_last) return;
+    if (!*s_is_last) return;
     __threadfence();
-    const float* first = p.scratch + (size_t)(mtile * p.tiles + tile) * p.ksplit * tile_floats;
+    const float* first = p.scratch + (size_t)(ti.mtile * p.tiles + ti.tile) * p.ksplit * tile_floats;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
-        const int row = mtile * 16 * MB + 16 * mb + out_m;
+        const int row = ti.mtile * 16 * MB + 16 * mb + out_m;
         if (row >= p.m) continue;
         float v[8];
 #pragma unroll
@@ -363,6 +252,360 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
         store_row(row, v);
     }
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ------------------------------------------------------------------------------------------------ m <= 16: LDS-ring kernel
+//
+// Every wave keeps a private ring of DEPTH slots in LDS.  A slot is one k step (32 rows of k) of its
+// tile: the packed words (2 x 1 KiB 4-bit/INT4, + 2 x 512 B FP6 2-bit) and the 16 x 32 fp16 activation
+// block (1 KiB).  Slots are filled by direct-to-LDS global loads (no VGPR staging): lane L's data lands
+// at slot + 16 L, so the *global* granule each lane fetches is permuted (inside aligned 64-byte quads,
+// which keeps the loads coalesced) to obtain a layout that the permuted reads hit without bank
+// conflicts.  The loads of step s + DEPTH - 1 are issued before step s is consumed; `s_waitcnt vmcnt`
+// with a constant count is the only synchronisation in the loop.  LDS reads are inline asm so that
+// the compiler does not serialise them behind every outstanding direct-to-LDS load.
+
+#define FP6M_AS1 __attribute__((address_space(1)))
+#define FP6M_AS3 __attribute__((address_space(3)))
+
+__device__ __forceinline__ void dma16(const void* gsrc, unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void* gsrc, unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 4, 0, 0);
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* ptr) { return (uint32_t)(uintptr_t)(const FP6M_AS3 void*)ptr; }
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt = [3:0] and [15:14]).
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+template <bool FP6, bool G128, int DEPTH>
+__device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
+                                            int step_begin, int step_end, f4 (&acc)[1][8])
+{
+    constexpr bool kGroup = G128 && !FP6;                 // group scales apply to INT4 tiles only
+    constexpr int kSlot = FP6 ? 4096 : 3072;
+    constexpr int kAOff = kSlot - 1024;
+    constexpr int kOps = FP6 ? 4 : 3;                     // direct-to-LDS loads per step
+    const int lane = threadIdx.x & 63;
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+
+    // ---- fetch side (lane = position in the slot)
+    const int g4_granule = lane ^ ((lane >> 4) & 3);
+    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const unsigned char* g4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                              (size_t)ti.tcol * 1024 + g4_granule * 16;
+    const int lg = lane & 31;
+    const unsigned char* g2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
+                              (size_t)(lane >> 5) * row2 + (lg ^ (lg >> 4)) * 16;
+    const int a_m = lane >> 2;
+    const bool a_active = ti.mtile * 16 + a_m < p.m;
+    const uint16_t* a_src = p.A + (size_t)(a_active ? ti.mtile * 16 + a_m : 0) * p.k + 8 * ((lane & 3) ^ (a_m >> 2));
+    const uint16_t* gs_src = p.s_int4 + (size_t)ti.tcol * kTileN + 2 * lane;
+    unsigned char* gs_ring = ring + DEPTH * kSlot;        // four 256-byte slabs of group scales
+
+    auto issue = [&](int sp, int slot) {
+        unsigned char* dst = ring + slot * kSlot;
+        const unsigned char* src4 = g4 + (size_t)(2 * sp) * row4;
+        dma16(src4, dst);
+        dma16(src4 + row4, dst + 1024);
+        if (FP6) dma16(g2 + (size_t)(2 * sp) * row2, dst + 2048);
+        if (a_active) dma16(a_src + 32 * sp, dst + kAOff);
+        if (kGroup && (sp & 3) == 0) dma4(gs_src + (size_t)(sp >> 2) * p.n4, gs_ring + ((sp >> 2) & 3) * 256);
+    };
+
+    // ---- read side (lane = MFMA identity)
+    const int owner = 32 * sigma + 4 * l + i;
+    const uint32_t ring_lds = lds_addr(ring);
+    const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
+    const int gr2 = owner >> 1;
+    const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
+    uint32_t rda[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * c + (d ^ (c >> 2))) * 16 + 4 * i;
+    const int q = i;                                      // result side: quarter of the column slots
+    const uint32_t rdgs = lds_addr(gs_ring) + (64 * (q >> 1) + 4 * (q & 1)) * 2;
+
+    f4 grp[8];
+    if (kGroup) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) grp[t] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int last = step_end - 1;
+    int slot_in = 0;
+#pragma unroll 1
+    for (int d = 0; d < DEPTH - 1; d++) {
+        const int sp = step_begin + d;
+        issue(sp < last ? sp : last, slot_in);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    }
+    int slot_out = 0;
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s++) {
+        const int sp = s + DEPTH - 1;
+        issue(sp < last ? sp : last, slot_in);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 1)));
+
+        const uint32_t so = slot_out * kSlot;
+        slot_out = slot_out + 1 == DEPTH ? 0 : slot_out + 1;
+        u4 q0, q1, araw;
+        u2 t0 = {0, 0}, t1 = {0, 0};
+        if (FP6) {
+            asm volatile(
+                "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
+                "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
+                : "=&v"(q0), "=&v"(q1), "=&v"(t0), "=&v"(t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
+        } else {
+            asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
+                         : "=&v"(q0), "=&v"(q1) : "v"(rd4 + so) : "memory");
+        }
+        {
+            uint32_t a0, a1, a2, a3;
+            asm volatile(
+                "ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7\n\t"
+                "s_waitcnt lgkmcnt(0)"
+                : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
+                : "v"(rda[0] + so), "v"(rda[1] + so), "v"(rda[2] + so), "v"(rda[3] + so) : "memory");
+            araw = u4{a0, a1, a2, a3};
+        }
+        // the wait above also covers q0/q1/t0/t1 (LDS returns in order); tie them to it for the compiler
+        asm volatile("" : "+v"(q0), "+v"(q1));
+        if (FP6) asm volatile("" : "+v"(t0), "+v"(t1));
+        const h8 av = __builtin_bit_cast(h8, araw);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h2 r0[4], r1[4];
+            if (FP6) {
+                dequant_fp6(t0[j >> 1] << (4 * (j & 1)), q0[j], r0);
+                dequant_fp6(t1[j >> 1] << (4 * (j & 1)), q1[j], r1);
+            } else {
+                dequant_int4(q0[j], r0);
+                dequant_int4(q1[j], r1);
+            }
+            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
+            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
+            if (kGroup) {
+                grp[2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, grp[2 * j + 0], 0, 0, 0);
+                grp[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, grp[2 * j + 1], 0, 0, 0);
+            } else {
+                acc[0][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, acc[0][2 * j + 0], 0, 0, 0);
+                acc[0][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, acc[0][2 * j + 1], 0, 0, 0);
+            }
+        }
+        if (kGroup && (s & 3) == 3) {
+            // end of a 128-row group: fold it into the running sum with its scales (fp32)
+            const uint32_t ga = rdgs + ((s >> 2) & 3) * 256;
+            u2 sv[8];
+            asm volatile(
+                "ds_read_b64 %0, %8\n\tds_read_b64 %1, %8 offset:16\n\tds_read_b64 %2, %8 offset:32\n\t"
+                "ds_read_b64 %3, %8 offset:48\n\tds_read_b64 %4, %8 offset:64\n\tds_read_b64 %5, %8 offset:80\n\t"
+                "ds_read_b64 %6, %8 offset:96\n\tds_read_b64 %7, %8 offset:112\n\ts_waitcnt lgkmcnt(0)"
+                : "=&v"(sv[0]), "=&v"(sv[1]), "=&v"(sv[2]), "=&v"(sv[3]), "=&v"(sv[4]), "=&v"(sv[5]), "=&v"(sv[6]),
+                  "=&v"(sv[7])
+                : "v"(ga) : "memory");
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const h2 lo = as_h2(sv[t][0]), hi = as_h2(sv[t][1]);
+                acc[0][t][0] += (float)lo[0] * grp[t][0];
+                acc[0][t][1] += (float)lo[1] * grp[t][1];
+                acc[0][t][2] += (float)hi[0] * grp[t][2];
+                acc[0][t][3] += (float)hi[1] * grp[t][3];
+                grp[t] = f4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    }
+    // Redundant tail prefetches may still be landing in the ring, which the epilogue reuses.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+}
+
+constexpr int ring_bytes_per_wave(int depth) { return depth * 3072 + 1024; }
+constexpr int fp6_depth(int depth) { return ring_bytes_per_wave(depth) / 4096; }
+
+template <bool G128, int DEPTH>
+__global__ __launch_bounds__(kThreads) void gemm_m16_kernel(const GemmArgs p)
+{
+    constexpr int kWaveLds = ring_bytes_per_wave(DEPTH);
+    constexpr int kLds = kWaves * kWaveLds > kRedBytes ? kWaves * kWaveLds : kRedBytes;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kLds];
+    __shared__ int s_is_last;
+
+    const TileInfo ti = locate_tile(p);
+    const int wave = threadIdx.x >> 6;
+    int step_begin, step_end;
+    wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
+
+    f4 acc[1][8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[0][t] = f4{0.f, 0.f, 0.f, 0.f};
+    unsigned char* ring = smem + wave * kWaveLds;
+    if (step_begin < step_end) {
+        if (ti.fp6)
+            stream_tile<true, G128, fp6_depth(DEPTH)>(p, ti, ring, step_begin, step_end, acc);
+        else
+            stream_tile<false, G128, DEPTH>(p, ti, ring, step_begin, step_end, acc);
+    }
+    finish_tile<1>(p, ti, acc, ti.fp6 || !G128, smem, &s_is_last);
+}
+
+// ------------------------------------------------------------------------------------------------ m > 16: register-staged kernel
+//
+// Up to 64 rows of A per workgroup pass (MB 16-row blocks): each dequantised weight fragment feeds MB
+// MFMAs.  Packed words are loaded to registers two steps ahead, turned through a wave-private LDS slab
+// and read back permuted; activations come straight from global memory in MFMA operand order.
+
+template <int MB, bool FP6>
+struct Stage {
+    u4 w4[2];            // 4-bit plane / INT4 words of k-blocks 2s, 2s+1 (this lane's linear 16 bytes)
+    u2 w2[2];            // FP6 2-bit plane (this lane's linear 8 bytes)
+    uint32_t a[MB][4];   // activations, already in MFMA operand order
+};
+
+template <int MB, bool FP6, bool G128>
+__device__ __forceinline__ void stream_tile_regs(const GemmArgs& p, const TileInfo& ti, unsigned char* slab,
+                                                 int step_begin, int step_end, f4 (&acc)[MB][8])
+{
+    constexpr bool kGroup = G128 && !FP6;
+    const int lane = threadIdx.x & 63;
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+    const int owner = 32 * sigma + 4 * l + i;               // linear 16-byte granule of (group sigma, owner 4l+i)
+    const int wr4 = (lane ^ ((lane >> 4) & 3)) * 16;        // swizzled so both sides are bank-conflict free
+    const int rd4 = (owner ^ ((owner >> 4) & 3)) * 16;
+    const int wr2 = (lane ^ ((lane >> 5) << 1)) * 8;
+    const int rd2 = (owner ^ ((owner >> 5) << 1)) * 8;
+
+    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const unsigned char* g4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                              (size_t)ti.tcol * 1024 + lane * 16;
+    const unsigned char* g2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 + lane * 8;
+    const uint16_t* a_row[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        int row = ti.mtile * 16 * MB + 16 * mb + c;
+        row = row < p.m ? row : p.m - 1;
+        a_row[mb] = p.A + (size_t)row * p.k + 2 * i;
+    }
+
+    auto load = [&](Stage<MB, FP6>& st, int s) {
+        const unsigned char* src4 = g4 + (size_t)(2 * s) * row4;
+        st.w4[0] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4));
+        st.w4[1] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4 + row4));
+        if (FP6) {
+            const unsigned char* src2 = g2 + (size_t)(2 * s) * row2;
+            st.w2[0] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2));
+            st.w2[1] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2 + row2));
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                st.a[mb][d] = *reinterpret_cast<const uint32_t*>(a_row[mb] + 32 * s + 8 * d);
+    };
+
+    h2 gscale[8];  // group scale of column (j, half), duplicated into both halves
+    auto load_group_scales = [&](int s) {
+        const uint16_t* srow = p.s_int4 + (size_t)(s >> 2) * p.n4 + ti.tcol * kTileN + 64 * sigma + l;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint16_t v = srow[16 * (t >> 1) + 8 * (t & 1)];
+            gscale[t] = as_h2((uint32_t)v | ((uint32_t)v << 16));
+        }
+    };
+
+    auto consume = [&](Stage<MB, FP6>& st, int s) {
+        wave_lds_fence();
+        *reinterpret_cast<u4*>(slab + wr4) = st.w4[0];
+        *reinterpret_cast<u4*>(slab + 1024 + wr4) = st.w4[1];
+        if (FP6) {
+            *reinterpret_cast<u2*>(slab + 2048 + wr2) = st.w2[0];
+            *reinterpret_cast<u2*>(slab + 2560 + wr2) = st.w2[1];
+        }
+        wave_lds_fence();
+        const u4 q0 = *reinterpret_cast<const u4*>(slab + rd4);
+        const u4 q1 = *reinterpret_cast<const u4*>(slab + 1024 + rd4);
+        u2 t0 = {0, 0}, t1 = {0, 0};
+        if (FP6) {
+            t0 = *reinterpret_cast<const u2*>(slab + 2048 + rd2);
+            t1 = *reinterpret_cast<const u2*>(slab + 2560 + rd2);
+        }
+        if (kGroup && (s & 3) == 0) load_group_scales(s);
+
+        h8 av[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            u4 raw = {st.a[mb][0], st.a[mb][1], st.a[mb][2], st.a[mb][3]};
+            av[mb] = __builtin_bit_cast(h8, raw);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h2 r0[4], r1[4];
+            if (FP6) {
+                dequant_fp6(t0[j >> 1] << (4 * (j & 1)), q0[j], r0);
+                dequant_fp6(t1[j >> 1] << (4 * (j & 1)), q1[j], r1);
+            } else {
+                dequant_int4(q0[j], r0);
+                dequant_int4(q1[j], r1);
+                if (kGroup) {
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        r0[x] = r0[x] * gscale[2 * j + (x >> 1)];
+                        r1[x] = r1[x] * gscale[2 * j + (x >> 1)];
+                    }
+                }
+            }
+            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
+            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                acc[mb][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av[mb], acc[mb][2 * j + 0], 0, 0, 0);
+                acc[mb][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av[mb], acc[mb][2 * j + 1], 0, 0, 0);
+            }
+        }
+    };
+
+    // Two steps of loads stay in flight in registers.  The step count is even, and the prefetch index
+    // is clamped instead of guarded, so the loop body is branch-free and the compiler's wait counts
+    // stay exact.
+    const int last = step_end - 1;
+    Stage<MB, FP6> st0, st1;
+    load(st0, step_begin);
+    load(st1, step_begin + 1);
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s += 2) {
+        consume(st0, s);
+        load(st0, s + 2 < last ? s + 2 : last);
+        consume(st1, s + 1);
+        load(st1, s + 3 < last ? s + 3 : last);
+    }
+}
+
+template <int MB, bool G128>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes];
+    __shared__ int s_is_last;
+
+    const TileInfo ti = locate_tile(p);
+    const int wave = threadIdx.x >> 6;
+    int step_begin, step_end;
+    wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
+
+    f4 acc[MB][8];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
+    unsigned char* slab = smem + wave * kSlabBytes;
+    if (step_begin < step_end) {
+        if (ti.fp6)
+            stream_tile_regs<MB, true, G128>(p, ti, slab, step_begin, step_end, acc);
+        else
+            stream_tile_regs<MB, false, G128>(p, ti, slab, step_begin, step_end, acc);
+    }
+    finish_tile<MB>(p, ti, acc, ti.fp6 || !G128, smem, &s_is_last);
 }
 
 // ------------------------------------------------------------------------------------------------ host
@@ -406,13 +649,22 @@ int ensure_scratch(int dev, DeviceScratch** out)
     return FP6M_OK;
 }
 
+constexpr int kRingDepth = 4;
+
 template <int MB>
 void launch(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
-    if (g128)
-        hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
-    else
-        hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
+    if (MB == 1) {
+        if (g128)
+            hipLaunchKernelGGL((gemm_m16_kernel<true, kRingDepth>), grid, dim3(kThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gemm_m16_kernel<false, kRingDepth>), grid, dim3(kThreads), 0, stream, a);
+    } else {
+        if (g128)
+            hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
+    }
 }
 
 }  // namespace fp6m
@@ -478,7 +730,7 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     const int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     const int rows_per_tile = 16 * mb;
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
-    const int units = g128 ? prob_k / 128 : prob_k / 32;
+    const int units = g128 ? prob_k / 128 : prob_k / 64;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     for (int mt0 = 0; mt0 < mtiles_total; mt0 += max_par) {

@@ -10,9 +10,16 @@ Same surface as liuchuan22/FP6-Marlin's ``fp6_marlin`` package (fp6_marlin/__ini
 plus what the reference keeps in its test harness or lacks: ``Layer`` (pack / forward), the INT4
 quantiser and packer, the scale permutation, the mixed-weight assembler and ``group_size=128`` scales.
 Everything is computed by ``libfp6m.so`` (C ABI in include/fp6m.h: host packers in C++, GEMM in
-hand-written HIP for gfx950).  If that library is missing the import fails; there is no fallback.
+hand-written HIP for gfx950).  The four reference entry points go through ``_fp6m_torch``, a thin
+PyTorch-ROCm C++ extension over that C ABI; ``fp6_marlin.cabi`` binds the same ABI with ctypes.
+If either shared object is missing the import fails; there is no fallback.
 """
 from . import cabi
+try:
+    from . import _fp6m_torch as _ext
+except ImportError as e:  # pragma: no cover
+    raise ImportError("fp6_marlin/_fp6m_torch.so is missing or does not load: build it with "
+                      "`python fp6-marlin_amd/build.py`; there is no fallback implementation") from e
 from .cabi import init, workspace_elems
 from .layer import Layer, pack_mixed_weight, int4_quantize, int4_pack, permute_scales, unpack_to_fp16
 
@@ -23,7 +30,7 @@ __all__ = ["prepacking", "quantize", "dequantize", "mul", "Layer", "pack_mixed_w
 def prepacking(fp6_tensor):
     """Prepack the FP6 weight in 2+4 format (CPU).  int32 [OC, IC*3/16] -> int32 [IC*3/32, OC*2].
     Bit-exact with the reference (fp6_marlin/__init__.py:8-16, weight_prepacking.cpp:123-177)."""
-    return cabi.fp6_prepack(fp6_tensor)
+    return _ext.prepacking_cpu(fp6_tensor)
 
 
 def quantize(fp16_tensor):
@@ -32,13 +39,13 @@ def quantize(fp16_tensor):
 
     Like the reference (pybind.cpp:52-57) this does NOT transpose: the contiguous buffer is read as IC
     rows of OC values.  ``Layer.pack`` transposes explicitly before calling it."""
-    return cabi.fp6_quantize(fp16_tensor)
+    return _ext.quantization_cpu(fp16_tensor)
 
 
 def dequantize(fp6_tensor, fp16_scales):
     """Dequantise FP6 to FP16 (CPU).  int32 [OC, IC*3/16], float16 [OC] -> float16 [OC, IC]
     (fp6_marlin/__init__.py:28-37)."""
-    return cabi.fp6_dequant(fp6_tensor, fp16_scales)
+    return _ext.dequantization_cpu(fp6_tensor, fp16_scales)
 
 
 def mul(A, B, C, s, workspace, quant_cols=-1, thread_k=-1, thread_n=-1, sms=-1, max_par=16, group_size=-1):
@@ -52,4 +59,4 @@ def mul(A, B, C, s, workspace, quant_cols=-1, thread_k=-1, thread_n=-1, sms=-1, 
     quant_cols -1: all INT4; n: all FP6; else the last quant_cols columns are FP6
     group_size -1: per-column INT4 scales; 128: INT4 scales [k/128, n-quant_cols] in natural column order
     """
-    return cabi.mul(A, B, C, s, workspace, quant_cols, thread_k, thread_n, sms, max_par, group_size)
+    return _ext.mul(A, B, C, s, workspace, quant_cols, thread_k, thread_n, sms, max_par, group_size)
