@@ -215,25 +215,29 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
             if (p.ksplit == 1) {
                 store_row(row, v);
             } else {
+                // agent-scope stores go straight to the level all XCDs share: no cache-wide write-back later
                 float* dst = my_partial + (size_t)(16 * mb + out_m) * kTileN + out_n;
-                *reinterpret_cast<f4*>(dst) = f4{v[0], v[1], v[2], v[3]};
-                *reinterpret_cast<f4*>(dst + 4) = f4{v[4], v[5], v[6], v[7]};
+#pragma unroll
+                for (int e = 0; e < 8; e++) __hip_atomic_store(dst + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
     if (p.ksplit == 1) return;
 
-    // Publish the partial, then count arrivals; the last workgroup of the tile finishes it.
-    __threadfence();
+    // Publish the partial, then count arrivals; the last workgroup of the tile finishes it.  Partials
+    // are written and read with agent-scope accesses, so ordering needs only "my stores have completed"
+    // (workgroup-scope release = wait counters) before the counter is bumped: no L2 write-back or
+    // invalidate, which would stall every workgroup of the XCD.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
     if (threadIdx.x == 0) {
-        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         *s_is_last = (seen == p.ksplit - 1);
     }
     __syncthreads();
     if (!*s_is_last) return;
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     const float* first = p.scratch + (size_t)(ti.mtile * p.tiles + ti.tile) * p.ksplit * tile_floats;
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) {
@@ -244,10 +248,8 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
         for (int e = 0; e < 8; e++) v[e] = 0.f;
         for (int pp = 0; pp < p.ksplit; pp++) {
             const float* src = first + (size_t)pp * tile_floats + (size_t)(16 * mb + out_m) * kTileN + out_n;
-            const f4 lo = __builtin_nontemporal_load(reinterpret_cast<const f4*>(src));
-            const f4 hi = __builtin_nontemporal_load(reinterpret_cast<const f4*>(src + 4));
 #pragma unroll
-            for (int e = 0; e < 4; e++) { v[e] += lo[e]; v[4 + e] += hi[e]; }
+            for (int e = 0; e < 8; e++) v[e] += __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         store_row(row, v);
     }
