@@ -283,6 +283,50 @@ __device__ __forceinline__ uint32_t lds_addr(const void* ptr) { return (uint32_t
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt = [3:0] and [15:14]).
 constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
+// A value the optimiser must treat as an unknown VGPR: keeps bit masks in registers so that
+// (x & mask) | magic selects the three-operand v_and_or_b32 (VOP3 cannot take literals on gfx9).
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+struct DequantConsts {
+    uint32_t lo, hi, ex;          // INT4 nibble masks and the 1024.0 magic
+    uint32_t top2, exp_man;       // FP6 plane mask and the s00eeemm field mask
+};
+
+__device__ __forceinline__ void dequant_int4_fast(uint32_t q, const DequantConsts& k, h2 (&r)[4])
+{
+    const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+    const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+    const uint32_t q8 = q >> 8;
+    r[0] = as_h2((q & k.lo) | k.ex) - bias_lo;
+    r[1] = __builtin_elementwise_fma(as_h2((q & k.hi) | k.ex), mul_hi, bias_hi);
+    r[2] = as_h2((q8 & k.lo) | k.ex) - bias_lo;
+    r[3] = __builtin_elementwise_fma(as_h2((q8 & k.hi) | k.ex), mul_hi, bias_hi);
+}
+
+typedef short s2 __attribute__((ext_vector_type(2)));
+
+// FP6 without the multiply by 4096 (the MFMA keeps fp16 sub-normal inputs; 4096 goes into the epilogue
+// scale).  p holds four bytes `s eee mm xx`, MSB first e1 e3 e0 e2; an arithmetic shift right by two of
+// each 16-bit half moves eee mm under the sign and the mask 0x9f00 clears the sign copies and the low byte.
+__device__ __forceinline__ void dequant_fp6_fast(uint32_t q2, uint32_t q4, const DequantConsts& k, h2 (&r)[4])
+{
+    const s2 two = {2, 2};
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const uint32_t lo = half == 0 ? (q4 >> 2) : (q4 << 2);
+        const uint32_t hi = half == 0 ? q2 : (q2 << 2);
+        const uint32_t p = (hi & k.top2) | (lo & ~k.top2);                       // v_bfi_b32
+        const uint32_t p8 = p << 8;
+        r[2 * half + 0] = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p) >> two) & k.exp_man);
+        r[2 * half + 1] = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p8) >> two) & k.exp_man);
+    }
+}
+
 template <bool FP6, bool G128, int DEPTH>
 __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                             int step_begin, int step_end, f4 (&acc)[1][8])
@@ -291,31 +335,52 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     constexpr int kSlot = FP6 ? 4096 : 3072;
     constexpr int kAOff = kSlot - 1024;
     constexpr int kOps = FP6 ? 4 : 3;                     // direct-to-LDS loads per step
+    constexpr int kUnroll = kGroup ? 4 : 2;               // steps per loop trip (step counts are multiples of it)
     const int lane = threadIdx.x & 63;
     const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
 
-    // ---- fetch side (lane = position in the slot)
-    const int g4_granule = lane ^ ((lane >> 4) & 3);
+    DequantConsts kc;
+    kc.lo = vgpr_const(0x000f000fu);
+    kc.hi = vgpr_const(0x00f000f0u);
+    kc.ex = vgpr_const(0x64006400u);
+    kc.top2 = vgpr_const(0xc0c0c0c0u);
+    kc.exp_man = vgpr_const(0x9f009f00u);
+
+    // ---- fetch side (lane = position in the slot).  Uniform 64-bit bases advance on the scalar unit;
+    // each lane only contributes a constant 32-bit offset.
+    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
     const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
-    const unsigned char* g4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
-                              (size_t)ti.tcol * 1024 + g4_granule * 16;
+    const unsigned char* base4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                                 (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4;
     const int lg = lane & 31;
-    const unsigned char* g2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
-                              (size_t)(lane >> 5) * row2 + (lg ^ (lg >> 4)) * 16;
+    const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
+    const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
+                                 (size_t)(2 * step_begin) * row2;
     const int a_m = lane >> 2;
     const bool a_active = ti.mtile * 16 + a_m < p.m;
-    const uint16_t* a_src = p.A + (size_t)(a_active ? ti.mtile * 16 + a_m : 0) * p.k + 8 * ((lane & 3) ^ (a_m >> 2));
-    const uint16_t* gs_src = p.s_int4 + (size_t)ti.tcol * kTileN + 2 * lane;
+    const uint32_t va = (uint32_t)(a_active ? a_m : 0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ (a_m >> 2));
+    const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)ti.mtile * 16 * p.k) +
+                                  (size_t)step_begin * 64;
+    const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
+    const uint32_t vgs = 4 * lane;
     unsigned char* gs_ring = ring + DEPTH * kSlot;        // four 256-byte slabs of group scales
 
-    auto issue = [&](int sp, int slot) {
+    int issued = step_begin;                              // next step to fetch (clamped at the last one)
+    const int last = step_end - 1;
+    auto issue = [&](int slot) {
         unsigned char* dst = ring + slot * kSlot;
-        const unsigned char* src4 = g4 + (size_t)(2 * sp) * row4;
-        dma16(src4, dst);
-        dma16(src4 + row4, dst + 1024);
-        if (FP6) dma16(g2 + (size_t)(2 * sp) * row2, dst + 2048);
-        if (a_active) dma16(a_src + 32 * sp, dst + kAOff);
-        if (kGroup && (sp & 3) == 0) dma4(gs_src + (size_t)(sp >> 2) * p.n4, gs_ring + ((sp >> 2) & 3) * 256);
+        dma16(base4 + v4, dst);
+        dma16(base4 + row4 + v4, dst + 1024);
+        if (FP6) dma16(base2 + v2, dst + 2048);
+        if (a_active) dma16(base_a + va, dst + kAOff);
+        if (kGroup && (issued & 3) == 0)
+            dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & 3) * 256);
+        if (issued < last) {                              // uniform: pointers move on the scalar unit
+            issued++;
+            base4 += 2 * row4;
+            base2 += 2 * row2;
+            base_a += 64;
+        }
     };
 
     // ---- read side (lane = MFMA identity)
@@ -330,30 +395,10 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const int q = i;                                      // result side: quarter of the column slots
     const uint32_t rdgs = lds_addr(gs_ring) + (64 * (q >> 1) + 4 * (q & 1)) * 2;
 
-    f4 grp[8];
-    if (kGroup) {
-#pragma unroll
-        for (int t = 0; t < 8; t++) grp[t] = f4{0.f, 0.f, 0.f, 0.f};
-    }
-
-    const int last = step_end - 1;
-    int slot_in = 0;
-#pragma unroll 1
-    for (int d = 0; d < DEPTH - 1; d++) {
-        const int sp = step_begin + d;
-        issue(sp < last ? sp : last, slot_in);
-        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
-    }
-    int slot_out = 0;
-#pragma unroll 1
-    for (int s = step_begin; s < step_end; s++) {
-        const int sp = s + DEPTH - 1;
-        issue(sp < last ? sp : last, slot_in);
-        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    // One k step out of ring slot `slot_out` into dst (fresh = start a new sum).
+    auto step = [&](int slot_out, f4 (&dst)[8], bool fresh) {
         __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 1)));
-
         const uint32_t so = slot_out * kSlot;
-        slot_out = slot_out + 1 == DEPTH ? 0 : slot_out + 1;
         u4 q0, q1, araw;
         u2 t0 = {0, 0}, t1 = {0, 0};
         if (FP6) {
@@ -378,27 +423,45 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
         asm volatile("" : "+v"(q0), "+v"(q1));
         if (FP6) asm volatile("" : "+v"(t0), "+v"(t1));
         const h8 av = __builtin_bit_cast(h8, araw);
+        const f4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             h2 r0[4], r1[4];
             if (FP6) {
-                dequant_fp6(t0[j >> 1] << (4 * (j & 1)), q0[j], r0);
-                dequant_fp6(t1[j >> 1] << (4 * (j & 1)), q1[j], r1);
+                dequant_fp6_fast(t0[j >> 1] << (4 * (j & 1)), q0[j], kc, r0);
+                dequant_fp6_fast(t1[j >> 1] << (4 * (j & 1)), q1[j], kc, r1);
             } else {
-                dequant_int4(q0[j], r0);
-                dequant_int4(q1[j], r1);
+                dequant_int4_fast(q0[j], kc, r0);
+                dequant_int4_fast(q1[j], kc, r1);
             }
             const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
             const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
-            if (kGroup) {
-                grp[2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, grp[2 * j + 0], 0, 0, 0);
-                grp[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, grp[2 * j + 1], 0, 0, 0);
-            } else {
-                acc[0][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, acc[0][2 * j + 0], 0, 0, 0);
-                acc[0][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, acc[0][2 * j + 1], 0, 0, 0);
-            }
+            dst[2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, fresh ? zero : dst[2 * j + 0], 0, 0, 0);
+            dst[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, fresh ? zero : dst[2 * j + 1], 0, 0, 0);
         }
-        if (kGroup && (s & 3) == 3) {
+    };
+
+    int slot_in = 0;
+#pragma unroll 1
+    for (int d = 0; d < DEPTH - 1; d++) {
+        issue(slot_in);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    }
+    int slot_out = 0;
+    f4 grp[8];
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s += kUnroll) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            issue(slot_in);
+            slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+            if (kGroup)
+                step(slot_out, grp, u == 0);
+            else
+                step(slot_out, acc[0], false);
+            slot_out = slot_out + 1 == DEPTH ? 0 : slot_out + 1;
+        }
+        if (kGroup) {
             // end of a 128-row group: fold it into the running sum with its scales (fp32)
             const uint32_t ga = rdgs + ((s >> 2) & 3) * 256;
             u2 sv[8];
@@ -416,19 +479,22 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
                 acc[0][t][1] += (float)lo[1] * grp[t][1];
                 acc[0][t][2] += (float)hi[0] * grp[t][2];
                 acc[0][t][3] += (float)hi[1] * grp[t][3];
-                grp[t] = f4{0.f, 0.f, 0.f, 0.f};
             }
         }
     }
     // Redundant tail prefetches may still be landing in the ring, which the epilogue reuses.
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    if (FP6) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[0][t] *= 4096.0f;  // the deferred e3m2 exponent re-bias
+    }
 }
 
 constexpr int ring_bytes_per_wave(int depth) { return depth * 3072 + 1024; }
 constexpr int fp6_depth(int depth) { return ring_bytes_per_wave(depth) / 4096; }
 
 template <bool G128, int DEPTH>
-__global__ __launch_bounds__(kThreads) void gemm_m16_kernel(const GemmArgs p)
+__global__ __launch_bounds__(kThreads, 2) void gemm_m16_kernel(const GemmArgs p)
 {
     constexpr int kWaveLds = ring_bytes_per_wave(DEPTH);
     constexpr int kLds = kWaves * kWaveLds > kRedBytes ? kWaves * kWaveLds : kRedBytes;
@@ -436,7 +502,7 @@ __global__ __launch_bounds__(kThreads) void gemm_m16_kernel(const GemmArgs p)
     __shared__ int s_is_last;
 
     const TileInfo ti = locate_tile(p);
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
     int step_begin, step_end;
     wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
 
