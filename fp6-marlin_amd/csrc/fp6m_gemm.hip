@@ -274,6 +274,11 @@ __device__ __forceinline__ void dma16(const void* gsrc, unsigned char* lds_dst)
 {
     __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 0);
 }
+// Same, with the non-temporal hint: for the packed words, which are read exactly once.
+__device__ __forceinline__ void dma16_stream(const void* gsrc, unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 2);
+}
 __device__ __forceinline__ void dma4(const void* gsrc, unsigned char* lds_dst)
 {
     __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 4, 0, 0);
@@ -327,14 +332,26 @@ __device__ __forceinline__ void dequant_fp6_fast(uint32_t q2, uint32_t q4, const
     }
 }
 
-template <bool FP6, bool G128, int DEPTH>
+// s_waitcnt immediate that waits for lgkmcnt <= n only.
+constexpr int lgkmcnt_only(int n) { return 15 | (3 << 14) | (7 << 4) | ((n & 15) << 8); }
+
+struct StepRegs {
+    u4 q0, q1;          // 4-bit plane / INT4 words of the two k-blocks
+    u2 t0, t1;          // FP6 2-bit plane
+    uint32_t a[4];      // activations in MFMA operand order
+};
+
+// AROWS = rows of A a slot holds (4 or 16): 64 bytes per row and step.
+template <bool FP6, bool G128, int DEPTH, int AROWS>
 __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                             int step_begin, int step_end, f4 (&acc)[1][8])
 {
+    static_assert(DEPTH >= 3, "needs two steps of look-ahead");
     constexpr bool kGroup = G128 && !FP6;                 // group scales apply to INT4 tiles only
-    constexpr int kSlot = FP6 ? 4096 : 3072;
-    constexpr int kAOff = kSlot - 1024;
+    constexpr int kAOff = FP6 ? 3072 : 2048;
+    constexpr int kSlot = kAOff + AROWS * 64;
     constexpr int kOps = FP6 ? 4 : 3;                     // direct-to-LDS loads per step
+    constexpr int kReads = FP6 ? 8 : 6;                   // LDS reads per step
     constexpr int kUnroll = kGroup ? 4 : 2;               // steps per loop trip (step counts are multiples of it)
     const int lane = threadIdx.x & 63;
     const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
@@ -357,8 +374,8 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
                                  (size_t)(2 * step_begin) * row2;
     const int a_m = lane >> 2;
-    const bool a_active = ti.mtile * 16 + a_m < p.m;
-    const uint32_t va = (uint32_t)(a_active ? a_m : 0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ (a_m >> 2));
+    const bool a_active = a_m < AROWS && ti.mtile * 16 + a_m < p.m;
+    const uint32_t va = (uint32_t)(a_active ? a_m : 0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3));
     const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)ti.mtile * 16 * p.k) +
                                   (size_t)step_begin * 64;
     const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
@@ -369,9 +386,9 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const int last = step_end - 1;
     auto issue = [&](int slot) {
         unsigned char* dst = ring + slot * kSlot;
-        dma16(base4 + v4, dst);
-        dma16(base4 + row4 + v4, dst + 1024);
-        if (FP6) dma16(base2 + v2, dst + 2048);
+        dma16_stream(base4 + v4, dst);
+        dma16_stream(base4 + row4 + v4, dst + 1024);
+        if (FP6) dma16_stream(base2 + v2, dst + 2048);
         if (a_active) dma16(base_a + va, dst + kAOff);
         if (kGroup && (issued & 3) == 0)
             dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & 3) * 256);
@@ -389,50 +406,46 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
     const int gr2 = owner >> 1;
     const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
+    const int ar = c & (AROWS - 1);                       // rows beyond AROWS re-read a valid row; their sums are never stored
     uint32_t rda[4];
 #pragma unroll
-    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * c + (d ^ (c >> 2))) * 16 + 4 * i;
+    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * ar + (d ^ ((ar >> 2) & 3))) * 16 + 4 * i;
     const int q = i;                                      // result side: quarter of the column slots
     const uint32_t rdgs = lds_addr(gs_ring) + (64 * (q >> 1) + 4 * (q & 1)) * 2;
 
-    // One k step out of ring slot `slot_out` into dst (fresh = start a new sum).
-    auto step = [&](int slot_out, f4 (&dst)[8], bool fresh) {
-        __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 1)));
-        const uint32_t so = slot_out * kSlot;
-        u4 q0, q1, araw;
-        u2 t0 = {0, 0}, t1 = {0, 0};
+    // kReads LDS reads of one step, not waited for.
+    auto fetch = [&](StepRegs& r, int slot) {
+        const uint32_t so = slot * kSlot;
         if (FP6) {
             asm volatile(
                 "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
                 "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
-                : "=&v"(q0), "=&v"(q1), "=&v"(t0), "=&v"(t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
+                : "=&v"(r.q0), "=&v"(r.q1), "=&v"(r.t0), "=&v"(r.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
         } else {
             asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
-                         : "=&v"(q0), "=&v"(q1) : "v"(rd4 + so) : "memory");
+                         : "=&v"(r.q0), "=&v"(r.q1) : "v"(rd4 + so) : "memory");
         }
-        {
-            uint32_t a0, a1, a2, a3;
-            asm volatile(
-                "ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7\n\t"
-                "s_waitcnt lgkmcnt(0)"
-                : "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3)
-                : "v"(rda[0] + so), "v"(rda[1] + so), "v"(rda[2] + so), "v"(rda[3] + so) : "memory");
-            araw = u4{a0, a1, a2, a3};
-        }
-        // the wait above also covers q0/q1/t0/t1 (LDS returns in order); tie them to it for the compiler
-        asm volatile("" : "+v"(q0), "+v"(q1));
-        if (FP6) asm volatile("" : "+v"(t0), "+v"(t1));
-        const h8 av = __builtin_bit_cast(h8, araw);
+        asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7"
+                     : "=&v"(r.a[0]), "=&v"(r.a[1]), "=&v"(r.a[2]), "=&v"(r.a[3])
+                     : "v"(rda[0] + so), "v"(rda[1] + so), "v"(rda[2] + so), "v"(rda[3] + so) : "memory");
+    };
+    // After the counter wait, the registers of `r` hold their data: make every later use depend on it.
+    auto settle = [&](StepRegs& r) {
+        asm volatile("" : "+v"(r.q0), "+v"(r.q1), "+v"(r.a[0]), "+v"(r.a[1]), "+v"(r.a[2]), "+v"(r.a[3]));
+        if (FP6) asm volatile("" : "+v"(r.t0), "+v"(r.t1));
+    };
+    auto compute = [&](const StepRegs& r, f4 (&dst)[8], bool fresh) {
+        const h8 av = __builtin_bit_cast(h8, u4{r.a[0], r.a[1], r.a[2], r.a[3]});
         const f4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             h2 r0[4], r1[4];
             if (FP6) {
-                dequant_fp6_fast(t0[j >> 1] << (4 * (j & 1)), q0[j], kc, r0);
-                dequant_fp6_fast(t1[j >> 1] << (4 * (j & 1)), q1[j], kc, r1);
+                dequant_fp6_fast(r.t0[j >> 1] << (4 * (j & 1)), r.q0[j], kc, r0);
+                dequant_fp6_fast(r.t1[j >> 1] << (4 * (j & 1)), r.q1[j], kc, r1);
             } else {
-                dequant_int4_fast(q0[j], kc, r0);
-                dequant_int4_fast(q1[j], kc, r1);
+                dequant_int4_fast(r.q0[j], kc, r0);
+                dequant_int4_fast(r.q1[j], kc, r1);
             }
             const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
             const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
@@ -441,13 +454,18 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
         }
     };
 
+    // Pipeline: while step s is being computed, the LDS reads of step s+1 are in flight and the
+    // direct-to-LDS loads of steps s+2 .. s+DEPTH-1 are outstanding.
     int slot_in = 0;
 #pragma unroll 1
     for (int d = 0; d < DEPTH - 1; d++) {
         issue(slot_in);
         slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
     }
-    int slot_out = 0;
+    StepRegs regs[2];
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+    fetch(regs[0], 0);
+    int slot_rd = 1;                                      // slot of the step whose LDS reads come next
     f4 grp[8];
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
@@ -455,11 +473,15 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
         for (int u = 0; u < kUnroll; u++) {
             issue(slot_in);
             slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));   // step s+u+1 has landed
+            fetch(regs[(u + 1) & 1], slot_rd);
+            slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
+            __builtin_amdgcn_s_waitcnt(lgkmcnt_only(kReads));             // reads of step s+u (older) are done
+            settle(regs[u & 1]);
             if (kGroup)
-                step(slot_out, grp, u == 0);
+                compute(regs[u & 1], grp, u == 0);
             else
-                step(slot_out, acc[0], false);
-            slot_out = slot_out + 1 == DEPTH ? 0 : slot_out + 1;
+                compute(regs[u & 1], acc[0], false);
         }
         if (kGroup) {
             // end of a 128-row group: fold it into the running sum with its scales (fp32)
@@ -472,6 +494,7 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
                 : "=&v"(sv[0]), "=&v"(sv[1]), "=&v"(sv[2]), "=&v"(sv[3]), "=&v"(sv[4]), "=&v"(sv[5]), "=&v"(sv[6]),
                   "=&v"(sv[7])
                 : "v"(ga) : "memory");
+            settle(regs[0]);                              // lgkmcnt(0) also completed the look-ahead reads
 #pragma unroll
             for (int t = 0; t < 8; t++) {
                 const h2 lo = as_h2(sv[t][0]), hi = as_h2(sv[t][1]);
@@ -482,24 +505,37 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
             }
         }
     }
-    // Redundant tail prefetches may still be landing in the ring, which the epilogue reuses.
-    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    // Redundant tail prefetches and look-ahead reads may still be in flight; the epilogue reuses the ring.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    settle(regs[0]);
     if (FP6) {
 #pragma unroll
         for (int t = 0; t < 8; t++) acc[0][t] *= 4096.0f;  // the deferred e3m2 exponent re-bias
     }
 }
 
-constexpr int ring_bytes_per_wave(int depth) { return depth * 3072 + 1024; }
-constexpr int fp6_depth(int depth) { return ring_bytes_per_wave(depth) / 4096; }
+// LDS per wave: DEPTH slots of an INT4 tile plus four 256-byte group-scale slabs; an FP6 tile (slots
+// 1 KiB larger) gets as many slots as fit in the same space.
+constexpr int int4_ring_bytes(int depth, int arows) { return depth * (2048 + arows * 64) + 1024; }
+constexpr int fp6_depth(int depth, int arows)
+{
+    return int4_ring_bytes(depth, arows) / (3072 + arows * 64) > 3 ? int4_ring_bytes(depth, arows) / (3072 + arows * 64) : 3;
+}
+constexpr int ring_bytes_per_wave(int depth, int arows)
+{
+    return int4_ring_bytes(depth, arows) > fp6_depth(depth, arows) * (3072 + arows * 64)
+               ? int4_ring_bytes(depth, arows)
+               : fp6_depth(depth, arows) * (3072 + arows * 64);
+}
 
-template <bool G128, int DEPTH>
+template <bool G128, int DEPTH, int AROWS>
 __global__ __launch_bounds__(kThreads, 2) void gemm_m16_kernel(const GemmArgs p)
 {
-    constexpr int kWaveLds = ring_bytes_per_wave(DEPTH);
+    constexpr int kWaveLds = ring_bytes_per_wave(DEPTH, AROWS);
     constexpr int kLds = kWaves * kWaveLds > kRedBytes ? kWaves * kWaveLds : kRedBytes;
+    static_assert(kLds >= kRedBytes + 16, "the arrival flag lives behind the reduction slab");
     __shared__ __attribute__((aligned(16))) unsigned char smem[kLds];
-    __shared__ int s_is_last;
+    int* const s_is_last_ptr = reinterpret_cast<int*>(smem + kRedBytes);   // free once the ring has drained
 
     const TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
@@ -512,11 +548,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_m16_kernel(const GemmArgs p)
     unsigned char* ring = smem + wave * kWaveLds;
     if (step_begin < step_end) {
         if (ti.fp6)
-            stream_tile<true, G128, fp6_depth(DEPTH)>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile<true, G128, fp6_depth(DEPTH, AROWS), AROWS>(p, ti, ring, step_begin, step_end, acc);
         else
-            stream_tile<false, G128, DEPTH>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile<false, G128, DEPTH, AROWS>(p, ti, ring, step_begin, step_end, acc);
     }
-    finish_tile<1>(p, ti, acc, ti.fp6 || !G128, smem, &s_is_last);
+    finish_tile<1>(p, ti, acc, ti.fp6 || !G128, smem, s_is_last_ptr);
 }
 
 // ------------------------------------------------------------------------------------------------ m > 16: register-staged kernel
@@ -717,16 +753,32 @@ int ensure_scratch(int dev, DeviceScratch** out)
     return FP6M_OK;
 }
 
-constexpr int kRingDepth = 4;
+template <int DEPTH, int AROWS>
+void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
+{
+    if (g128)
+        hipLaunchKernelGGL((gemm_m16_kernel<true, DEPTH, AROWS>), grid, dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((gemm_m16_kernel<false, DEPTH, AROWS>), grid, dim3(kThreads), 0, stream, a);
+}
 
 template <int MB>
 void launch(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
     if (MB == 1) {
-        if (g128)
-            hipLaunchKernelGGL((gemm_m16_kernel<true, kRingDepth>), grid, dim3(kThreads), 0, stream, a);
-        else
-            hipLaunchKernelGGL((gemm_m16_kernel<false, kRingDepth>), grid, dim3(kThreads), 0, stream, a);
+        int depth = 4;
+        if (const char* e = getenv("FP6M_DEPTH")) depth = atoi(e);
+        if (a.m <= 4) {
+            if (depth == 3) launch_m16<3, 4>(a, g128, grid, stream);
+            else if (depth == 5) launch_m16<5, 4>(a, g128, grid, stream);
+            else if (depth == 6) launch_m16<6, 4>(a, g128, grid, stream);
+            else launch_m16<4, 4>(a, g128, grid, stream);
+        } else {
+            if (depth == 3) launch_m16<3, 16>(a, g128, grid, stream);
+            else if (depth == 5) launch_m16<5, 16>(a, g128, grid, stream);
+            else if (depth == 6) launch_m16<6, 16>(a, g128, grid, stream);
+            else launch_m16<4, 16>(a, g128, grid, stream);
+        }
     } else {
         if (g128)
             hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
