@@ -215,10 +215,13 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
             if (p.ksplit == 1) {
                 store_row(row, v);
             } else {
-                // agent-scope stores go straight to the level all XCDs share: no cache-wide write-back later
-                float* dst = my_partial + (size_t)(16 * mb + out_m) * kTileN + out_n;
+                // Agent-scope stores go straight to the level all XCDs share (no cache-wide write-back
+                // later).  Element e of thread t lives at [mb][e][t]: every store instruction of a wave
+                // writes 256 contiguous bytes.
+                float* dst = my_partial + (size_t)mb * 8 * kThreads + threadIdx.x;
 #pragma unroll
-                for (int e = 0; e < 8; e++) __hip_atomic_store(dst + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int e = 0; e < 8; e++)
+                    __hip_atomic_store(dst + e * kThreads, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
@@ -246,10 +249,27 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
         float v[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) v[e] = 0.f;
-        for (int pp = 0; pp < p.ksplit; pp++) {
-            const float* src = first + (size_t)pp * tile_floats + (size_t)(16 * mb + out_m) * kTileN + out_n;
+        // Four partners' loads are in flight at a time; the sum runs in partner order (deterministic).
+        const float* src = first + (size_t)mb * 8 * kThreads + threadIdx.x;
+        int pp = 0;
+        for (; pp + 4 <= p.ksplit; pp += 4) {
+            float t[4][8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] += __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    t[u][e] = __hip_atomic_load(src + (size_t)(pp + u) * tile_floats + e * kThreads, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] += t[u][e];
+        }
+        for (; pp < p.ksplit; pp++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                v[e] += __hip_atomic_load(src + (size_t)pp * tile_floats + e * kThreads, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
         }
         store_row(row, v);
     }
