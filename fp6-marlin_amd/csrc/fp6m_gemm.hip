@@ -17,6 +17,7 @@
 //  * INT4 and FP6 tiles are entries of one tile list handled by the same launch.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <cstdlib>
 #include <mutex>
 
@@ -54,7 +55,23 @@ struct GemmArgs {
     int tiles6;               // FP6 tiles come first in the tile list
     int tiles;                // all tiles
     int ksplit;               // workgroups per (tile, m-tile)
+    // m <= 16 kernel: the FP6 and the INT4 region are covered by separate ranges of workgroups
+    int ks6, ks4;             // k parts (workgroups) per tile group, per region
+    int groups6, groups4;     // tile groups (WN adjacent tiles) per region
+#ifdef FP6M_TIMELINE
+    unsigned long long* timeline;   // 8 realtime-clock stamps per workgroup (performance debugging builds only)
+#endif
 };
+
+#ifdef FP6M_TIMELINE
+#define FP6M_MARK(p, i)                                                                            \
+    do {                                                                                           \
+        if (threadIdx.x == 0 && (p).timeline)                                                      \
+            (p).timeline[(size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#else
+#define FP6M_MARK(p, i) do { } while (0)
+#endif
 
 // ------------------------------------------------------------------------------------------------ bit tricks
 
@@ -225,6 +242,7 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
             }
         }
     }
+    FP6M_MARK(p, 3);
     if (p.ksplit == 1) return;
 
     // Publish the partial, then count arrivals; the last workgroup of the tile finishes it.  Partials
@@ -233,12 +251,14 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
     // invalidate, which would stall every workgroup of the XCD.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
+    FP6M_MARK(p, 4);
     int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
     if (threadIdx.x == 0) {
         const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         *s_is_last = (seen == p.ksplit - 1);
     }
     __syncthreads();
+    FP6M_MARK(p, 5);
     if (!*s_is_last) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     const float* first = p.scratch + (size_t)(ti.mtile * p.tiles + ti.tile) * p.ksplit * tile_floats;
@@ -273,6 +293,7 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& t
         }
         store_row(row, v);
     }
+    FP6M_MARK(p, 6);
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -400,7 +421,8 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
                                   (size_t)step_begin * 64;
     const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
     const uint32_t vgs = 4 * lane;
-    unsigned char* gs_ring = ring + DEPTH * kSlot;        // four 256-byte slabs of group scales
+    constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;        // 256-byte slabs of group scales: 2 suffice up to depth 5
+    unsigned char* gs_ring = ring + DEPTH * kSlot;
 
     int issued = step_begin;                              // next step to fetch (clamped at the last one)
     const int last = step_end - 1;
@@ -411,7 +433,7 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
         if (FP6) dma16_stream(base2 + v2, dst + 2048);
         if (a_active) dma16(base_a + va, dst + kAOff);
         if (kGroup && (issued & 3) == 0)
-            dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & 3) * 256);
+            dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & kScaleMask) * 256);
         if (issued < last) {                              // uniform: pointers move on the scalar unit
             issued++;
             base4 += 2 * row4;
@@ -484,6 +506,7 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     }
     StepRegs regs[2];
     __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+    FP6M_MARK(p, 1);
     fetch(regs[0], 0);
     int slot_rd = 1;                                      // slot of the step whose LDS reads come next
     f4 grp[8];
@@ -505,7 +528,7 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
         }
         if (kGroup) {
             // end of a 128-row group: fold it into the running sum with its scales (fp32)
-            const uint32_t ga = rdgs + ((s >> 2) & 3) * 256;
+            const uint32_t ga = rdgs + ((s >> 2) & kScaleMask) * 256;
             u2 sv[8];
             asm volatile(
                 "ds_read_b64 %0, %8\n\tds_read_b64 %1, %8 offset:16\n\tds_read_b64 %2, %8 offset:32\n\t"
@@ -534,45 +557,190 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     }
 }
 
-// LDS per wave: DEPTH slots of an INT4 tile plus four 256-byte group-scale slabs; an FP6 tile (slots
-// 1 KiB larger) gets as many slots as fit in the same space.
-constexpr int int4_ring_bytes(int depth, int arows) { return depth * (2048 + arows * 64) + 1024; }
-constexpr int fp6_depth(int depth, int arows)
+// LDS per wave: the larger of an INT4 ring (D4 slots + the group-scale slabs) and an FP6 ring (D6
+// slots), and at least the 16 x 128 fp32 row slab of the epilogue.
+constexpr int scale_slab_bytes(int depth) { return depth <= 5 ? 512 : 1024; }
+constexpr int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
+constexpr int wave_lds_bytes(int d4, int d6, int arows)
 {
-    return int4_ring_bytes(depth, arows) / (3072 + arows * 64) > 3 ? int4_ring_bytes(depth, arows) / (3072 + arows * 64) : 3;
-}
-constexpr int ring_bytes_per_wave(int depth, int arows)
-{
-    return int4_ring_bytes(depth, arows) > fp6_depth(depth, arows) * (3072 + arows * 64)
-               ? int4_ring_bytes(depth, arows)
-               : fp6_depth(depth, arows) * (3072 + arows * 64);
+    return max3(d4 * (2048 + arows * 64) + scale_slab_bytes(d4), d6 * (3072 + arows * 64), 16 * kRedStride * 4);
 }
 
-template <bool G128, int DEPTH, int AROWS>
-__global__ __launch_bounds__(kThreads, 2) void gemm_m16_kernel(const GemmArgs p)
+// The m <= 16 kernel.
+//
+// A workgroup is WN x WK waves: WN adjacent 128-column tiles (one per wave column, so the workgroup
+// reads WN KiB contiguous runs of every k-block row) times WK consecutive slices of the workgroup's
+// k range.  Waves never synchronise in the main loop.  Epilogue: every wave turns its MFMA fragments
+// into fp32 rows in its own drained ring, one barrier, then wave (wn, wk) sums rows wk, wk+WK, ... of
+// tile wn over the WK slices (fixed order) with lane L owning columns 2L, 2L+1.  With one k part per
+// tile group it scales and writes C; otherwise it publishes the rows with agent-scope stores, the
+// workgroup bumps the group's counter, and the workgroup that arrives last sums all parts in part order.
+template <int WN, int WK>
+__device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti, bool tile_valid, int wn, int wk,
+                                          int ks, int slot_base, int* counter, f4 (&acc)[1][8],
+                                          bool per_column_scale, unsigned char* smem, int wave_lds, int* flag)
 {
-    constexpr int kWaveLds = ring_bytes_per_wave(DEPTH, AROWS);
-    constexpr int kLds = kWaves * kWaveLds > kRedBytes ? kWaves * kWaveLds : kRedBytes;
-    static_assert(kLds >= kRedBytes + 16, "the arrival flag lives behind the reduction slab");
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kLds];
-    int* const s_is_last_ptr = reinterpret_cast<int*>(smem + kRedBytes);   // free once the ring has drained
+    constexpr int RMAX = (16 + WK - 1) / WK;                             // rows one wave finishes
+    constexpr int PCHUNK = 32 / RMAX;                                    // parts whose loads are in flight together
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15, q = lane >> 4;
+    const int wave = wk * WN + wn;
+    if (tile_valid) {
+        float* mine = reinterpret_cast<float*>(smem + wave * wave_lds) + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[0][t];
+    }
+    __syncthreads();
+    FP6M_MARK(p, 3);
 
-    const TileInfo ti = locate_tile(p);
+    const int nrows = p.m < 16 ? p.m : 16;
+    float s0 = 1.0f, s1 = 1.0f;
+    if (tile_valid && per_column_scale) {
+        const uint16_t* sp = ti.fp6 ? p.s_fp6 : p.s_int4;
+        const int nr = ti.tcol * kTileN + 2 * lane;                      // even column inside the region
+        const h2 sv = *reinterpret_cast<const h2*>(sp + (nr & ~31) + scale_slot(nr & 31));
+        s0 = (float)sv[0];
+        s1 = (float)sv[1];
+    }
+    uint16_t* c_out = p.C + ti.col0 + 2 * lane;
+    auto store_row = [&](int m, float v0, float v1) {
+        h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
+        *reinterpret_cast<h2*>(c_out + (size_t)m * p.n) = o;
+    };
+
+    // Sum of the WK slices of my rows.
+    float v0[RMAX], v1[RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+        v0[r] = 0.f;
+        v1[r] = 0.f;
+        const int m = wk + r * WK;
+        if (tile_valid && m < nrows) {
+#pragma unroll
+            for (int j = 0; j < WK; j++) {
+                const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + (j * WN + wn) * wave_lds) +
+                                                          m * kRedStride + 2 * lane);
+                v0[r] += v[0];
+                v1[r] += v[1];
+            }
+        }
+    }
+    if (ks == 1) {
+#pragma unroll
+        for (int r = 0; r < RMAX; r++)
+            if (tile_valid && wk + r * WK < nrows) store_row(wk + r * WK, v0[r], v1[r]);
+        return;
+    }
+
+    // Publish.  A slot holds [WN tiles][16 rows][128 columns] fp32; 8-byte agent-scope accesses.
+    constexpr size_t kSlotU64 = (size_t)WN * 16 * kTileN / 2;
+    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) + (size_t)slot_base * kSlotU64 +
+                                (size_t)wn * (16 * kTileN / 2) + lane;
+    unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+        const int m = wk + r * WK;
+        if (tile_valid && m < nrows) {
+            const f2 v = {v0[r], v1[r]};
+            __hip_atomic_store(my + m * (kTileN / 2), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");               // my stores have completed
+    __syncthreads();
+    FP6M_MARK(p, 4);
+    if (threadIdx.x == 0) {
+        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = (seen == ks - 1);
+    }
+    __syncthreads();
+    FP6M_MARK(p, 5);
+    if (!*flag) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+        v0[r] = 0.f;
+        v1[r] = 0.f;
+    }
+    for (int pp = 0; pp < ks; pp += PCHUNK) {
+        unsigned long long t[PCHUNK][RMAX];
+#pragma unroll
+        for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                const int m = wk + r * WK;
+                t[u][r] = 0;
+                if (tile_valid && m < nrows && pp + u < ks)
+                    t[u][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + m * (kTileN / 2), __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+        for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                const f2 v = __builtin_bit_cast(f2, t[u][r]);
+                v0[r] += v[0];
+                v1[r] += v[1];
+            }
+    }
+#pragma unroll
+    for (int r = 0; r < RMAX; r++)
+        if (tile_valid && wk + r * WK < nrows) store_row(wk + r * WK, v0[r], v1[r]);
+    FP6M_MARK(p, 6);
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <bool G128, int AROWS, int WN, int WK, int D4, int D6>
+// second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
+__global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArgs p)
+{
+    constexpr int NW = WN * WK;
+    constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);
+    __shared__ __attribute__((aligned(16))) unsigned char smem[NW * kWaveLds + 16];
+
+    FP6M_MARK(p, 0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
-    int step_begin, step_end;
-    wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
+    const int wn = wave % WN, wk = wave / WN;
+    const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int wgs6 = p.groups6 * p.ks6;                                  // the FP6 region's workgroups come first
+    TileInfo ti;
+    ti.fp6 = logical < wgs6;
+    const int local = ti.fp6 ? logical : logical - wgs6;
+    const int groups = ti.fp6 ? p.groups6 : p.groups4;
+    const int ks = ti.fp6 ? p.ks6 : p.ks4;
+    ti.part = local / groups;                                            // part-major: neighbours share k, adjoin in n
+    const int group = local - ti.part * groups;
+    ti.tcol = group * WN + wn;
+    ti.region_n = ti.fp6 ? p.qc : p.n4;
+    const bool tile_valid = ti.tcol * kTileN < ti.region_n;
+    ti.tile = ti.fp6 ? ti.tcol : p.tiles6 + ti.tcol;
+    ti.mtile = 0;
+    ti.col0 = (ti.fp6 ? p.n4 : 0) + ti.tcol * kTileN;
+
+    constexpr int unit_steps = G128 ? 4 : 2;
+    const int units = p.k / (32 * unit_steps);
+    const int kp = ti.part * WK + wk, kparts = ks * WK;
+    const int step_begin = (int)((long long)units * kp / kparts) * unit_steps;
+    const int step_end = (int)((long long)units * (kp + 1) / kparts) * unit_steps;
 
     f4 acc[1][8];
 #pragma unroll
     for (int t = 0; t < 8; t++) acc[0][t] = f4{0.f, 0.f, 0.f, 0.f};
     unsigned char* ring = smem + wave * kWaveLds;
-    if (step_begin < step_end) {
+    if (tile_valid && step_begin < step_end) {
         if (ti.fp6)
-            stream_tile<true, G128, fp6_depth(DEPTH, AROWS), AROWS>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile<true, G128, D6, AROWS>(p, ti, ring, step_begin, step_end, acc);
         else
-            stream_tile<false, G128, DEPTH, AROWS>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile<false, G128, D4, AROWS>(p, ti, ring, step_begin, step_end, acc);
     }
-    finish_tile<1>(p, ti, acc, ti.fp6 || !G128, smem, s_is_last_ptr);
+    FP6M_MARK(p, 2);
+    // scratch slots: FP6 groups first (groups6 * ks6 slots), then INT4 groups; counters likewise
+    const int slot_base = ti.fp6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
+    int* counter = p.counters + (ti.fp6 ? group : p.groups6 + group);
+    wg_finish<WN, WK>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, ti.fp6 || !G128, smem, kWaveLds,
+                      reinterpret_cast<int*>(smem + NW * kWaveLds));
+    FP6M_MARK(p, 7);
 }
 
 // ------------------------------------------------------------------------------------------------ m > 16: register-staged kernel
@@ -773,38 +941,44 @@ int ensure_scratch(int dev, DeviceScratch** out)
     return FP6M_OK;
 }
 
-template <int DEPTH, int AROWS>
+// m <= 16 configurations: rows of A per ring slot, WN x WK waves, ring depths of INT4 / FP6 tiles.
+//   0: rows <= 4,  one tile x four k slices per workgroup, four ring slots (three for FP6 tiles)
+//   1: rows <= 16, same shape, 1 KiB of A per slot
+// Workgroups of several adjacent tiles (WN > 1) were measured and were never faster on MI355X; the
+// kernel keeps the template parameter, only WN = 1 is instantiated.
+template <int AROWS, int WN, int WK, int D4, int D6>
 void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
     if (g128)
-        hipLaunchKernelGGL((gemm_m16_kernel<true, DEPTH, AROWS>), grid, dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL((gemm_m16_kernel<true, AROWS, WN, WK, D4, D6>), grid, dim3(64 * WN * WK), 0, stream, a);
     else
-        hipLaunchKernelGGL((gemm_m16_kernel<false, DEPTH, AROWS>), grid, dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL((gemm_m16_kernel<false, AROWS, WN, WK, D4, D6>), grid, dim3(64 * WN * WK), 0, stream, a);
+}
+
+struct M16Config {
+    int id, wn, wk;
+};
+
+inline M16Config m16_config(int m)
+{
+    return m <= 4 ? M16Config{0, 1, 4} : M16Config{1, 1, 4};
+}
+
+inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
+{
+    if (cfg.id == 0)
+        launch_m16<4, 1, 4, 4, 3>(a, g128, grid, stream);
+    else
+        launch_m16<16, 1, 4, 4, 3>(a, g128, grid, stream);
 }
 
 template <int MB>
 void launch(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
-    if (MB == 1) {
-        int depth = 4;
-        if (const char* e = getenv("FP6M_DEPTH")) depth = atoi(e);
-        if (a.m <= 4) {
-            if (depth == 3) launch_m16<3, 4>(a, g128, grid, stream);
-            else if (depth == 5) launch_m16<5, 4>(a, g128, grid, stream);
-            else if (depth == 6) launch_m16<6, 4>(a, g128, grid, stream);
-            else launch_m16<4, 4>(a, g128, grid, stream);
-        } else {
-            if (depth == 3) launch_m16<3, 16>(a, g128, grid, stream);
-            else if (depth == 5) launch_m16<5, 16>(a, g128, grid, stream);
-            else if (depth == 6) launch_m16<6, 16>(a, g128, grid, stream);
-            else launch_m16<4, 16>(a, g128, grid, stream);
-        }
-    } else {
-        if (g128)
-            hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
-        else
-            hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
-    }
+    if (g128)
+        hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
 }
 
 }  // namespace fp6m
@@ -866,6 +1040,10 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     a.qc = qc;
     a.tiles6 = qc / kTileN;
     a.tiles = prob_n / kTileN;
+#ifdef FP6M_TIMELINE
+    a.timeline = nullptr;
+    if (const char* e = getenv("FP6M_TIMELINE_PTR")) a.timeline = reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0));
+#endif
 
     const int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     const int rows_per_tile = 16 * mb;
@@ -880,30 +1058,60 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
         a.C = static_cast<uint16_t*>(C) + (size_t)rows0 * prob_n;
         a.m = prob_m - rows0 < mtiles * rows_per_tile ? prob_m - rows0 : mtiles * rows_per_tile;
 
-        // How many workgroups share one tile's k range: enough to put several workgroups on every CU,
-        // never so many that a wave gets less than one unit of k, that the partial tiles outgrow the
-        // scratch, or that partial-sum traffic rivals the weight stream.
-        const long long base = (long long)a.tiles * mtiles;
-        const long long want_wgs = (long long)scratch->cus * 4;
-        long long ks = (want_wgs + base - 1) / base;
-        const long long ks_k = units / (kWaves * 2) > 0 ? units / (kWaves * 2) : 1;
-        if (ks > ks_k) ks = ks_k;
-        const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
-        if (ks > traffic_cap) ks = traffic_cap;
-        if (sms > 0 && ks > sms) ks = sms;
         const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
-        while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
-        if (const char* e = getenv("FP6M_KSPLIT")) {
-            const int v = atoi(e);
-            if (v >= 1 && (size_t)base * v * tile_bytes <= kScratchBytes && v * kWaves <= units) ks = v;
+        const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
+        long long env_ks = 0;
+        if (const char* e = getenv("FP6M_KSPLIT")) env_ks = atoi(e);   // tuning/testing override
+        if (mb == 1) {
+            // m <= 16.  Each region (FP6, INT4) has its own number of k parts (workgroups) per tile group;
+            // FP6 steps cost about twice an INT4 step, so the FP6 region is split twice as finely.  The
+            // split is bounded so that every wave keeps at least one k unit, partial-sum traffic stays
+            // well below the weight stream and the partial tiles fit the scratch.
+            const M16Config cfg = m16_config(a.m);
+            a.groups6 = (a.tiles6 + cfg.wn - 1) / cfg.wn;
+            a.groups4 = (a.tiles - a.tiles6 + cfg.wn - 1) / cfg.wn;
+            const long long groups = a.groups6 + a.groups4;
+            const long long ks_k = units / cfg.wk > 0 ? units / cfg.wk : 1;   // at least one k unit per wave
+            // Measured on MI355X: the kernel is fastest with about one and a half workgroups per CU
+            // (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle), as long as every
+            // wave keeps at least four k steps.
+            const long long target_wgs = (long long)scratch->cus * 3 / 2;
+            long long ks = (target_wgs + groups / 2) / groups;
+            const long long ks_steps = prob_k / 32 / (4 * cfg.wk) > 0 ? prob_k / 32 / (4 * cfg.wk) : 1;
+            if (ks > ks_steps) ks = ks_steps;
+            if (ks > ks_k) ks = ks_k;
+            if (ks > traffic_cap) ks = traffic_cap;
+            if (sms > 0 && ks > sms) ks = sms;
+            if (env_ks >= 1) ks = env_ks;
+            if (ks < 1) ks = 1;
+            const size_t slot_bytes = (size_t)cfg.wn * 16 * kTileN * sizeof(float);
+            while (ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > kScratchBytes) ks--;
+            a.ks4 = (int)ks;
+            a.ks6 = (int)(2 * ks <= ks_k ? 2 * ks : (ks > ks_k ? ks : ks_k));
+            if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
+            a.ksplit = a.ks4;
+            dim3 grid((unsigned)(a.groups6 * a.ks6 + a.groups4 * a.ks4), 1);
+            if (getenv("FP6M_VERBOSE"))
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u\n", a.m, prob_n,
+                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x);
+            launch_m16_any(cfg, a, g128, grid, st);
+        } else {
+            // m > 16: a task is one workgroup (four waves splitting k) on one (tile, m tile, k part).
+            const long long base = (long long)a.tiles * mtiles;
+            const long long want_wgs = (long long)scratch->cus * 4;
+            long long ks = (want_wgs + base - 1) / base;
+            const long long ks_k = units / (kWaves * 2) > 0 ? units / (kWaves * 2) : 1;
+            if (ks > ks_k) ks = ks_k;
+            if (ks > traffic_cap) ks = traffic_cap;
+            if (sms > 0 && ks > sms) ks = sms;
+            if (env_ks >= 1) ks = env_ks;
+            while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
+            if (ks < 1) ks = 1;
+            a.ksplit = (int)ks;
+            dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
+            if (mb == 2) launch<2>(a, g128, grid, st);
+            else launch<4>(a, g128, grid, st);
         }
-        if (ks < 1) ks = 1;
-        a.ksplit = (int)ks;
-
-        dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
-        if (mb == 1) launch<1>(a, g128, grid, st);
-        else if (mb == 2) launch<2>(a, g128, grid, st);
-        else launch<4>(a, g128, grid, st);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return hip_fail(e);
     }
