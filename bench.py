@@ -30,6 +30,10 @@ for _p in (ROOT, os.path.join(ROOT, "fp6-marlin_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the headline workload (mean of its four GEMMs): FETCH_SIZE + WRITE_SIZE from two
+# `rocprofv3 --pmc` runs of `bench.py --traffic-probe`, each scaled by what the same counter reads for a
+# 256 MiB device copy (x2.000 and x1.000); figures in profiles/gemm_m16_kernel_decode7b_hbm_traffic.txt.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27194837
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLAMA7B = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
 LLAMA70B = [(8192, 10240), (8192, 8192), (8192, 57344), (28672, 8192)]
@@ -106,6 +110,23 @@ def cpu_baseline(torch):
                       f"{nbytes} weight bytes; host has {os.cpu_count()} logical cores"}
 
 
+def graphed(torch, step, layers, steps):
+    """fn(i) for time_region that replays a HIP graph of `layers` consecutive steps (launch-bound loops
+    belong in graphs); steps that do not fill a whole graph run eagerly."""
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(layers):
+            step(i)
+    whole = steps // layers
+
+    def run(i):
+        if i < whole:
+            graph.replay()
+        else:
+            step(i - whole)
+    return run, whole + (steps - whole * layers)
+
+
 def headline(args):
     import torch
     import fp6_marlin
@@ -126,10 +147,20 @@ def headline(args):
 
     for i in range(args.warmup):
         step(i)
-    wall, ev = time_region(torch, step, args.steps)
+    torch.cuda.synchronize()
+    if args.no_graph:
+        wall, ev = time_region(torch, step, args.steps)
+    else:
+        fn, calls = graphed(torch, step, layers, args.steps)
+        wall, ev = time_region(torch, fn, calls)
     for i in range(max(2, args.warmup // 4)):
         step_fp16(i)
-    wall16, _ = time_region(torch, step_fp16, args.steps)
+    torch.cuda.synchronize()
+    if args.no_graph:
+        wall16, _ = time_region(torch, step_fp16, args.steps)
+    else:
+        fn16, calls16 = graphed(torch, step_fp16, layers, args.steps)
+        wall16, _ = time_region(torch, fn16, calls16)
 
     gbs = step_bytes * args.steps / wall / 1e9
     per_launch = ev / (args.steps * launches_per_step)
@@ -143,14 +174,34 @@ def headline(args):
                                "INT4 g128 + 256 FP6 columns, one step = one layer (4 GEMMs), 8 layers cycled",
                    "m": m, "quant_cols": qc, "group_size": gs, "weight_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "fp6m::gemm_kernel<1, true>", "us_per_launch": round(per_launch * 1e6, 3),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "fp6m::gemm_m16_kernel<true, 4, 1, 4, 4, 3>", "us_per_launch": round(per_launch * 1e6, 3),
                      "bytes_per_launch": step_bytes // launches_per_step},
         "cpu_baseline": cpu_baseline(torch),
         "fp16_hipblaslt": {"ms_per_step": round(wall16 / args.steps * 1e3, 5),
                            "speedup": round(wall16 / wall, 3)},
     }
     print(json.dumps(out), flush=True)
+
+
+def traffic_probe():
+    """Work for a counter run: a plain copy of known size calibrates FETCH_SIZE / WRITE_SIZE (both must read
+    256 MiB for it), then the four headline GEMMs run three times over distinct weights."""
+    import torch
+    import fp6_marlin
+    gen = torch.Generator().manual_seed(0)
+    fp6_marlin.init(0)
+    src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    probs = [[Problem(torch, 1, k, n, 256, 128, gen) for (k, n) in LLAMA7B] for _ in range(3)]
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    for layer in probs:
+        for p in layer:
+            p.run(fp6_marlin.mul)
+    torch.cuda.synchronize()
+    print("traffic probe done: copy of", src.numel(), "bytes; GEMM weight bytes per launch",
+          [p.bytes for p in probs[0]], flush=True)
 
 
 def sweep(args):
@@ -206,11 +257,16 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
+    ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 256 MiB device copy, then one layer of GEMMs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the op shards along N without any exchange); "
                  "run with --gpus 1")
-    if args.sweep:
+    if args.traffic_probe:
+        traffic_probe()
+    elif args.sweep:
         sweep(args)
     else:
         headline(args)
