@@ -743,6 +743,364 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     FP6M_MARK(p, 7);
 }
 
+// ------------------------------------------------------------------------------------------------ 16 < m: ring kernel with MB row blocks
+//
+// Same ring and lane routing as the m <= 16 kernel, but a slot carries MB blocks of 16 rows of A (1 KiB
+// each) and every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per
+// 16*MB rows.  A workgroup is one tile x four k slices; blockIdx.y walks the row tiles.  Group scales are
+// applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more
+// registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
+// the number of direct-to-LDS loads per step is constant) and never stored.
+
+template <int MB>
+struct StepRegsMB {
+    u4 q0, q1;
+    u2 t0, t1;
+    uint32_t a[MB][4];
+};
+
+template <int OFF>
+__device__ __forceinline__ void lds_read_a4(uint32_t (&a)[4], const uint32_t (&addr)[4])
+{
+    asm volatile(
+        "ds_read_b32 %0, %4 offset:%8\n\tds_read_b32 %1, %5 offset:%8\n\t"
+        "ds_read_b32 %2, %6 offset:%8\n\tds_read_b32 %3, %7 offset:%8"
+        : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3])
+        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "n"(OFF) : "memory");
+}
+template <int MB, int I = 0>
+__device__ __forceinline__ void lds_read_a_blocks(uint32_t (&a)[MB][4], const uint32_t (&addr)[4])
+{
+    if constexpr (I < MB) {
+        lds_read_a4<I * 1024>(a[I], addr);
+        lds_read_a_blocks<MB, I + 1>(a, addr);
+    }
+}
+
+template <bool FP6, bool G128, int DEPTH, int MB>
+__device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
+                                               int step_begin, int step_end, f4 (&acc)[MB][8])
+{
+    static_assert(DEPTH >= 3, "needs two steps of look-ahead");
+    constexpr bool kGroup = G128 && !FP6;
+    constexpr int kAOff = FP6 ? 3072 : 2048;
+    constexpr int kSlot = kAOff + MB * 1024;
+    constexpr int kOps = (FP6 ? 3 : 2) + MB;              // direct-to-LDS loads per step
+    constexpr int kUnroll = kGroup ? 4 : 2;
+    static_assert(kOps * (DEPTH - 2) <= 63, "vmcnt is a 6-bit counter");
+    const int lane = threadIdx.x & 63;
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+
+    DequantConsts kc;
+    kc.lo = vgpr_const(0x000f000fu);
+    kc.hi = vgpr_const(0x00f000f0u);
+    kc.ex = vgpr_const(0x64006400u);
+    kc.top2 = vgpr_const(0xc0c0c0c0u);
+    kc.exp_man = vgpr_const(0x9f009f00u);
+
+    // ---- fetch side
+    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
+    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const unsigned char* base4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                                 (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4;
+    const int lg = lane & 31;
+    const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
+    const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
+                                 (size_t)(2 * step_begin) * row2;
+    const int a_m = lane >> 2;
+    const int tile_row0 = ti.mtile * 16 * MB;
+    uint32_t va[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        int row = tile_row0 + 16 * mb + a_m;
+        row = row < p.m ? row : p.m - 1;
+        va[mb] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3));
+    }
+    const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
+                                  (size_t)step_begin * 64;
+    const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
+    const uint32_t vgs = 4 * lane;
+    constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;
+    unsigned char* gs_ring = ring + DEPTH * kSlot;
+
+    int issued = step_begin;
+    const int last = step_end - 1;
+    auto issue = [&](int slot) {
+        unsigned char* dst = ring + slot * kSlot;
+        dma16_stream(base4 + v4, dst);
+        dma16_stream(base4 + row4 + v4, dst + 1024);
+        if (FP6) dma16_stream(base2 + v2, dst + 2048);
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) dma16(base_a + va[mb], dst + kAOff + mb * 1024);
+        if (kGroup && (issued & 3) == 0)
+            dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & kScaleMask) * 256);
+        if (issued < last) {
+            issued++;
+            base4 += 2 * row4;
+            base2 += 2 * row2;
+            base_a += 64;
+        }
+    };
+
+    // ---- read side
+    const int owner = 32 * sigma + 4 * l + i;
+    const uint32_t ring_lds = lds_addr(ring);
+    const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
+    const int gr2 = owner >> 1;
+    const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
+    uint32_t rda[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * c + (d ^ ((c >> 2) & 3))) * 16 + 4 * i;
+    const uint32_t rdgs = lds_addr(gs_ring) + (64 * sigma + l) * 2;    // weight side: column (j, half) at +32j +16half
+
+    uint32_t gs_next[8];
+    h2 gs_cur[8];
+    auto fetch = [&](StepRegsMB<MB>& r, int slot, bool with_scales, int group) {
+        const uint32_t so = slot * kSlot;
+        if (FP6) {
+            asm volatile(
+                "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
+                "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
+                : "=&v"(r.q0), "=&v"(r.q1), "=&v"(r.t0), "=&v"(r.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
+        } else {
+            asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
+                         : "=&v"(r.q0), "=&v"(r.q1) : "v"(rd4 + so) : "memory");
+        }
+        const uint32_t addr[4] = {rda[0] + so, rda[1] + so, rda[2] + so, rda[3] + so};
+        lds_read_a_blocks<MB>(r.a, addr);
+        if (kGroup && with_scales) {
+            const uint32_t ga = rdgs + (group & kScaleMask) * 256;
+            asm volatile(
+                "ds_read_u16 %0, %8\n\tds_read_u16 %1, %8 offset:16\n\tds_read_u16 %2, %8 offset:32\n\t"
+                "ds_read_u16 %3, %8 offset:48\n\tds_read_u16 %4, %8 offset:64\n\tds_read_u16 %5, %8 offset:80\n\t"
+                "ds_read_u16 %6, %8 offset:96\n\tds_read_u16 %7, %8 offset:112"
+                : "=&v"(gs_next[0]), "=&v"(gs_next[1]), "=&v"(gs_next[2]), "=&v"(gs_next[3]), "=&v"(gs_next[4]),
+                  "=&v"(gs_next[5]), "=&v"(gs_next[6]), "=&v"(gs_next[7])
+                : "v"(ga) : "memory");
+        }
+    };
+    auto settle = [&](StepRegsMB<MB>& r, bool with_scales) {
+        asm volatile("" : "+v"(r.q0), "+v"(r.q1));
+        if (FP6) asm volatile("" : "+v"(r.t0), "+v"(r.t1));
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) asm volatile("" : "+v"(r.a[mb][0]), "+v"(r.a[mb][1]), "+v"(r.a[mb][2]), "+v"(r.a[mb][3]));
+        if (kGroup && with_scales) {
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                asm volatile("" : "+v"(gs_next[t]));
+                gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
+            }
+        }
+    };
+    auto compute = [&](const StepRegsMB<MB>& r) {
+        h8 av[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) av[mb] = __builtin_bit_cast(h8, u4{r.a[mb][0], r.a[mb][1], r.a[mb][2], r.a[mb][3]});
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h2 r0[4], r1[4];
+            if (FP6) {
+                dequant_fp6_fast(r.t0[j >> 1] << (4 * (j & 1)), r.q0[j], kc, r0);
+                dequant_fp6_fast(r.t1[j >> 1] << (4 * (j & 1)), r.q1[j], kc, r1);
+            } else {
+                dequant_int4_fast(r.q0[j], kc, r0);
+                dequant_int4_fast(r.q1[j], kc, r1);
+                if (kGroup) {
+#pragma unroll
+                    for (int x = 0; x < 4; x++) {
+                        r0[x] = r0[x] * gs_cur[2 * j + (x >> 1)];
+                        r1[x] = r1[x] * gs_cur[2 * j + (x >> 1)];
+                    }
+                }
+            }
+            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);
+            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                acc[mb][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av[mb], acc[mb][2 * j + 0], 0, 0, 0);
+                acc[mb][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av[mb], acc[mb][2 * j + 1], 0, 0, 0);
+            }
+        }
+    };
+
+    int slot_in = 0;
+#pragma unroll 1
+    for (int d = 0; d < DEPTH - 1; d++) {
+        issue(slot_in);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    }
+    StepRegsMB<MB> regs[2];
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+    fetch(regs[0], 0, true, step_begin >> 2);
+    __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
+    settle(regs[0], true);
+    int slot_rd = 1;
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s += kUnroll) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            issue(slot_in);
+            slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));   // step s+u+1 (and its group scales) landed
+            const bool next_group = kGroup && u == kUnroll - 1;           // step s+u+1 starts a 128-row group
+            fetch(regs[(u + 1) & 1], slot_rd, next_group, (s + u + 1) >> 2);
+            slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
+            compute(regs[u & 1]);
+            __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
+            settle(regs[(u + 1) & 1], next_group);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    if (FP6) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int t = 0; t < 8; t++) acc[mb][t] *= 4096.0f;
+    }
+}
+
+// Epilogue of the MB kernel: block by block, the four k slices are summed through LDS (wave wk finishes
+// rows wk, wk+4, ... of the block, lane L owns columns 2L, 2L+1); then C is written, or the rows are
+// published and the last-arriving workgroup of the (tile, row tile) gathers all parts in part order.
+template <int MB>
+__device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, f4 (&acc)[MB][8],
+                                             bool per_column_scale, unsigned char* smem, int wave_lds, int* flag)
+{
+    constexpr int WK = kWaves, RMAX = 16 / WK, PCHUNK = 8;
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15, q = lane >> 4;
+    const int row0 = ti.mtile * 16 * MB;
+    const int nrows = p.m - row0 < 16 * MB ? p.m - row0 : 16 * MB;
+    float s0 = 1.0f, s1 = 1.0f;
+    if (per_column_scale) {
+        const uint16_t* sp = ti.fp6 ? p.s_fp6 : p.s_int4;
+        const int nr = ti.tcol * kTileN + 2 * lane;
+        const h2 sv = *reinterpret_cast<const h2*>(sp + (nr & ~31) + scale_slot(nr & 31));
+        s0 = (float)sv[0];
+        s1 = (float)sv[1];
+    }
+    uint16_t* c_out = p.C + (size_t)row0 * p.n + ti.col0 + 2 * lane;
+    auto store_row = [&](int row, float v0, float v1) {
+        h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
+        *reinterpret_cast<h2*>(c_out + (size_t)row * p.n) = o;
+    };
+    constexpr size_t kSlotU64 = (size_t)MB * 16 * kTileN / 2;
+    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) +
+                                (size_t)(ti.mtile * p.tiles + ti.tile) * ks * kSlotU64 + lane;
+    unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
+
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        __syncthreads();
+        float* mine = reinterpret_cast<float*>(smem + wk * wave_lds) + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[mb][t];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            const int m = wk + r * WK, row = 16 * mb + m;
+            if (row < nrows) {
+                float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                for (int j = 0; j < WK; j++) {
+                    const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + j * wave_lds) +
+                                                              m * kRedStride + 2 * lane);
+                    v0 += v[0];
+                    v1 += v[1];
+                }
+                if (ks == 1) {
+                    store_row(row, v0, v1);
+                } else {
+                    const f2 v = {v0, v1};
+                    __hip_atomic_store(my + (size_t)row * (kTileN / 2), __builtin_bit_cast(unsigned long long, v),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+    }
+    if (ks == 1) return;
+
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
+    if (threadIdx.x == 0) {
+        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = (seen == ks - 1);
+    }
+    __syncthreads();
+    if (!*flag) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll 1
+    for (int mb = 0; mb < MB; mb++) {
+        float v0[RMAX], v1[RMAX];
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            v0[r] = 0.f;
+            v1[r] = 0.f;
+        }
+        for (int pp = 0; pp < ks; pp += PCHUNK) {
+            unsigned long long t[PCHUNK][RMAX];
+#pragma unroll
+            for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+                for (int r = 0; r < RMAX; r++) {
+                    const int row = 16 * mb + wk + r * WK;
+                    t[u][r] = 0;
+                    if (row < nrows && pp + u < ks)
+                        t[u][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + (size_t)row * (kTileN / 2),
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+            for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+                for (int r = 0; r < RMAX; r++) {
+                    const f2 v = __builtin_bit_cast(f2, t[u][r]);
+                    v0[r] += v[0];
+                    v1[r] += v[1];
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            const int row = 16 * mb + wk + r * WK;
+            if (row < nrows) store_row(row, v0[r], v1[r]);
+        }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr int mb_wave_lds(int mb, int d4, int d6)
+{
+    return max3(d4 * (2048 + mb * 1024) + scale_slab_bytes(d4), d6 * (3072 + mb * 1024), 16 * kRedStride * 4);
+}
+
+template <bool G128, int MB, int D4, int D6>
+__global__ __launch_bounds__(kThreads, 1) void gemm_mb_kernel(const GemmArgs p)
+{
+    constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kWaves * kWaveLds + 16];
+
+    const TileInfo ti = locate_tile(p);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int step_begin, step_end;
+    wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
+
+    f4 acc[MB][8];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
+    unsigned char* ring = smem + wave * kWaveLds;
+    if (step_begin < step_end) {
+        if (ti.fp6)
+            stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+        else
+            stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
+    }
+    wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, ti.fp6 || !G128, smem, kWaveLds,
+                     reinterpret_cast<int*>(smem + kWaves * kWaveLds));
+}
+
 // ------------------------------------------------------------------------------------------------ m > 16: register-staged kernel
 //
 // Up to 64 rows of A per workgroup pass (MB 16-row blocks): each dequantised weight fragment feeds MB
@@ -972,13 +1330,22 @@ inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, d
         launch_m16<16, 1, 4, 4, 3>(a, g128, grid, stream);
 }
 
-template <int MB>
-void launch(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
+template <int MB, int D4, int D6>
+void launch_mb(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
+    if (getenv("FP6M_OLD_MB")) {   // previous register-staged kernel, kept for comparison while tuning
+        if constexpr (MB <= 4) {
+            if (g128)
+                hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
+            else
+                hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
+            return;
+        }
+    }
     if (g128)
-        hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6>), grid, dim3(kThreads), 0, stream, a);
     else
-        hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
+        hipLaunchKernelGGL((gemm_mb_kernel<false, MB, D4, D6>), grid, dim3(kThreads), 0, stream, a);
 }
 
 }  // namespace fp6m
@@ -1045,7 +1412,11 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     if (const char* e = getenv("FP6M_TIMELINE_PTR")) a.timeline = reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0));
 #endif
 
-    const int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
+    int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : (prob_m <= 64 ? 4 : 8));
+    if (const char* e = getenv("FP6M_MB")) {   // tuning/testing override
+        const int v = atoi(e);
+        if (prob_m > 16 && (v == 2 || v == 4 || v == 8)) mb = v;
+    }
     const int rows_per_tile = 16 * mb;
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
     const int units = g128 ? prob_k / 128 : prob_k / 64;
@@ -1096,21 +1467,27 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
                         prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x);
             launch_m16_any(cfg, a, g128, grid, st);
         } else {
-            // m > 16: a task is one workgroup (four waves splitting k) on one (tile, m tile, k part).
+            // m > 16: a task is one workgroup (one tile x four k slices) on one row tile and k part.
+            // Split k only as far as needed to give every CU a workgroup; partial tiles are 16*MB rows
+            // of fp32, so the split is also capped by their traffic relative to the weight stream.
             const long long base = (long long)a.tiles * mtiles;
-            const long long want_wgs = (long long)scratch->cus * 4;
-            long long ks = (want_wgs + base - 1) / base;
+            long long ks = scratch->cus / base;
             const long long ks_k = units / (kWaves * 2) > 0 ? units / (kWaves * 2) : 1;
+            const long long cap = (long long)prob_k / (16LL * rows_per_tile) > 0 ? (long long)prob_k / (16LL * rows_per_tile) : 1;
             if (ks > ks_k) ks = ks_k;
-            if (ks > traffic_cap) ks = traffic_cap;
+            if (ks > cap) ks = cap;
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
-            while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
             if (ks < 1) ks = 1;
+            while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
             a.ksplit = (int)ks;
             dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
-            if (mb == 2) launch<2>(a, g128, grid, st);
-            else launch<4>(a, g128, grid, st);
+            if (getenv("FP6M_VERBOSE"))
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d grid=%ux%u\n", a.m, prob_n, prob_k, mb, mtiles,
+                        a.ksplit, grid.x, grid.y);
+            if (mb == 2) launch_mb<2, 4, 3>(a, g128, grid, st);
+            else if (mb == 4) launch_mb<4, 3, 3>(a, g128, grid, st);
+            else launch_mb<8, 3, 3>(a, g128, grid, st);
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return hip_fail(e);
