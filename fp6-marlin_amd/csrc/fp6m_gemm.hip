@@ -326,6 +326,38 @@ __device__ __forceinline__ void dma4(const void* gsrc, unsigned char* lds_dst)
 }
 __device__ __forceinline__ uint32_t lds_addr(const void* ptr) { return (uint32_t)(uintptr_t)(const FP6M_AS3 void*)ptr; }
 
+// Direct-to-LDS loads in their scalar-base form: global address = sbase + voff + OFF, LDS address =
+// M0 + OFF + 16 * lane.  The immediate moves both sides, so loads whose LDS targets lie within 4 KiB of
+// each other share one M0 value (the global side is compensated in voff or sbase) and no vector address
+// arithmetic is left in the loop.  One wait state separates the M0 write from its first use.
+__device__ __forceinline__ void set_m0(uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_base) : "memory");
+}
+template <int OFF, bool STREAM>
+__device__ __forceinline__ void dma16_m0(const void* sbase, uint32_t voff)
+{
+    static_assert(OFF >= 0 && OFF < 4096, "13-bit signed immediate");
+    if constexpr (STREAM)
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2 nt" : : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+    else
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ void dma4_m0(const void* sbase, uint32_t voff)
+{
+    asm volatile("global_load_lds_dword %0, %1" : : "v"(voff), "s"(sbase) : "memory");
+}
+template <int MB, int A_OFF, int I = 0>
+__device__ __forceinline__ void dma_a_blocks(uint32_t slot_lds, const void* sbase_a, const uint32_t (&voff)[MB])
+{
+    if constexpr (I < MB) {
+        constexpr int lds_off = A_OFF + 1024 * I;
+        if constexpr (lds_off % 4096 == 0) set_m0(slot_lds + lds_off);
+        dma16_m0<lds_off % 4096, false>(sbase_a, voff[I]);
+        dma_a_blocks<MB, A_OFF, I + 1>(slot_lds, sbase_a, voff);
+    }
+}
+
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt = [3:0] and [15:14]).
 constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
@@ -752,11 +784,14 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
 // registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
 // the number of direct-to-LDS loads per step is constant) and never stored.
 
-template <int MB>
-struct StepRegsMB {
+struct WeightRegs {
     u4 q0, q1;
     u2 t0, t1;
-    uint32_t a[MB][4];
+};
+
+template <int N>
+struct Int {
+    static constexpr int value = N;
 };
 
 template <int OFF>
@@ -768,25 +803,104 @@ __device__ __forceinline__ void lds_read_a4(uint32_t (&a)[4], const uint32_t (&a
         : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3])
         : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "n"(OFF) : "memory");
 }
-template <int MB, int I = 0>
-__device__ __forceinline__ void lds_read_a_blocks(uint32_t (&a)[MB][4], const uint32_t (&addr)[4])
+
+// acc += w (16 columns x 32 k) * a (16 rows x 32 k), in place.  Written as asm so that the accumulator
+// stays in one register quad for the whole loop (AGPR when the kernel runs one wave per SIMD) and the
+// MFMAs keep their place between the LDS reads.  The hazards the compiler would pad for are handled
+// here: an MFMA must not read a VGPR in the two wait states after a VALU wrote it (register copies the
+// allocator places in front of the asm count), hence the s_nop; the loop never reads an accumulator
+// except as the addend of the same MFMA a full step later; the wait states before the first VALU read
+// of a result follow the loop.
+template <bool AGPR, bool FIRST>
+__device__ __forceinline__ void mfma_acc(f4& acc, const h8& w, const h8& a)
 {
-    if constexpr (I < MB) {
-        lds_read_a4<I * 1024>(a[I], addr);
-        lds_read_a_blocks<MB, I + 1>(a, addr);
+    if constexpr (AGPR && FIRST)
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
+    else if constexpr (AGPR)
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
+    else if constexpr (FIRST)
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
+    else
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
+}
+
+// Two of the four h2 a packed word expands to (half 0: fragment columns +0, half 1: columns +8).
+template <bool FP6>
+__device__ __forceinline__ void dequant_half(uint32_t q2, uint32_t q4, int half, const DequantConsts& k, h2& r0, h2& r1)
+{
+    if constexpr (FP6) {
+        const s2 two = {2, 2};
+        const uint32_t lo = half == 0 ? (q4 >> 2) : (q4 << 2);
+        const uint32_t hi = half == 0 ? q2 : (q2 << 2);
+        const uint32_t p = (hi & k.top2) | (lo & ~k.top2);
+        const uint32_t p8 = p << 8;
+        r0 = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p) >> two) & k.exp_man);
+        r1 = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p8) >> two) & k.exp_man);
+    } else {
+        const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+        const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+        const uint32_t q = half == 0 ? q4 : (q4 >> 8);
+        r0 = as_h2((q & k.lo) | k.ex) - bias_lo;
+        r1 = __builtin_elementwise_fma(as_h2((q & k.hi) | k.ex), mul_hi, bias_hi);
     }
 }
 
-template <bool FP6, bool G128, int DEPTH, int MB>
+struct MbCtx {
+    uint32_t abuf[4][4];
+    uint32_t addr_cur[4], addr_next[4];
+};
+
+// One step of the MB loop, fully static in BLK: block by block the 16 rows of A are multiplied into
+// the step's eight weight fragments.  Activations travel through a ring of four register buffers,
+// fetched from LDS two blocks ahead of their use (the latency hides behind 16 MFMAs); the s_waitcnt
+// immediates follow from the fixed issue order: [A(0), A(1)] from the previous step, the next step's
+// weight words (kExtra reads), then A(2), A(3), ...  After every MFMA `hook(block, t)` runs: the caller
+// uses it to dequantise the next step's fragments a few VALU instructions at a time.
+template <bool AGPR, int MB, int kExtra, int BLK = 0>
+struct MbBlocks {
+    template <int phase, typename Hook>
+    static __device__ __forceinline__ void run(MbCtx& cx, const h8 (&frag)[8], f4 (&acc)[MB][8], Hook&& hook)
+    {
+        if constexpr (BLK < MB) {
+            constexpr int nb = BLK + 2;
+            uint32_t (&dst)[4] = cx.abuf[(phase + nb) & 3];
+            if constexpr (nb < MB)
+                lds_read_a4<nb * 1024>(dst, cx.addr_cur);
+            else
+                lds_read_a4<(nb - MB) * 1024>(dst, cx.addr_next);
+            // block 0 needs A(0): A(1), the extra reads and A(2) may be outstanding; from block 1 on the
+            // extra reads must be complete as well
+            constexpr int allow = BLK == 0 ? (8 + kExtra < 15 ? 8 + kExtra : 15) : 8;
+            __builtin_amdgcn_s_waitcnt(lgkmcnt_only(allow));
+            uint32_t (&src)[4] = cx.abuf[(phase + BLK) & 3];
+            asm volatile("" : "+v"(src[0]), "+v"(src[1]), "+v"(src[2]), "+v"(src[3]));
+            const h8 av = __builtin_bit_cast(h8, u4{src[0], src[1], src[2], src[3]});
+            mfma_acc<AGPR, true>(acc[BLK][0], frag[0], av); hook(Int<BLK>{}, Int<0>{});
+            mfma_acc<AGPR, false>(acc[BLK][1], frag[1], av); hook(Int<BLK>{}, Int<1>{});
+            mfma_acc<AGPR, false>(acc[BLK][2], frag[2], av); hook(Int<BLK>{}, Int<2>{});
+            mfma_acc<AGPR, false>(acc[BLK][3], frag[3], av); hook(Int<BLK>{}, Int<3>{});
+            mfma_acc<AGPR, false>(acc[BLK][4], frag[4], av); hook(Int<BLK>{}, Int<4>{});
+            mfma_acc<AGPR, false>(acc[BLK][5], frag[5], av); hook(Int<BLK>{}, Int<5>{});
+            mfma_acc<AGPR, false>(acc[BLK][6], frag[6], av); hook(Int<BLK>{}, Int<6>{});
+            mfma_acc<AGPR, false>(acc[BLK][7], frag[7], av); hook(Int<BLK>{}, Int<7>{});
+            MbBlocks<AGPR, MB, kExtra, BLK + 1>::template run<phase>(cx, frag, acc, hook);
+        }
+    }
+};
+
+template <bool FP6, bool G128, int DEPTH, int MB, bool AGPR>
 __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                                int step_begin, int step_end, f4 (&acc)[MB][8])
 {
     static_assert(DEPTH >= 3, "needs two steps of look-ahead");
+    static_assert(MB == 2 || MB == 4 || MB == 8, "the A register ring assumes MB | 8");
     constexpr bool kGroup = G128 && !FP6;
     constexpr int kAOff = FP6 ? 3072 : 2048;
     constexpr int kSlot = kAOff + MB * 1024;
     constexpr int kOps = (FP6 ? 3 : 2) + MB;              // direct-to-LDS loads per step
     constexpr int kUnroll = kGroup ? 4 : 2;
+    constexpr int kW = FP6 ? 4 : 2;                       // LDS reads of one step's weight words
     static_assert(kOps * (DEPTH - 2) <= 63, "vmcnt is a 6-bit counter");
     const int lane = threadIdx.x & 63;
     const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
@@ -798,15 +912,19 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     kc.top2 = vgpr_const(0xc0c0c0c0u);
     kc.exp_man = vgpr_const(0x9f009f00u);
 
-    // ---- fetch side
-    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
+    // ---- fetch side: uniform 64-bit bases on the scalar unit, per-lane 32-bit offsets that never change.
+    // The offsets carry the compensation for the immediates (see dma16_m0): the second k-block of the
+    // words sits 1 KiB further in LDS and one row further in memory; the 2-bit plane and the A blocks
+    // get their compensation on the scalar base, so that the lane offsets stay non-negative.
     const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
+    const uint32_t v4b = v4 + (uint32_t)row4 - 1024;
     const unsigned char* base4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
                                  (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4;
     const int lg = lane & 31;
     const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
     const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
-                                 (size_t)(2 * step_begin) * row2;
+                                 (size_t)(2 * step_begin) * row2 - 2048;
     const int a_m = lane >> 2;
     const int tile_row0 = ti.mtile * 16 * MB;
     uint32_t va[MB];
@@ -814,26 +932,31 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     for (int mb = 0; mb < MB; mb++) {
         int row = tile_row0 + 16 * mb + a_m;
         row = row < p.m ? row : p.m - 1;
-        va[mb] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3));
+        va[mb] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3)) + 4096 -
+                 (kAOff + 1024 * mb) % 4096;
     }
     const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
-                                  (size_t)step_begin * 64;
+                                  (size_t)step_begin * 64 - 4096;
     const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
     const uint32_t vgs = 4 * lane;
     constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;
     unsigned char* gs_ring = ring + DEPTH * kSlot;
+    const uint32_t ring_lds = lds_addr(ring);
+    const uint32_t gs_lds = lds_addr(gs_ring);
 
     int issued = step_begin;
     const int last = step_end - 1;
     auto issue = [&](int slot) {
-        unsigned char* dst = ring + slot * kSlot;
-        dma16_stream(base4 + v4, dst);
-        dma16_stream(base4 + row4 + v4, dst + 1024);
-        if (FP6) dma16_stream(base2 + v2, dst + 2048);
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) dma16(base_a + va[mb], dst + kAOff + mb * 1024);
-        if (kGroup && (issued & 3) == 0)
-            dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & kScaleMask) * 256);
+        const uint32_t dst = ring_lds + slot * kSlot;
+        set_m0(dst);
+        dma16_m0<0, true>(base4, v4);
+        dma16_m0<1024, true>(base4, v4b);
+        if (FP6) dma16_m0<2048, true>(base2, v2);
+        dma_a_blocks<MB, kAOff>(dst, base_a, va);
+        if (kGroup && (issued & 3) == 0) {
+            set_m0(gs_lds + ((issued >> 2) & kScaleMask) * 256);
+            dma4_m0(base_gs + (size_t)(issued >> 2) * p.n4 * 2, vgs);
+        }
         if (issued < last) {
             issued++;
             base4 += 2 * row4;
@@ -844,83 +967,82 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
 
     // ---- read side
     const int owner = 32 * sigma + 4 * l + i;
-    const uint32_t ring_lds = lds_addr(ring);
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
     const int gr2 = owner >> 1;
     const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
     uint32_t rda[4];
 #pragma unroll
     for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * c + (d ^ ((c >> 2) & 3))) * 16 + 4 * i;
-    const uint32_t rdgs = lds_addr(gs_ring) + (64 * sigma + l) * 2;    // weight side: column (j, half) at +32j +16half
+    const uint32_t rdgs = gs_lds + (64 * sigma + l) * 2;    // weight side: column (j, half) at +32j +16half
 
     uint32_t gs_next[8];
     h2 gs_cur[8];
-    auto fetch = [&](StepRegsMB<MB>& r, int slot, bool with_scales, int group) {
+    MbCtx cx;
+    WeightRegs w;
+    auto fetch_w = [&](int slot) {
         const uint32_t so = slot * kSlot;
         if (FP6) {
             asm volatile(
                 "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
                 "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
-                : "=&v"(r.q0), "=&v"(r.q1), "=&v"(r.t0), "=&v"(r.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
+                : "=&v"(w.q0), "=&v"(w.q1), "=&v"(w.t0), "=&v"(w.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
         } else {
             asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
-                         : "=&v"(r.q0), "=&v"(r.q1) : "v"(rd4 + so) : "memory");
-        }
-        const uint32_t addr[4] = {rda[0] + so, rda[1] + so, rda[2] + so, rda[3] + so};
-        lds_read_a_blocks<MB>(r.a, addr);
-        if (kGroup && with_scales) {
-            const uint32_t ga = rdgs + (group & kScaleMask) * 256;
-            asm volatile(
-                "ds_read_u16 %0, %8\n\tds_read_u16 %1, %8 offset:16\n\tds_read_u16 %2, %8 offset:32\n\t"
-                "ds_read_u16 %3, %8 offset:48\n\tds_read_u16 %4, %8 offset:64\n\tds_read_u16 %5, %8 offset:80\n\t"
-                "ds_read_u16 %6, %8 offset:96\n\tds_read_u16 %7, %8 offset:112"
-                : "=&v"(gs_next[0]), "=&v"(gs_next[1]), "=&v"(gs_next[2]), "=&v"(gs_next[3]), "=&v"(gs_next[4]),
-                  "=&v"(gs_next[5]), "=&v"(gs_next[6]), "=&v"(gs_next[7])
-                : "v"(ga) : "memory");
+                         : "=&v"(w.q0), "=&v"(w.q1) : "v"(rd4 + so) : "memory");
         }
     };
-    auto settle = [&](StepRegsMB<MB>& r, bool with_scales) {
-        asm volatile("" : "+v"(r.q0), "+v"(r.q1));
-        if (FP6) asm volatile("" : "+v"(r.t0), "+v"(r.t1));
+    auto fetch_scales = [&](int group) {
+        const uint32_t ga = rdgs + (group & kScaleMask) * 256;
+        asm volatile(
+            "ds_read_u16 %0, %8\n\tds_read_u16 %1, %8 offset:16\n\tds_read_u16 %2, %8 offset:32\n\t"
+            "ds_read_u16 %3, %8 offset:48\n\tds_read_u16 %4, %8 offset:64\n\tds_read_u16 %5, %8 offset:80\n\t"
+            "ds_read_u16 %6, %8 offset:96\n\tds_read_u16 %7, %8 offset:112"
+            : "=&v"(gs_next[0]), "=&v"(gs_next[1]), "=&v"(gs_next[2]), "=&v"(gs_next[3]), "=&v"(gs_next[4]),
+              "=&v"(gs_next[5]), "=&v"(gs_next[6]), "=&v"(gs_next[7])
+            : "v"(ga) : "memory");
+    };
+    auto settle_scales = [&]() {
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) asm volatile("" : "+v"(r.a[mb][0]), "+v"(r.a[mb][1]), "+v"(r.a[mb][2]), "+v"(r.a[mb][3]));
-        if (kGroup && with_scales) {
-#pragma unroll
-            for (int t = 0; t < 8; t++) {
-                asm volatile("" : "+v"(gs_next[t]));
-                gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
-            }
+        for (int t = 0; t < 8; t++) {
+            asm volatile("" : "+v"(gs_next[t]));
+            gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
         }
     };
-    auto compute = [&](const StepRegsMB<MB>& r) {
-        h8 av[MB];
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) av[mb] = __builtin_bit_cast(h8, u4{r.a[mb][0], r.a[mb][1], r.a[mb][2], r.a[mb][3]});
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            h2 r0[4], r1[4];
-            if (FP6) {
-                dequant_fp6_fast(r.t0[j >> 1] << (4 * (j & 1)), r.q0[j], kc, r0);
-                dequant_fp6_fast(r.t1[j >> 1] << (4 * (j & 1)), r.q1[j], kc, r1);
-            } else {
-                dequant_int4_fast(r.q0[j], kc, r0);
-                dequant_int4_fast(r.q1[j], kc, r1);
-                if (kGroup) {
-#pragma unroll
-                    for (int x = 0; x < 4; x++) {
-                        r0[x] = r0[x] * gs_cur[2 * j + (x >> 1)];
-                        r1[x] = r1[x] * gs_cur[2 * j + (x >> 1)];
-                    }
-                }
-            }
-            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);
-            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                acc[mb][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av[mb], acc[mb][2 * j + 0], 0, 0, 0);
-                acc[mb][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av[mb], acc[mb][2 * j + 1], 0, 0, 0);
-            }
+    // A quarter of one j group (a "chunk": 4..8 VALU instructions): chunk = 4j + 2*half + word.  The
+    // word is tied to this point of the program first, the results after, so the instructions stay
+    // between the two MFMAs the chunk was placed between.
+    h2 part[2];
+    auto chunk = [&](int ck, h8 (&frag)[8]) {
+        const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
+        uint32_t q4 = word ? w.q1[j] : w.q0[j];
+        uint32_t q2 = 0;
+        asm volatile("" : "+v"(q4));
+        if (word) w.q1[j] = q4; else w.q0[j] = q4;
+        if (FP6) {
+            uint32_t t = word ? w.t1[j >> 1] : w.t0[j >> 1];
+            asm volatile("" : "+v"(t));
+            if (word) w.t1[j >> 1] = t; else w.t0[j >> 1] = t;
+            q2 = t << (4 * (j & 1));
         }
+        h2 r0, r1;
+        dequant_half<FP6>(q2, q4, half, kc, r0, r1);
+        if (kGroup) {
+            r0 = r0 * gs_cur[2 * j + half];
+            r1 = r1 * gs_cur[2 * j + half];
+        }
+        if (word == 0) {
+            part[0] = r0;
+            part[1] = r1;
+            asm volatile("" : "+v"(part[0]), "+v"(part[1]));
+        } else {
+            frag[2 * j + half] = join(part[0], part[1], r0, r1);
+            asm volatile("" : "+v"(frag[2 * j + half]));
+        }
+    };
+    auto slot_addrs = [&](uint32_t (&addr)[4], int slot) {
+        const uint32_t so = slot * kSlot;
+#pragma unroll
+        for (int d = 0; d < 4; d++) addr[d] = rda[d] + so;
     };
 
     int slot_in = 0;
@@ -929,11 +1051,17 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
         issue(slot_in);
         slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
     }
-    StepRegsMB<MB> regs[2];
+    h8 frag[2][8];
     __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
-    fetch(regs[0], 0, true, step_begin >> 2);
+    slot_addrs(cx.addr_next, 0);
+    fetch_w(0);
+    lds_read_a4<0>(cx.abuf[0], cx.addr_next);
+    lds_read_a4<1024>(cx.abuf[1], cx.addr_next);
+    if (kGroup) fetch_scales(step_begin >> 2);
     __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
-    settle(regs[0], true);
+    if (kGroup) settle_scales();
+#pragma unroll
+    for (int ck = 0; ck < 16; ck++) chunk(ck, frag[0]);
     int slot_rd = 1;
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
@@ -941,16 +1069,39 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
         for (int u = 0; u < kUnroll; u++) {
             issue(slot_in);
             slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));   // step s+u+1 (and its group scales) landed
-            const bool next_group = kGroup && u == kUnroll - 1;           // step s+u+1 starts a 128-row group
-            fetch(regs[(u + 1) & 1], slot_rd, next_group, (s + u + 1) >> 2);
+#pragma unroll
+            for (int d = 0; d < 4; d++) cx.addr_cur[d] = cx.addr_next[d];
+            slot_addrs(cx.addr_next, slot_rd);
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+            // step s+u+1 (and its group scales) has landed: read its words now, dequantise them
+            // between this step's MFMAs
+            fetch_w(slot_rd);
+            const bool next_group = kGroup && u == kUnroll - 1;       // step s+u+1 starts a 128-row group
+            if (next_group) fetch_scales((s + u + 1) >> 2);
             slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
-            compute(regs[u & 1]);
-            __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
-            settle(regs[(u + 1) & 1], next_group);
+            h8 (&cur)[8] = frag[u & 1];
+            h8 (&nxt)[8] = frag[(u + 1) & 1];
+            auto hook = [&](auto blk, auto t) {
+                constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
+                constexpr int avail = 8 * MB - 8;                     // chunks go after the MFMAs of blocks >= 1
+                if constexpr (mslot == 8) {
+                    if (next_group) settle_scales();
+                }
+                if constexpr (mslot >= 8) {
+                    constexpr int c0 = (mslot - 8) * 16 / avail, c1 = (mslot - 7) * 16 / avail;
+#pragma unroll
+                    for (int ck = c0; ck < c1; ck++) chunk(ck, nxt);
+                }
+            };
+            constexpr int kExtraMax = kW + (kGroup ? 8 : 0);
+            if ((u & 1) == 0)                                          // buffer of block 0: (u * MB) mod 4
+                MbBlocks<AGPR, MB, kExtraMax>::template run<0>(cx, cur, acc, hook);
+            else
+                MbBlocks<AGPR, MB, kExtraMax>::template run<(MB & 3)>(cx, cur, acc, hook);
         }
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");                   // MFMA results -> VALU reads
     if (FP6) {
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
@@ -1075,7 +1226,7 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 }
 
 template <bool G128, int MB, int D4, int D6>
-__global__ __launch_bounds__(kThreads, 1) void gemm_mb_kernel(const GemmArgs p)
+__global__ __launch_bounds__(kThreads, MB >= 4 ? 1 : 2) void gemm_mb_kernel(const GemmArgs p)
 {
     constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
     __shared__ __attribute__((aligned(16))) unsigned char smem[kWaves * kWaveLds + 16];
@@ -1093,9 +1244,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mb_kernel(const GemmArgs p)
     unsigned char* ring = smem + wave * kWaveLds;
     if (step_begin < step_end) {
         if (ti.fp6)
-            stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile_mb<true, G128, D6, MB, (MB >= 4)>(p, ti, ring, step_begin, step_end, acc);
         else
-            stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile_mb<false, G128, D4, MB, (MB >= 4)>(p, ti, ring, step_begin, step_end, acc);
     }
     wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, ti.fp6 || !G128, smem, kWaveLds,
                      reinterpret_cast<int*>(smem + kWaves * kWaveLds));
