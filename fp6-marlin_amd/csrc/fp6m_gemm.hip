@@ -66,7 +66,7 @@ struct GemmArgs {
 #ifdef FP6M_TIMELINE
 #define FP6M_MARK(p, i)                                                                            \
     do {                                                                                           \
-        if (threadIdx.x == 0 && (p).timeline)                                                      \
+        if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0 && (p).timeline) /* uniform branch */ \
             (p).timeline[(size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
     } while (0)
 #else
@@ -330,6 +330,17 @@ __device__ __forceinline__ uint32_t lds_addr(const void* ptr) { return (uint32_t
 // M0 + OFF + 16 * lane.  The immediate moves both sides, so loads whose LDS targets lie within 4 KiB of
 // each other share one M0 value (the global side is compensated in voff or sbase) and no vector address
 // arithmetic is left in the loop.  One wait state separates the M0 write from its first use.
+// The "s" operands below must live in SGPRs: values are made wave-uniform explicitly where they are
+// created (a no-op when the compiler already knows it).
+__device__ __forceinline__ uint32_t uniform32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename T>
+__device__ __forceinline__ const T* uniform_ptr(const T* ptr)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const T*>(((uint64_t)hi << 32) | lo);
+}
 __device__ __forceinline__ void set_m0(uint32_t lds_base)
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_base) : "memory");
@@ -786,7 +797,6 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
 
 struct WeightRegs {
     u4 q0, q1;
-    u2 t0, t1;
 };
 
 template <int N>
@@ -896,11 +906,12 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     static_assert(DEPTH >= 3, "needs two steps of look-ahead");
     static_assert(MB == 2 || MB == 4 || MB == 8, "the A register ring assumes MB | 8");
     constexpr bool kGroup = G128 && !FP6;
-    constexpr int kAOff = FP6 ? 3072 : 2048;
+    static_assert(!FP6 || DEPTH == 3, "the 2-bit plane alternates between two register sets");
+    constexpr int kAOff = 2048;
     constexpr int kSlot = kAOff + MB * 1024;
-    constexpr int kOps = (FP6 ? 3 : 2) + MB;              // direct-to-LDS loads per step
+    constexpr int kOps = 2 + MB + (FP6 ? 2 : 0);          // vector-memory loads per step
     constexpr int kUnroll = kGroup ? 4 : 2;
-    constexpr int kW = FP6 ? 4 : 2;                       // LDS reads of one step's weight words
+    constexpr int kW = 2;                                 // LDS reads of one step's weight words
     static_assert(kOps * (DEPTH - 2) <= 63, "vmcnt is a 6-bit counter");
     const int lane = threadIdx.x & 63;
     const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
@@ -914,17 +925,19 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
 
     // ---- fetch side: uniform 64-bit bases on the scalar unit, per-lane 32-bit offsets that never change.
     // The offsets carry the compensation for the immediates (see dma16_m0): the second k-block of the
-    // words sits 1 KiB further in LDS and one row further in memory; the 2-bit plane and the A blocks
-    // get their compensation on the scalar base, so that the lane offsets stay non-negative.
+    // words sits 1 KiB further in LDS and one row further in memory; the A blocks get theirs on the
+    // scalar base, so that the lane offsets stay non-negative.  The FP6 2-bit plane (8 bytes per lane and
+    // k-block, already in owner order in memory) skips LDS: it is loaded into registers two steps ahead,
+    // alternating between two register sets, which keeps an FP6 slot as small as an INT4 one.
     const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
     const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
     const uint32_t v4b = v4 + (uint32_t)row4 - 1024;
-    const unsigned char* base4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
-                                 (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4;
-    const int lg = lane & 31;
-    const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
-    const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
-                                 (size_t)(2 * step_begin) * row2 - 2048;
+    const unsigned char* base4 = uniform_ptr(reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                                             (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4);
+    const uint32_t v2 = (uint32_t)(32 * sigma + 4 * l + i) * 8, v2b = v2 + (uint32_t)row2;
+    const unsigned char* base2 = uniform_ptr(reinterpret_cast<const unsigned char*>(p.b_fp6_2) +
+                                             (size_t)ti.tcol * 512 + (size_t)(2 * step_begin) * row2);
+    u2 tq[2][2];                                          // [register set][k-block]
     const int a_m = lane >> 2;
     const int tile_row0 = ti.mtile * 16 * MB;
     uint32_t va[MB];
@@ -935,27 +948,31 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
         va[mb] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3)) + 4096 -
                  (kAOff + 1024 * mb) % 4096;
     }
-    const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
-                                  (size_t)step_begin * 64 - 4096;
-    const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
+    const unsigned char* base_a = uniform_ptr(reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
+                                              (size_t)step_begin * 64 - 4096);
+    const unsigned char* base_gs =
+        uniform_ptr(reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN));
     const uint32_t vgs = 4 * lane;
     constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;
     unsigned char* gs_ring = ring + DEPTH * kSlot;
-    const uint32_t ring_lds = lds_addr(ring);
-    const uint32_t gs_lds = lds_addr(gs_ring);
+    const uint32_t ring_lds = uniform32(lds_addr(ring));
+    const uint32_t gs_lds = uniform32(lds_addr(gs_ring));
 
     int issued = step_begin;
     const int last = step_end - 1;
-    auto issue = [&](int slot) {
+    auto issue = [&](int slot, int set) {
         const uint32_t dst = ring_lds + slot * kSlot;
         set_m0(dst);
         dma16_m0<0, true>(base4, v4);
         dma16_m0<1024, true>(base4, v4b);
-        if (FP6) dma16_m0<2048, true>(base2, v2);
         dma_a_blocks<MB, kAOff>(dst, base_a, va);
+        if (FP6) {
+            asm volatile("global_load_dwordx2 %0, %2, %4 nt\n\tglobal_load_dwordx2 %1, %3, %4 nt"
+                         : "=&v"(tq[set][0]), "=&v"(tq[set][1]) : "v"(v2), "v"(v2b), "s"(base2) : "memory");
+        }
         if (kGroup && (issued & 3) == 0) {
             set_m0(gs_lds + ((issued >> 2) & kScaleMask) * 256);
-            dma4_m0(base_gs + (size_t)(issued >> 2) * p.n4 * 2, vgs);
+            dma4_m0(base_gs + (size_t)(issued >> 2) * (size_t)uniform32(p.n4) * 2, vgs);
         }
         if (issued < last) {
             issued++;
@@ -968,8 +985,6 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     // ---- read side
     const int owner = 32 * sigma + 4 * l + i;
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
-    const int gr2 = owner >> 1;
-    const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
     uint32_t rda[4];
 #pragma unroll
     for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * c + (d ^ ((c >> 2) & 3))) * 16 + 4 * i;
@@ -981,15 +996,8 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     WeightRegs w;
     auto fetch_w = [&](int slot) {
         const uint32_t so = slot * kSlot;
-        if (FP6) {
-            asm volatile(
-                "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
-                "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
-                : "=&v"(w.q0), "=&v"(w.q1), "=&v"(w.t0), "=&v"(w.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
-        } else {
-            asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
-                         : "=&v"(w.q0), "=&v"(w.q1) : "v"(rd4 + so) : "memory");
-        }
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
+                     : "=&v"(w.q0), "=&v"(w.q1) : "v"(rd4 + so) : "memory");
     };
     auto fetch_scales = [&](int group) {
         const uint32_t ga = rdgs + (group & kScaleMask) * 256;
@@ -1012,16 +1020,16 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     // word is tied to this point of the program first, the results after, so the instructions stay
     // between the two MFMAs the chunk was placed between.
     h2 part[2];
-    auto chunk = [&](int ck, h8 (&frag)[8]) {
+    auto chunk = [&](int ck, int set, h8 (&frag)[8]) {
         const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
         uint32_t q4 = word ? w.q1[j] : w.q0[j];
         uint32_t q2 = 0;
         asm volatile("" : "+v"(q4));
         if (word) w.q1[j] = q4; else w.q0[j] = q4;
         if (FP6) {
-            uint32_t t = word ? w.t1[j >> 1] : w.t0[j >> 1];
+            uint32_t t = tq[set][word][j >> 1];
             asm volatile("" : "+v"(t));
-            if (word) w.t1[j >> 1] = t; else w.t0[j >> 1] = t;
+            tq[set][word][j >> 1] = t;
             q2 = t << (4 * (j & 1));
         }
         h2 r0, r1;
@@ -1046,9 +1054,9 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     };
 
     int slot_in = 0;
-#pragma unroll 1
+#pragma unroll
     for (int d = 0; d < DEPTH - 1; d++) {
-        issue(slot_in);
+        issue(slot_in, d & 1);
         slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
     }
     h8 frag[2][8];
@@ -1061,13 +1069,13 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
     if (kGroup) settle_scales();
 #pragma unroll
-    for (int ck = 0; ck < 16; ck++) chunk(ck, frag[0]);
+    for (int ck = 0; ck < 16; ck++) chunk(ck, 0, frag[0]);
     int slot_rd = 1;
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            issue(slot_in);
+            issue(slot_in, u & 1);                                    // step s+u+2 (FP6: DEPTH is 3)
             slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
 #pragma unroll
             for (int d = 0; d < 4; d++) cx.addr_cur[d] = cx.addr_next[d];
@@ -1090,7 +1098,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
                 if constexpr (mslot >= 8) {
                     constexpr int c0 = (mslot - 8) * 16 / avail, c1 = (mslot - 7) * 16 / avail;
 #pragma unroll
-                    for (int ck = c0; ck < c1; ck++) chunk(ck, nxt);
+                    for (int ck = c0; ck < c1; ck++) chunk(ck, (u + 1) & 1, nxt);
                 }
             };
             constexpr int kExtraMax = kW + (kGroup ? 8 : 0);
@@ -1101,7 +1109,18 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
         }
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");                   // MFMA results -> VALU reads
+    // MFMA results -> VALU reads: the wait states, then every accumulator is passed through an (empty)
+    // asm so that no read of it can be scheduled above them.
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            if constexpr (AGPR)
+                asm volatile("" : "+a"(acc[mb][t]));
+            else
+                asm volatile("" : "+v"(acc[mb][t]));
+        }
     if (FP6) {
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
@@ -1172,6 +1191,7 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     }
     if (ks == 1) return;
 
+    FP6M_MARK(p, 3);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
@@ -1181,6 +1201,7 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     }
     __syncthreads();
     if (!*flag) return;
+    FP6M_MARK(p, 5);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll 1
     for (int mb = 0; mb < MB; mb++) {
@@ -1222,15 +1243,16 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
 
 constexpr int mb_wave_lds(int mb, int d4, int d6)
 {
-    return max3(d4 * (2048 + mb * 1024) + scale_slab_bytes(d4), d6 * (3072 + mb * 1024), 16 * kRedStride * 4);
+    return max3(d4 * (2048 + mb * 1024) + scale_slab_bytes(d4), d6 * (2048 + mb * 1024), 16 * kRedStride * 4);
 }
 
 template <bool G128, int MB, int D4, int D6>
-__global__ __launch_bounds__(kThreads, MB >= 4 ? 1 : 2) void gemm_mb_kernel(const GemmArgs p)
+__global__ __launch_bounds__(kThreads, MB >= 8 ? 1 : 2) void gemm_mb_kernel(const GemmArgs p)
 {
     constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
     __shared__ __attribute__((aligned(16))) unsigned char smem[kWaves * kWaveLds + 16];
 
+    FP6M_MARK(p, 0);
     const TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int step_begin, step_end;
@@ -1244,12 +1266,14 @@ __global__ __launch_bounds__(kThreads, MB >= 4 ? 1 : 2) void gemm_mb_kernel(cons
     unsigned char* ring = smem + wave * kWaveLds;
     if (step_begin < step_end) {
         if (ti.fp6)
-            stream_tile_mb<true, G128, D6, MB, (MB >= 4)>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile_mb<true, G128, D6, MB, (MB >= 8)>(p, ti, ring, step_begin, step_end, acc);
         else
-            stream_tile_mb<false, G128, D4, MB, (MB >= 4)>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile_mb<false, G128, D4, MB, (MB >= 8)>(p, ti, ring, step_begin, step_end, acc);
     }
+    FP6M_MARK(p, 2);
     wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, ti.fp6 || !G128, smem, kWaveLds,
                      reinterpret_cast<int*>(smem + kWaves * kWaveLds));
+    FP6M_MARK(p, 7);
 }
 
 // ------------------------------------------------------------------------------------------------ m > 16: register-staged kernel
@@ -1563,7 +1587,9 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     if (const char* e = getenv("FP6M_TIMELINE_PTR")) a.timeline = reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0));
 #endif
 
-    int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : (prob_m <= 64 ? 4 : 8));
+    // Row blocks per workgroup pass, by measurement on 8192 x 8192: 64 rows (two workgroups per CU) up to
+    // m = 256, 128 rows (one wave per SIMD, half the re-reads of the words) beyond.
+    int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : (prob_m <= 256 ? 4 : 8));
     if (const char* e = getenv("FP6M_MB")) {   // tuning/testing override
         const int v = atoi(e);
         if (prob_m > 16 && (v == 2 || v == 4 || v == 8)) mb = v;
