@@ -224,8 +224,6 @@ def sweep(args):
         copies = max(2, min(24, int(640e6 // nbytes) + 1))           # rotate over > 512 MB of weights
         probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
         w16 = [(torch.randn((k, n), generator=gen) * 0.02).half().cuda() for _ in range(max(2, min(copies, int(640e6 // (2 * k * n)) + 1)))]
-        iters = 100
-
         def f(i):
             probs[i % copies].run(fp6_marlin.mul)
 
@@ -235,9 +233,14 @@ def sweep(args):
         for i in range(10):
             f(i)
             f16(i)
-        _, ev = time_region(torch, f, iters)
-        _, ev16 = time_region(torch, f16, iters)
-        t, t16 = ev / iters, ev16 / iters
+        torch.cuda.synchronize()
+        # one graph = one pass over all the weight copies; replayed until about 100 GEMMs have run
+        iters, iters16 = copies * max(1, 100 // copies), len(w16) * max(1, 100 // len(w16))
+        fn, calls = graphed(torch, f, copies, iters)
+        _, ev = time_region(torch, fn, calls)
+        fn16, calls16 = graphed(torch, f16, len(w16), iters16)
+        _, ev16 = time_region(torch, fn16, calls16)
+        t, t16 = ev / iters, ev16 / iters16
         row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "us": round(t * 1e6, 2),
                "weight_GBs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
                "TFLOPs": round(2 * m * k * n / t / 1e12, 2), "mfma_frac": round(2 * m * k * n / t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),

@@ -36,8 +36,6 @@ constexpr int kThreads = 256;        // four wavefronts
 constexpr int kWaves = 4;
 constexpr int kTileN = 128;          // columns per tile
 constexpr int kRedStride = kTileN + 4;                       // floats per row of the reduction slab
-constexpr int kRedBytes = kWaves * 16 * kRedStride * 4;      // one 16-row block from every wave
-constexpr int kSlabBytes = 3072;                             // per wave: 2 x 1 KiB (4-bit) + 2 x 512 B (2-bit)
 constexpr size_t kScratchBytes = size_t(64) << 20;           // per-device partial-sum scratch
 
 struct GemmArgs {
@@ -77,54 +75,12 @@ struct GemmArgs {
 
 __device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
 
-// Eight INT4 weights of one packed word -> (e0,e1) (e2,e3) (e4,e5) (e6,e7), value = nibble - 8.
-// 0x6400 | u is the half 1024 + u;  0x6400 | (u << 4) is 1024 + 16 u.
-__device__ __forceinline__ void dequant_int4(uint32_t q, h2 (&r)[4])
-{
-    const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
-    const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
-    const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-    r[0] = as_h2((q & 0x000f000fu) | 0x64006400u) - bias_lo;
-    r[1] = __builtin_elementwise_fma(as_h2((q & 0x00f000f0u) | 0x64006400u), mul_hi, bias_hi);
-    const uint32_t q8 = q >> 8;
-    r[2] = as_h2((q8 & 0x000f000fu) | 0x64006400u) - bias_lo;
-    r[3] = __builtin_elementwise_fma(as_h2((q8 & 0x00f000f0u) | 0x64006400u), mul_hi, bias_hi);
-}
-
-// Eight FP6 weights from the tile's 2-bit word (already shifted so the tile's fields are the top two
-// bits of every byte) and its 4-bit word.  A byte `s eee mm 00` moved to s 00eee mm 0000 0000 is the
-// half value * 2^-12 (sub-normal codes become half sub-normals); the multiply by 4096 is exact.
-__device__ __forceinline__ void dequant_fp6(uint32_t q2, uint32_t q4, h2 (&r)[4])
-{
-    const h2 unbias = {(_Float16)4096.0f, (_Float16)4096.0f};
-#pragma unroll
-    for (int half = 0; half < 2; half++) {
-        const uint32_t p = (q2 & 0xc0c0c0c0u) | ((q4 & 0xf0f0f0f0u) >> 2);  // bytes, MSB first: e1 e3 e0 e2 (then e5 e7 e4 e6)
-        const uint32_t a = (p & 0x80008000u) | ((p & 0x7c007c00u) >> 2);
-        const uint32_t p8 = p << 8;
-        const uint32_t b = (p8 & 0x80008000u) | ((p8 & 0x7c007c00u) >> 2);
-        r[2 * half + 0] = as_h2(a) * unbias;
-        r[2 * half + 1] = as_h2(b) * unbias;
-        q2 <<= 2;
-        q4 <<= 4;
-    }
-}
-
 __device__ __forceinline__ h8 join(h2 a, h2 b, h2 c, h2 d)
 {
     h8 v;
     v[0] = a[0]; v[1] = a[1]; v[2] = b[0]; v[3] = b[1];
     v[4] = c[0]; v[5] = c[1]; v[6] = d[0]; v[7] = d[1];
     return v;
-}
-
-// Orders this wave's LDS writes before its LDS reads (and the reverse) for the compiler.  The LDS
-// unit executes one wave's instructions in order, so no hardware wait is needed.
-__device__ __forceinline__ void wave_lds_fence()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Workgroup b of a 1-D grid runs on XCD b % 8.  Renumber so that every XCD sees a contiguous range of
@@ -170,131 +126,6 @@ __device__ __forceinline__ void wave_k_range(const GemmArgs& p, int part, int wa
     const int wv = part * kWaves + wave;
     begin = (int)((long long)units * wv / nwaves) * unit_steps;
     end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
-}
-
-// Epilogue shared by both kernels: sum the four waves of the workgroup through LDS, then either write
-// C (scaled, fp16) or publish an fp32 partial tile and let the last-arriving partner finish.
-// MFMA result layout: lane (m = lane & 15, q = lane >> 4) holds column slots 4q .. 4q+3 of each of the
-// eight 16-column accumulators (t = 2*j + half): column = 64*(q >> 1) + 16*j + 8*half + 4*(q & 1) + r.
-template <int MB>
-__device__ __forceinline__ void finish_tile(const GemmArgs& p, const TileInfo& ti, f4 (&acc)[MB][8],
-                                            bool per_column_scale, unsigned char* smem, int* s_is_last)
-{
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int c = lane & 15, q = lane >> 4;
-    float* red = reinterpret_cast<float*>(smem);
-    const int out_m = threadIdx.x >> 4;          // row inside the 16-row block
-    const int out_n = (threadIdx.x & 15) * 8;    // first of eight consecutive columns
-    const size_t tile_floats = (size_t)MB * 16 * kTileN;
-    float* my_partial = p.scratch + ((size_t)(ti.mtile * p.tiles + ti.tile) * p.ksplit + ti.part) * tile_floats;
-
-    float sc[8];
-    if (per_column_scale) {
-        const uint16_t* sp = (ti.fp6 ? p.s_fp6 : p.s_int4);
-        const int nr = ti.tcol * kTileN + out_n;    // column inside the region, multiple of 8
-        const int base = (nr & ~31) + 4 * ((nr >> 4) & 1) + 2 * ((nr >> 3) & 1);
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const uint16_t v = sp[base + 8 * (e >> 1) + (e & 1)];
-            sc[e] = (float)__builtin_bit_cast(_Float16, v);
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 8; e++) sc[e] = 1.0f;
-    }
-
-    auto store_row = [&](int row, const float (&v)[8]) {
-        h8 o;
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = (_Float16)(v[e] * sc[e]);
-        *reinterpret_cast<h8*>(p.C + (size_t)row * p.n + ti.col0 + out_n) = o;
-    };
-
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        __syncthreads();
-        float* mine = red + wave * 16 * kRedStride + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
-#pragma unroll
-        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[mb][t];
-        __syncthreads();
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; w++) {
-            const float* src = red + w * 16 * kRedStride + out_m * kRedStride + out_n;
-            const f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
-#pragma unroll
-            for (int e = 0; e < 4; e++) { v[e] += lo[e]; v[4 + e] += hi[e]; }
-        }
-        const int row = ti.mtile * 16 * MB + 16 * mb + out_m;
-        if (row < p.m) {
-            if (p.ksplit == 1) {
-                store_row(row, v);
-            } else {
-                // Agent-scope stores go straight to the level all XCDs share (no cache-wide write-back
-                // later).  Element e of thread t lives at [mb][e][t]: every store instruction of a wave
-                // writes 256 contiguous bytes.
-                float* dst = my_partial + (size_t)mb * 8 * kThreads + threadIdx.x;
-#pragma unroll
-                for (int e = 0; e < 8; e++)
-                    __hip_atomic_store(dst + e * kThreads, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-    }
-    FP6M_MARK(p, 3);
-    if (p.ksplit == 1) return;
-
-    // Publish the partial, then count arrivals; the last workgroup of the tile finishes it.  Partials
-    // are written and read with agent-scope accesses, so ordering needs only "my stores have completed"
-    // (workgroup-scope release = wait counters) before the counter is bumped: no L2 write-back or
-    // invalidate, which would stall every workgroup of the XCD.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    FP6M_MARK(p, 4);
-    int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
-    if (threadIdx.x == 0) {
-        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *s_is_last = (seen == p.ksplit - 1);
-    }
-    __syncthreads();
-    FP6M_MARK(p, 5);
-    if (!*s_is_last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    const float* first = p.scratch + (size_t)(ti.mtile * p.tiles + ti.tile) * p.ksplit * tile_floats;
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        const int row = ti.mtile * 16 * MB + 16 * mb + out_m;
-        if (row >= p.m) continue;
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = 0.f;
-        // Four partners' loads are in flight at a time; the sum runs in partner order (deterministic).
-        const float* src = first + (size_t)mb * 8 * kThreads + threadIdx.x;
-        int pp = 0;
-        for (; pp + 4 <= p.ksplit; pp += 4) {
-            float t[4][8];
-#pragma unroll
-            for (int u = 0; u < 4; u++)
-#pragma unroll
-                for (int e = 0; e < 8; e++)
-                    t[u][e] = __hip_atomic_load(src + (size_t)(pp + u) * tile_floats + e * kThreads, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-            for (int u = 0; u < 4; u++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) v[e] += t[u][e];
-        }
-        for (; pp < p.ksplit; pp++) {
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-                v[e] += __hip_atomic_load(src + (size_t)pp * tile_floats + e * kThreads, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-        }
-        store_row(row, v);
-    }
-    FP6M_MARK(p, 6);
-    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ------------------------------------------------------------------------------------------------ m <= 16: LDS-ring kernel
@@ -1276,163 +1107,6 @@ __global__ __launch_bounds__(kThreads, MB >= 8 ? 1 : 2) void gemm_mb_kernel(cons
     FP6M_MARK(p, 7);
 }
 
-// ------------------------------------------------------------------------------------------------ m > 16: register-staged kernel
-//
-// Up to 64 rows of A per workgroup pass (MB 16-row blocks): each dequantised weight fragment feeds MB
-// MFMAs.  Packed words are loaded to registers two steps ahead, turned through a wave-private LDS slab
-// and read back permuted; activations come straight from global memory in MFMA operand order.
-
-template <int MB, bool FP6>
-struct Stage {
-    u4 w4[2];            // 4-bit plane / INT4 words of k-blocks 2s, 2s+1 (this lane's linear 16 bytes)
-    u2 w2[2];            // FP6 2-bit plane (this lane's linear 8 bytes)
-    uint32_t a[MB][4];   // activations, already in MFMA operand order
-};
-
-template <int MB, bool FP6, bool G128>
-__device__ __forceinline__ void stream_tile_regs(const GemmArgs& p, const TileInfo& ti, unsigned char* slab,
-                                                 int step_begin, int step_end, f4 (&acc)[MB][8])
-{
-    constexpr bool kGroup = G128 && !FP6;
-    const int lane = threadIdx.x & 63;
-    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
-    const int owner = 32 * sigma + 4 * l + i;               // linear 16-byte granule of (group sigma, owner 4l+i)
-    const int wr4 = (lane ^ ((lane >> 4) & 3)) * 16;        // swizzled so both sides are bank-conflict free
-    const int rd4 = (owner ^ ((owner >> 4) & 3)) * 16;
-    const int wr2 = (lane ^ ((lane >> 5) << 1)) * 8;
-    const int rd2 = (owner ^ ((owner >> 5) << 1)) * 8;
-
-    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
-    const unsigned char* g4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
-                              (size_t)ti.tcol * 1024 + lane * 16;
-    const unsigned char* g2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 + lane * 8;
-    const uint16_t* a_row[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        int row = ti.mtile * 16 * MB + 16 * mb + c;
-        row = row < p.m ? row : p.m - 1;
-        a_row[mb] = p.A + (size_t)row * p.k + 2 * i;
-    }
-
-    auto load = [&](Stage<MB, FP6>& st, int s) {
-        const unsigned char* src4 = g4 + (size_t)(2 * s) * row4;
-        st.w4[0] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4));
-        st.w4[1] = __builtin_nontemporal_load(reinterpret_cast<const u4*>(src4 + row4));
-        if (FP6) {
-            const unsigned char* src2 = g2 + (size_t)(2 * s) * row2;
-            st.w2[0] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2));
-            st.w2[1] = __builtin_nontemporal_load(reinterpret_cast<const u2*>(src2 + row2));
-        }
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-                st.a[mb][d] = *reinterpret_cast<const uint32_t*>(a_row[mb] + 32 * s + 8 * d);
-    };
-
-    h2 gscale[8];  // group scale of column (j, half), duplicated into both halves
-    auto load_group_scales = [&](int s) {
-        const uint16_t* srow = p.s_int4 + (size_t)(s >> 2) * p.n4 + ti.tcol * kTileN + 64 * sigma + l;
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            const uint16_t v = srow[16 * (t >> 1) + 8 * (t & 1)];
-            gscale[t] = as_h2((uint32_t)v | ((uint32_t)v << 16));
-        }
-    };
-
-    auto consume = [&](Stage<MB, FP6>& st, int s) {
-        wave_lds_fence();
-        *reinterpret_cast<u4*>(slab + wr4) = st.w4[0];
-        *reinterpret_cast<u4*>(slab + 1024 + wr4) = st.w4[1];
-        if (FP6) {
-            *reinterpret_cast<u2*>(slab + 2048 + wr2) = st.w2[0];
-            *reinterpret_cast<u2*>(slab + 2560 + wr2) = st.w2[1];
-        }
-        wave_lds_fence();
-        const u4 q0 = *reinterpret_cast<const u4*>(slab + rd4);
-        const u4 q1 = *reinterpret_cast<const u4*>(slab + 1024 + rd4);
-        u2 t0 = {0, 0}, t1 = {0, 0};
-        if (FP6) {
-            t0 = *reinterpret_cast<const u2*>(slab + 2048 + rd2);
-            t1 = *reinterpret_cast<const u2*>(slab + 2560 + rd2);
-        }
-        if (kGroup && (s & 3) == 0) load_group_scales(s);
-
-        h8 av[MB];
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-            u4 raw = {st.a[mb][0], st.a[mb][1], st.a[mb][2], st.a[mb][3]};
-            av[mb] = __builtin_bit_cast(h8, raw);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            h2 r0[4], r1[4];
-            if (FP6) {
-                dequant_fp6(t0[j >> 1] << (4 * (j & 1)), q0[j], r0);
-                dequant_fp6(t1[j >> 1] << (4 * (j & 1)), q1[j], r1);
-            } else {
-                dequant_int4(q0[j], r0);
-                dequant_int4(q1[j], r1);
-                if (kGroup) {
-#pragma unroll
-                    for (int x = 0; x < 4; x++) {
-                        r0[x] = r0[x] * gscale[2 * j + (x >> 1)];
-                        r1[x] = r1[x] * gscale[2 * j + (x >> 1)];
-                    }
-                }
-            }
-            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
-            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                acc[mb][2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av[mb], acc[mb][2 * j + 0], 0, 0, 0);
-                acc[mb][2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av[mb], acc[mb][2 * j + 1], 0, 0, 0);
-            }
-        }
-    };
-
-    // Two steps of loads stay in flight in registers.  The step count is even, and the prefetch index
-    // is clamped instead of guarded, so the loop body is branch-free and the compiler's wait counts
-    // stay exact.
-    const int last = step_end - 1;
-    Stage<MB, FP6> st0, st1;
-    load(st0, step_begin);
-    load(st1, step_begin + 1);
-#pragma unroll 1
-    for (int s = step_begin; s < step_end; s += 2) {
-        consume(st0, s);
-        load(st0, s + 2 < last ? s + 2 : last);
-        consume(st1, s + 1);
-        load(st1, s + 3 < last ? s + 3 : last);
-    }
-}
-
-template <int MB, bool G128>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(const GemmArgs p)
-{
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kRedBytes];
-    __shared__ int s_is_last;
-
-    const TileInfo ti = locate_tile(p);
-    const int wave = threadIdx.x >> 6;
-    int step_begin, step_end;
-    wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
-
-    f4 acc[MB][8];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
-    unsigned char* slab = smem + wave * kSlabBytes;
-    if (step_begin < step_end) {
-        if (ti.fp6)
-            stream_tile_regs<MB, true, G128>(p, ti, slab, step_begin, step_end, acc);
-        else
-            stream_tile_regs<MB, false, G128>(p, ti, slab, step_begin, step_end, acc);
-    }
-    finish_tile<MB>(p, ti, acc, ti.fp6 || !G128, smem, &s_is_last);
-}
-
 // ------------------------------------------------------------------------------------------------ host
 
 thread_local int g_last_hip_error = 0;
@@ -1508,15 +1182,6 @@ inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, d
 template <int MB, int D4, int D6>
 void launch_mb(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
-    if (getenv("FP6M_OLD_MB")) {   // previous register-staged kernel, kept for comparison while tuning
-        if constexpr (MB <= 4) {
-            if (g128)
-                hipLaunchKernelGGL((gemm_kernel<MB, true>), grid, dim3(kThreads), 0, stream, a);
-            else
-                hipLaunchKernelGGL((gemm_kernel<MB, false>), grid, dim3(kThreads), 0, stream, a);
-            return;
-        }
-    }
     if (g128)
         hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6>), grid, dim3(kThreads), 0, stream, a);
     else

@@ -47,11 +47,15 @@ def run(oracle, m, n, k, thread_k=-1, thread_n=-1, qc=-1, gs=-1, seed=0, max_par
     try:
         fp6_marlin.mul(A.to(dev()), B, C, s, ws, qc, thread_k, thread_n, sms, max_par, gs)
         torch.cuda.synchronize()
+        C2 = torch.full_like(C, float("nan"))                          # same call again: results are reproducible
+        fp6_marlin.mul(A.to(dev()), B, C2, s, ws, qc, thread_k, thread_n, sms, max_par, gs)
+        torch.cuda.synchronize()
     finally:
         os.environ.pop("FP6M_KSPLIT", None)
     assert int(ws.abs().sum().item()) == 0, "workspace must be left zeroed"
     c = C.cpu().numpy()
     assert np.isfinite(c).all(), "C not fully written"
+    assert torch.equal(C, C2), "two identical calls differ"
     err = oracle.rel_err(c, oracle.matmul_ref(A.numpy(), ref))
     assert err <= TOL, f"rel err {err}"
     return c
