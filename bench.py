@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]          one JSON line (the driver's contract)
     python bench.py --sweep gpurun_out/sweep.json                per-shape table for all BASELINE configs
+    python bench.py --shape 128,8192,8192                        one shape (m,k,n[,quant_cols,group_size])
 
 Workload of the JSON line: decode (M=1) through Llama-2-7B layer shapes (K x N) 4096x12288, 4096x4096,
 4096x22016, 11008x4096; INT4 with group-128 scales plus 256 FP6 columns.  A *step* is one layer: those four
@@ -204,6 +205,57 @@ def traffic_probe():
           [p.bytes for p in probs[0]], flush=True)
 
 
+def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100):
+    """One (m, k, n) GEMM against fp16 torch.matmul (hipBLASLt), both replayed from HIP graphs that walk
+    over > 512 MB of distinct weights."""
+    nbytes = weight_bytes(k, n, qc, gs)
+    copies = max(2, min(24, int(640e6 // nbytes) + 1))
+    probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
+    w16 = [(torch.randn((k, n), generator=gen) * 0.02).half().cuda()
+           for _ in range(max(2, min(copies, int(640e6 // (2 * k * n)) + 1)))]
+
+    def f(i):
+        probs[i % copies].run(fp6_marlin.mul)
+
+    def f16(i):
+        torch.matmul(probs[0].A, w16[i % len(w16)], out=probs[0].C)
+
+    for i in range(10):
+        f(i)
+        f16(i)
+    torch.cuda.synchronize()
+    iters, iters16 = copies * max(1, calls_target // copies), len(w16) * max(1, calls_target // len(w16))
+    fn, calls = graphed(torch, f, copies, iters)
+    _, ev = time_region(torch, fn, calls)
+    fn16, calls16 = graphed(torch, f16, len(w16), iters16)
+    _, ev16 = time_region(torch, fn16, calls16)
+    t, t16 = ev / iters, ev16 / iters16
+    row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "us": round(t * 1e6, 2),
+           "weight_GBs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
+           "TFLOPs": round(2 * m * k * n / t / 1e12, 2), "mfma_frac": round(2 * m * k * n / t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+           "fp16_us": round(t16 * 1e6, 2), "speedup_vs_fp16": round(t16 / t, 2)}
+    del probs, w16
+    torch.cuda.empty_cache()
+    return row
+
+
+def one_shape(args):
+    """`--shape m,k,n[,quant_cols,group_size]`: one JSON row for one shape (used for profiles of the m > 16 kernel)."""
+    import torch
+    import fp6_marlin
+    v = [int(x) for x in args.shape.split(",")]
+    m, k, n = v[:3]
+    qc, gs = (v[3] if len(v) > 3 else 256), (v[4] if len(v) > 4 else 128)
+    fp6_marlin.init(0)
+    row = measure_shape(torch, fp6_marlin, torch.Generator().manual_seed(0), "shape", m, k, n, qc, gs)
+    bound = "mfma" if m >= 128 else "hbm"
+    row["roofline"] = ({"bound": "mfma", "achieved": row["TFLOPs"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": row["mfma_frac"]} if bound == "mfma" else
+                       {"bound": "hbm", "achieved": row["weight_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": row["hbm_frac"]})
+    print(json.dumps(row), flush=True)
+
+
 def sweep(args):
     """Per-shape numbers for every BASELINE configuration; written as JSON rows."""
     import torch
@@ -220,35 +272,9 @@ def sweep(args):
     cases += [("cfg4-13B", 33, 5120, 13824, 512, -1), ("cfg4-13B", 33, 13824, 5120, 512, -1)]
     cases += [("all-int4-g-1", 16, 8192, 8192, 0, -1), ("all-int4-g128", 16, 8192, 8192, 0, 128)]
     for tag, m, k, n, qc, gs in cases:
-        nbytes = weight_bytes(k, n, qc, gs)
-        copies = max(2, min(24, int(640e6 // nbytes) + 1))           # rotate over > 512 MB of weights
-        probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
-        w16 = [(torch.randn((k, n), generator=gen) * 0.02).half().cuda() for _ in range(max(2, min(copies, int(640e6 // (2 * k * n)) + 1)))]
-        def f(i):
-            probs[i % copies].run(fp6_marlin.mul)
-
-        def f16(i):
-            torch.matmul(probs[0].A, w16[i % len(w16)], out=probs[0].C)
-
-        for i in range(10):
-            f(i)
-            f16(i)
-        torch.cuda.synchronize()
-        # one graph = one pass over all the weight copies; replayed until about 100 GEMMs have run
-        iters, iters16 = copies * max(1, 100 // copies), len(w16) * max(1, 100 // len(w16))
-        fn, calls = graphed(torch, f, copies, iters)
-        _, ev = time_region(torch, fn, calls)
-        fn16, calls16 = graphed(torch, f16, len(w16), iters16)
-        _, ev16 = time_region(torch, fn16, calls16)
-        t, t16 = ev / iters, ev16 / iters16
-        row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "us": round(t * 1e6, 2),
-               "weight_GBs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
-               "TFLOPs": round(2 * m * k * n / t / 1e12, 2), "mfma_frac": round(2 * m * k * n / t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-               "fp16_us": round(t16 * 1e6, 2), "speedup_vs_fp16": round(t16 / t, 2)}
+        row = measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs)
         rows.append(row)
         print(json.dumps(row), flush=True)
-        del probs, w16
-        torch.cuda.empty_cache()
     os.makedirs(os.path.dirname(os.path.abspath(args.sweep)), exist_ok=True)
     with open(args.sweep, "w") as fh:
         json.dump(rows, fh, indent=1)
@@ -260,6 +286,7 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
+    ap.add_argument("--shape", type=str, default=None, help="m,k,n[,quant_cols,group_size]: measure one shape")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 256 MiB device copy, then one layer of GEMMs")
@@ -271,6 +298,8 @@ def main():
         traffic_probe()
     elif args.sweep:
         sweep(args)
+    elif args.shape:
+        one_shape(args)
     else:
         headline(args)
 
