@@ -646,20 +646,16 @@ __device__ __forceinline__ void lds_read_a4(uint32_t (&a)[4], const uint32_t (&a
 }
 
 // acc += w (16 columns x 32 k) * a (16 rows x 32 k), in place.  Written as asm so that the accumulator
-// stays in one register quad for the whole loop (AGPR when the kernel runs one wave per SIMD) and the
-// MFMAs keep their place between the LDS reads.  The hazards the compiler would pad for are handled
+// stays in one VGPR quad for the whole loop (the builtin let the allocator rotate the accumulators
+// through copies) and the MFMAs keep their place between the LDS reads.  The hazards the compiler would pad for are handled
 // here: an MFMA must not read a VGPR in the two wait states after a VALU wrote it (register copies the
 // allocator places in front of the asm count), hence the s_nop; the loop never reads an accumulator
 // except as the addend of the same MFMA a full step later; the wait states before the first VALU read
 // of a result follow the loop.
-template <bool AGPR, bool FIRST>
+template <bool FIRST>
 __device__ __forceinline__ void mfma_acc(f4& acc, const h8& w, const h8& a)
 {
-    if constexpr (AGPR && FIRST)
-        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
-    else if constexpr (AGPR)
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
-    else if constexpr (FIRST)
+    if constexpr (FIRST)
         asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
     else
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
@@ -698,7 +694,7 @@ struct MbCtx {
 // immediates follow from the fixed issue order: [A(0), A(1)] from the previous step, the next step's
 // weight words (kExtra reads), then A(2), A(3), ...  After every MFMA `hook(block, t)` runs: the caller
 // uses it to dequantise the next step's fragments a few VALU instructions at a time.
-template <bool AGPR, int MB, int kExtra, int BLK = 0>
+template <int MB, int kExtra, int BLK = 0>
 struct MbBlocks {
     template <int phase, typename Hook>
     static __device__ __forceinline__ void run(MbCtx& cx, const h8 (&frag)[8], f4 (&acc)[MB][8], Hook&& hook)
@@ -717,25 +713,25 @@ struct MbBlocks {
             uint32_t (&src)[4] = cx.abuf[(phase + BLK) & 3];
             asm volatile("" : "+v"(src[0]), "+v"(src[1]), "+v"(src[2]), "+v"(src[3]));
             const h8 av = __builtin_bit_cast(h8, u4{src[0], src[1], src[2], src[3]});
-            mfma_acc<AGPR, true>(acc[BLK][0], frag[0], av); hook(Int<BLK>{}, Int<0>{});
-            mfma_acc<AGPR, false>(acc[BLK][1], frag[1], av); hook(Int<BLK>{}, Int<1>{});
-            mfma_acc<AGPR, false>(acc[BLK][2], frag[2], av); hook(Int<BLK>{}, Int<2>{});
-            mfma_acc<AGPR, false>(acc[BLK][3], frag[3], av); hook(Int<BLK>{}, Int<3>{});
-            mfma_acc<AGPR, false>(acc[BLK][4], frag[4], av); hook(Int<BLK>{}, Int<4>{});
-            mfma_acc<AGPR, false>(acc[BLK][5], frag[5], av); hook(Int<BLK>{}, Int<5>{});
-            mfma_acc<AGPR, false>(acc[BLK][6], frag[6], av); hook(Int<BLK>{}, Int<6>{});
-            mfma_acc<AGPR, false>(acc[BLK][7], frag[7], av); hook(Int<BLK>{}, Int<7>{});
-            MbBlocks<AGPR, MB, kExtra, BLK + 1>::template run<phase>(cx, frag, acc, hook);
+            mfma_acc<true>(acc[BLK][0], frag[0], av); hook(Int<BLK>{}, Int<0>{});
+            mfma_acc<false>(acc[BLK][1], frag[1], av); hook(Int<BLK>{}, Int<1>{});
+            mfma_acc<false>(acc[BLK][2], frag[2], av); hook(Int<BLK>{}, Int<2>{});
+            mfma_acc<false>(acc[BLK][3], frag[3], av); hook(Int<BLK>{}, Int<3>{});
+            mfma_acc<false>(acc[BLK][4], frag[4], av); hook(Int<BLK>{}, Int<4>{});
+            mfma_acc<false>(acc[BLK][5], frag[5], av); hook(Int<BLK>{}, Int<5>{});
+            mfma_acc<false>(acc[BLK][6], frag[6], av); hook(Int<BLK>{}, Int<6>{});
+            mfma_acc<false>(acc[BLK][7], frag[7], av); hook(Int<BLK>{}, Int<7>{});
+            MbBlocks<MB, kExtra, BLK + 1>::template run<phase>(cx, frag, acc, hook);
         }
     }
 };
 
-template <bool FP6, bool G128, int DEPTH, int MB, bool AGPR>
+template <bool FP6, bool G128, int DEPTH, int MB>
 __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                                int step_begin, int step_end, f4 (&acc)[MB][8])
 {
     static_assert(DEPTH >= 3, "needs two steps of look-ahead");
-    static_assert(MB == 2 || MB == 4 || MB == 8, "the A register ring assumes MB | 8");
+    static_assert(MB == 2 || MB == 4, "the A register ring assumes MB | 4; 128 accumulator VGPRs at most");
     constexpr bool kGroup = G128 && !FP6;
     static_assert(!FP6 || DEPTH == 3, "the 2-bit plane alternates between two register sets");
     constexpr int kAOff = 2048;
@@ -934,9 +930,9 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
             };
             constexpr int kExtraMax = kW + (kGroup ? 8 : 0);
             if ((u & 1) == 0)                                          // buffer of block 0: (u * MB) mod 4
-                MbBlocks<AGPR, MB, kExtraMax>::template run<0>(cx, cur, acc, hook);
+                MbBlocks<MB, kExtraMax>::template run<0>(cx, cur, acc, hook);
             else
-                MbBlocks<AGPR, MB, kExtraMax>::template run<(MB & 3)>(cx, cur, acc, hook);
+                MbBlocks<MB, kExtraMax>::template run<(MB & 3)>(cx, cur, acc, hook);
         }
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
@@ -947,10 +943,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-            if constexpr (AGPR)
-                asm volatile("" : "+a"(acc[mb][t]));
-            else
-                asm volatile("" : "+v"(acc[mb][t]));
+            asm volatile("" : "+v"(acc[mb][t]));
         }
     if (FP6) {
 #pragma unroll
@@ -1078,7 +1071,7 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 }
 
 template <bool G128, int MB, int D4, int D6>
-__global__ __launch_bounds__(kThreads, MB >= 8 ? 1 : 2) void gemm_mb_kernel(const GemmArgs p)
+__global__ __launch_bounds__(kThreads, 2) void gemm_mb_kernel(const GemmArgs p)
 {
     constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
     __shared__ __attribute__((aligned(16))) unsigned char smem[kWaves * kWaveLds + 16];
@@ -1097,9 +1090,9 @@ __global__ __launch_bounds__(kThreads, MB >= 8 ? 1 : 2) void gemm_mb_kernel(cons
     unsigned char* ring = smem + wave * kWaveLds;
     if (step_begin < step_end) {
         if (ti.fp6)
-            stream_tile_mb<true, G128, D6, MB, (MB >= 8)>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
         else
-            stream_tile_mb<false, G128, D4, MB, (MB >= 8)>(p, ti, ring, step_begin, step_end, acc);
+            stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
     }
     FP6M_MARK(p, 2);
     wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, ti.fp6 || !G128, smem, kWaveLds,
@@ -1252,12 +1245,13 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     if (const char* e = getenv("FP6M_TIMELINE_PTR")) a.timeline = reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0));
 #endif
 
-    // Row blocks per workgroup pass, by measurement on 8192 x 8192: 64 rows (two workgroups per CU) up to
-    // m = 256, 128 rows (one wave per SIMD, half the re-reads of the words) beyond.
-    int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : (prob_m <= 256 ? 4 : 8));
+    // Row blocks per workgroup pass: 32 rows up to m = 32, 64 rows (accumulators in 128 VGPRs, two
+    // workgroups per CU) beyond.  128-row blocks (accumulators in AGPRs, one wave per SIMD) measured 10-15 %
+    // faster for m >= 512 but left the register allocator no slack, and were dropped.
+    int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     if (const char* e = getenv("FP6M_MB")) {   // tuning/testing override
         const int v = atoi(e);
-        if (prob_m > 16 && (v == 2 || v == 4 || v == 8)) mb = v;
+        if (prob_m > 16 && (v == 2 || v == 4)) mb = v;
     }
     const int rows_per_tile = 16 * mb;
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
@@ -1328,8 +1322,7 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d grid=%ux%u\n", a.m, prob_n, prob_k, mb, mtiles,
                         a.ksplit, grid.x, grid.y);
             if (mb == 2) launch_mb<2, 4, 3>(a, g128, grid, st);
-            else if (mb == 4) launch_mb<4, 3, 3>(a, g128, grid, st);
-            else launch_mb<8, 3, 3>(a, g128, grid, st);
+            else launch_mb<4, 3, 3>(a, g128, grid, st);
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return hip_fail(e);

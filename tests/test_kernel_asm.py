@@ -1,0 +1,94 @@
+"""Static checks on the compiler's output for the hand-scheduled m > 16 kernel.
+
+Its MFMAs and direct-to-LDS loads are inline asm, so the compiler's hazard recogniser does not see them; the
+rules it would have enforced are checked here on the generated gfx950 assembly of the shipped source
+(`hipcc -S --cuda-device-only`, about a minute, no GPU):
+
+* no MFMA reads a VGPR/AGPR that a VALU instruction wrote fewer than two wait states earlier;
+* every direct-to-LDS load in scalar-base form got SGPRs for its base and every M0 write an SGPR source
+  (an "s" asm operand that the compiler could not prove uniform silently becomes a VGPR);
+* the MFMA loops of the m > 16 kernel move no accumulator (no v_accvgpr_* inside them) and spill nothing.
+"""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "fp6-marlin_amd", "csrc", "fp6m_gemm.hip")
+HIPCC = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")
+
+
+@pytest.fixture(scope="module")
+def asm(tmp_path_factory):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not available")
+    out = tmp_path_factory.mktemp("asm") / "fp6m_gemm.s"
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+                           "-packed-fp32-ops", f"-I{ROOT}/include", f"-I{ROOT}/fp6-marlin_amd/csrc", "-S",
+                           "--cuda-device-only", "-o", str(out), SRC], stderr=subprocess.DEVNULL)
+    return out.read_text()
+
+
+def kernels(asm):
+    for m in re.finditer(r"^(_ZN4fp6m\w+):", asm, re.M):
+        body = asm[m.start():asm.index(".Lfunc_end", m.start())]
+        ins = [l.strip() for l in body.split("\n") if l.startswith("\t") and l.strip() and not l.strip().startswith((".", ";"))]
+        yield m.group(1), ins
+
+
+def regs(tok):
+    tok = tok.strip().rstrip(",")
+    m = re.match(r"^([va])\[(\d+):(\d+)\]$", tok)
+    if m:
+        return {(m.group(1), r) for r in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.match(r"^([va])(\d+)$", tok)
+    return {(m.group(1), int(m.group(2)))} if m else set()
+
+
+def test_no_valu_write_right_before_mfma_read(asm):
+    checked = 0
+    for name, ins in kernels(asm):
+        for n, l in enumerate(ins):
+            if not l.startswith("v_mfma"):
+                continue
+            checked += 1
+            src = set().union(*[regs(o) for o in l.split(None, 1)[1].split(",")[1:4]])
+            waited, k = 0, n - 1
+            while k >= 0 and waited < 2:
+                p = ins[k]
+                if p.startswith("s_nop"):
+                    waited += int(p.split()[1]) + 1
+                else:
+                    if p.startswith("v_") and not p.startswith("v_mfma"):
+                        dst = regs(p.split(None, 1)[1].split(",")[0])
+                        assert not (dst & src), f"{name}: `{p}` feeds `{l}` after {waited} wait states"
+                    waited += 1
+                k -= 1
+    assert checked > 500
+
+
+def test_scalar_operands_of_asm_loads(asm):
+    assert not re.findall(r"global_load_lds_dwordx?4? v\d+, v", asm), "direct-to-LDS load with a vector base"
+    assert not re.findall(r"s_mov_b32 m0, v", asm), "M0 written from a VGPR"
+    assert not re.findall(r"global_load_dwordx2 v\[\d+:\d+\], v\d+, v", asm), "2-bit plane load with a vector base"
+    assert len(re.findall(r"global_load_lds_dwordx4 v\d+, s\[", asm)) > 20
+
+
+def test_mb_kernel_loops_keep_accumulators_in_place(asm):
+    seen = 0
+    for name, ins in kernels(asm):
+        if "gemm_mb_kernel" not in name:
+            continue
+        seen += 1
+        meta = asm[asm.index(".name:           " + name) - 400:asm.index(".name:           " + name) + 800]
+        first, last = None, None
+        for n, l in enumerate(ins):
+            if l.startswith("v_mfma"):
+                first = n if first is None else first
+                last = n
+        moved = [l for l in ins[first:last] if l.startswith("v_accvgpr")]
+        assert not moved, f"{name}: accumulator copies between MFMAs: {moved[:4]}"
+    assert seen == 4
+    assert not re.findall(r"\.vgpr_spill_count:\s+[1-9]", asm), "a kernel spills VGPRs"
