@@ -186,6 +186,49 @@ def test_baseline_config4_edge_shapes(oracle):
         assert int(ws.abs().sum().item()) == 0
 
 
+def test_baseline_full_sizes_against_unpacked_words(oracle):
+    """BASELINE configs 1-3 at their real sizes.  The oracle cannot pack 8192 x 57344 in seconds, so the packed
+    words are random bits (every FP6 code and INT4 nibble occurs) and the reference weight comes from the shipped
+    unpacker, which tests/test_cpu_routines.py pins bit for bit against the oracle's dequantised weight; the
+    reference product is an fp32 matmul of A with it.  Also: linearity in A (C(a1 + a2) = C(a1) + C(a2))."""
+    import fp6_marlin
+    cases = [(1, 4096, 22016), (1, 11008, 4096), (16, 8192, 57344), (1, 28672, 8192), (128, 8192, 8192), (1024, 8192, 8192)]
+    qc, gs = 256, 128
+    g = torch.Generator().manual_seed(11)
+    for m, k, n in cases:
+        print(f"case full m={m} k={k} n={n}", flush=True)
+        n4 = n - qc
+        words = k * n4 // 8 + k * qc * 3 // 16
+        B = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), generator=g, dtype=torch.int64).to(torch.int32)
+        s = (torch.rand((k // gs) * n4 + qc, generator=g) * 0.01 + 0.001).half()
+        w = fp6_marlin.unpack_to_fp16(B, s, k, n, qc, gs).to(dev())
+        Bd, sd = B.to(dev()), s.to(dev())
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+
+        def gemm(a):
+            C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+            fp6_marlin.mul(a, Bd, C, sd, ws, qc, -1, -1, -1, 16, gs)
+            torch.cuda.synchronize()
+            return C
+
+        a1 = torch.randn((m, k), generator=g).half().to(dev())
+        c1 = gemm(a1)
+        ref = a1.float() @ w.float()
+        err = ((c1.float() - ref).abs().mean() / ref.abs().mean()).item()
+        assert err <= TOL, (m, k, n, err)
+        assert int(ws.abs().sum().item()) == 0
+        # linearity: a2 is a small integer multiple pattern so that a1 + a2 is exact in fp16 for most entries
+        a2 = (torch.randint(-2, 3, (m, k), generator=g).half() * 0.5).to(dev())
+        a12 = (a1.float() + a2.float()).half()
+        exact = (a12.float() == a1.float() + a2.float())
+        a2 = torch.where(exact, a2, torch.zeros_like(a2))               # keep only entries whose sum is representable
+        a12 = (a1.float() + a2.float()).half()
+        lin = (gemm(a12).float() - (c1.float() + gemm(a2).float())).abs().mean() / ref.abs().mean()
+        assert lin.item() <= TOL, (m, k, n, lin.item())
+        del w, Bd, sd, ref
+        torch.cuda.empty_cache()
+
+
 def test_layer_forward(oracle):
     import fp6_marlin
     torch.manual_seed(1)
