@@ -182,6 +182,12 @@ def headline(args):
         "fp16_hipblaslt": {"ms_per_step": round(wall16 / args.steps * 1e3, 5),
                            "speedup": round(wall16 / wall, 3)},
     }
+    del model
+    torch.cuda.empty_cache()
+    # the other two regimes BASELINE's metric names, one shape each (same protocol as --sweep)
+    out["other_regimes"] = [measure_shape(torch, fp6_marlin, gen, tag, mm, k, n, qc, gs, calls_target=60)
+                            for tag, mm, k, n in (("70B M=16 (HBM-bound)", 16, 8192, 57344),
+                                                  ("M=128 (MFMA-bound)", 128, 8192, 8192))]
     print(json.dumps(out), flush=True)
 
 
