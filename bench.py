@@ -262,6 +262,35 @@ def one_shape(args):
     print(json.dumps(row), flush=True)
 
 
+def pack_bench(args):
+    """`--pack k,n[,quant_cols,group_size]`: on-GPU weight preparation (fp16 [k, n] -> B, s) against the host
+    packers on the box's cores.  Algorithmic bytes: the fp16 weight read once, the packed words and scales
+    written once (no check weight)."""
+    import torch
+    import fp6_marlin
+    v = [int(x) for x in args.pack.split(",")]
+    k, n = v[:2]
+    qc, gs = (v[2] if len(v) > 2 else 256), (v[3] if len(v) > 3 else 128)
+    w = (torch.randn((k, n), generator=torch.Generator().manual_seed(0)) * 0.02).half()
+    wd = w.cuda()
+    nbytes = 2 * k * n + weight_bytes(k, n, qc, gs)
+    for _ in range(2):
+        fp6_marlin.pack_mixed_weight_device(wd, qc, gs, True, want_ref=False)
+    torch.cuda.synchronize()
+    iters = 10
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fp6_marlin.pack_mixed_weight_device(wd, qc, gs, True, want_ref=False)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / iters
+    t0 = time.perf_counter()
+    fp6_marlin.pack_mixed_weight(w, qc, gs)
+    th = time.perf_counter() - t0
+    print(json.dumps({"pack": f"{k}x{n} qc={qc} gs={gs}", "gpu_ms": round(t * 1e3, 3), "gpu_GBs": round(nbytes / t / 1e9, 1),
+                      "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4), "host_ms": round(th * 1e3, 1),
+                      "host_threads": os.cpu_count(), "speedup": round(th / t, 1)}), flush=True)
+
+
 def sweep(args):
     """Per-shape numbers for every BASELINE configuration; written as JSON rows."""
     import torch
@@ -293,6 +322,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
     ap.add_argument("--shape", type=str, default=None, help="m,k,n[,quant_cols,group_size]: measure one shape")
+    ap.add_argument("--pack", type=str, default=None, help="k,n[,quant_cols,group_size]: time the on-GPU weight packer")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 256 MiB device copy, then one layer of GEMMs")
@@ -306,6 +336,8 @@ def main():
         sweep(args)
     elif args.shape:
         one_shape(args)
+    elif args.pack:
+        pack_bench(args)
     else:
         headline(args)
 

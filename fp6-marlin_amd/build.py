@@ -34,7 +34,7 @@ def run(cmd):
 def build_lib():
     hipcc = os.path.join(ROCM, "bin", "hipcc")
     out = os.path.join(PKG, "libfp6m.so")
-    srcs = [os.path.join(CSRC, f) for f in ("fp6m_cpu.cpp", "fp6m_gemm.hip")]
+    srcs = [os.path.join(CSRC, f) for f in ("fp6m_cpu.cpp", "fp6m_gemm.hip", "fp6m_pack.hip")]
     run([hipcc, *HIP_FLAGS, "-shared", "-pthread", "-o", out, *srcs])
     return out
 

@@ -37,6 +37,7 @@ constexpr int kWaves = 4;
 constexpr int kTileN = 128;          // columns per tile
 constexpr int kRedStride = kTileN + 4;                       // floats per row of the reduction slab
 constexpr size_t kScratchBytes = size_t(64) << 20;           // per-device partial-sum scratch
+constexpr size_t kPackTempBytes = size_t(1) << 20;           // + the packer's flag and per-column maxima
 
 struct GemmArgs {
     const uint16_t* A;
@@ -1129,7 +1130,7 @@ int ensure_scratch(int dev, DeviceScratch** out)
         if (e != hipSuccess) return hip_fail(e);
         if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) return hip_fail(e);
         void* mem = nullptr;
-        e = hipMalloc(&mem, kScratchBytes);
+        e = hipMalloc(&mem, kScratchBytes + kPackTempBytes);          // partial tiles, then the packer's scratch
         int cus = 0;
         if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (prev != dev) (void)hipSetDevice(prev);
@@ -1138,6 +1139,16 @@ int ensure_scratch(int dev, DeviceScratch** out)
         d.cus = cus > 0 ? cus : 256;
     }
     *out = &d;
+    return FP6M_OK;
+}
+
+// Scratch of the on-GPU packer (fp6m_pack.hip): kPackTempBytes behind the partial-sum tiles.
+int pack_temp(int dev, void** ptr)
+{
+    DeviceScratch* d = nullptr;
+    const int rc = ensure_scratch(dev, &d);
+    if (rc != FP6M_OK) return rc;
+    *ptr = reinterpret_cast<unsigned char*>(d->ptr) + kScratchBytes;
     return FP6M_OK;
 }
 

@@ -1,0 +1,270 @@
+// Weight preparation on the GPU: fp16 [k, n] -> the operands of fp6m_mul (B, s) and the dequantised
+// check weight, bit for bit what the host path produces (INT4: reference test.py:85-121; FP6:
+// test.py:13-58 + weight_quant.cpp:27-124 + weight_prepacking.cpp:123-177; scale order test.py:80-83;
+// wire format test.py:123-152).  HBM-bound byte work: one thread builds the packed words of one fragment
+// owner (32 weights), so every weight is read once and every output word written once.
+//
+// Arithmetic follows the host path operation by operation: values are binary16, every operation is done in
+// binary32 and rounded back to binary16 (what torch's CPU half kernels and the reference's __hmul do), with
+// IEEE division and round-to-nearest-even conversions.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fp6m.h"
+#include "fp6m_layout.h"
+
+namespace fp6m {
+
+int hip_fail(hipError_t e);            // fp6m_gemm.hip: records the HIP error, returns FP6M_ERR_HIP
+int pack_temp(int dev, void** ptr);    // fp6m_gemm.hip: 1 MiB of per-device scratch behind the partial-sum tiles
+constexpr size_t kPackTemp = size_t(1) << 20;
+
+namespace {
+
+__device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+
+// Position of the per-column scale of column c in the reference's permuted order.
+__device__ __forceinline__ size_t scale_pos(size_t c) { return (c & ~size_t(31)) + scale_slot((int)(c & 31)); }
+
+// ---- INT4 region: columns [0, n4) of w
+
+// One thread per (group, column): s = max|w| * 2/15 (test.py:88-89).
+__global__ void int4_scales_kernel(const uint16_t* w, int k, int n, int n4, int g, uint16_t* s, int per_column)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, gi = blockIdx.y;
+    if (c >= n4) return;
+    uint16_t amax = 0;
+    for (int r = gi * g; r < (gi + 1) * g; r++) {
+        const uint16_t a = w[(size_t)r * n + c] & 0x7fffu;
+        amax = a > amax ? a : amax;
+    }
+    const uint16_t sh = f2h(h2f(amax) * (float)(2.0 / 15.0));
+    s[per_column ? scale_pos(c) : (size_t)gi * n4 + c] = sh;
+}
+
+// q = clamp(round(w / s) + 8, 0, 15) and the check weight (q - 8) * s (test.py:90-98).  The harness packs the
+// re-quantised check weight (test.py:99-101); that returns the same q (|q - 8| <= 8 and the product is
+// rounded by at most 2^-11 relative, far from the next rounding boundary), so it is not recomputed here.
+__device__ __forceinline__ int int4_code(uint16_t wv, float sf, uint16_t& ref)
+{
+    if (sf == 0.0f) {
+        ref = 0;
+        return 8;
+    }
+    float t = h2f(f2h(h2f(wv) / sf));
+    t = fminf(64.0f, fmaxf(-64.0f, t));
+    int q = (int)rintf(t) + 8;
+    q = q < 0 ? 0 : (q > 15 ? 15 : q);
+    ref = f2h((float)(q - 8) * sf);
+    return q;
+}
+
+// One workgroup per (k-block, 512 columns): the 16 x 512 fp16 block goes through LDS with 16-byte accesses
+// on the memory side (the fragment order scatters single values); thread = fragment owner (kb, g64, t): four
+// packed words (16 contiguous bytes).  The check weights replace the block in LDS and leave the same way.
+constexpr int kPackCols = 512;
+__global__ __launch_bounds__(256) void int4_pack_kernel(const uint16_t* w, int k, int n, int n4, int g,
+                                                        const uint16_t* s, int per_column, uint32_t* out, uint16_t* w_ref)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t tile[16 * kPackCols];
+    __shared__ uint16_t scale[kPackCols];
+    const int kb = blockIdx.y, col0 = blockIdx.x * kPackCols, tid = threadIdx.x;
+    const int cols = n4 - col0 < kPackCols ? n4 - col0 : kPackCols;      // a multiple of 64
+    for (int id = tid; id < 16 * kPackCols / 8; id += 256) {
+        const int row = id / (kPackCols / 8), c8 = (id % (kPackCols / 8)) * 8;
+        if (c8 < cols)
+            *reinterpret_cast<uint4*>(&tile[row * kPackCols + c8]) =
+                *reinterpret_cast<const uint4*>(&w[(size_t)(16 * kb + row) * n + col0 + c8]);
+    }
+    for (int c = tid; c < cols; c += 256)
+        scale[c] = s[per_column ? scale_pos(col0 + c) : (size_t)(16 * kb / g) * n4 + col0 + c];
+    __syncthreads();
+    const int g64l = tid >> 5, t = tid & 31, l = t >> 2, i = t & 3;
+    if (64 * g64l < cols) {
+        uint32_t words[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                const int c = 64 * g64l + 16 * j + l + 8 * (x >> 2);
+                const int pos = k_off(i, x & 3) * kPackCols + c;
+                uint16_t ref;
+                const int q = int4_code(tile[pos], h2f(scale[c]), ref);
+                tile[pos] = ref;                                         // every element has exactly one owner
+                word |= (uint32_t)q << (4 * ((x & 1) * 4 + (x >> 1)));
+            }
+            words[j] = word;
+        }
+        const size_t owner = ((size_t)kb * (n4 / 64) + col0 / 64 + g64l) * 32 + t;
+        uint4 v = {words[0], words[1], words[2], words[3]};
+        reinterpret_cast<uint4*>(out)[owner] = v;
+    }
+    if (!w_ref) return;
+    __syncthreads();
+    for (int id = tid; id < 16 * kPackCols / 8; id += 256) {
+        const int row = id / (kPackCols / 8), c8 = (id % (kPackCols / 8)) * 8;
+        if (c8 < cols)
+            *reinterpret_cast<uint4*>(&w_ref[(size_t)(16 * kb + row) * n + col0 + c8]) =
+                *reinterpret_cast<const uint4*>(&tile[row * kPackCols + c8]);
+    }
+}
+
+// ---- FP6 region: columns [n4, n) of w
+
+// e3m2 code of a binary16 value by truncation (weight_quant.cpp:27-96); 0xff when |x| is outside
+// {0} u [0.0625, 28] or x is a NaN.
+__device__ __forceinline__ uint32_t fp6_code(uint16_t h)
+{
+    const uint32_t sign = (h >> 15) << 5, e = (h >> 10) & 31u, m = h & 0x3ffu;
+    if ((h & 0x7fffu) == 0) return sign;
+    if (e >= 13 && e <= 19) {
+        if (e == 19 && m > 0x300u) return 0xff;                      // above 28
+        return sign | ((e - 12) << 2) | (m >> 8);
+    }
+    if (e == 12) return sign | ((0x400u | m) >> 9);                  // 0.125 .. 0.25: sub-normal codes 2, 3
+    if (e == 11) return sign | 1;                                    // 0.0625 .. 0.125
+    return 0xff;
+}
+
+// binary16 pattern of a code's value (exact).
+__device__ __forceinline__ uint16_t fp6_value(uint32_t c)
+{
+    const uint32_t e = (c >> 2) & 7u, m = c & 3u;
+    const float v = e == 0 ? (float)m * 0.0625f : (1.0f + 0.25f * (float)m) * __builtin_ldexpf(1.0f, (int)e - 3);
+    return (uint16_t)(f2h(v) | ((c & 32u) ? 0x8000u : 0u));
+}
+
+// Largest magnitude per FP6 column, as the bit pattern of |x| (monotonic for binary16): 64 columns x 64
+// rows per workgroup, one atomicMax per column and workgroup into `amax` (zeroed before).
+__global__ __launch_bounds__(256) void fp6_amax_kernel(const uint16_t* w, int k, int n, int n4, int qc, unsigned* amax)
+{
+    __shared__ unsigned red[4][64];
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63), part = threadIdx.x >> 6, r0 = blockIdx.y * 64 + part * 16;
+    unsigned m = 0;
+    if (c < qc)
+        for (int r = r0; r < r0 + 16 && r < k; r++) {
+            const unsigned a = w[(size_t)r * n + n4 + c] & 0x7fffu;
+            m = a > m ? a : m;
+        }
+    red[part][threadIdx.x & 63] = m;
+    __syncthreads();
+    if (part == 0 && c < qc) {
+        for (int p = 1; p < 4; p++) m = red[p][threadIdx.x] > m ? red[p][threadIdx.x] : m;
+        atomicMax(&amax[c], m);
+    }
+}
+
+// s = max|w| * (1/28) (test.py:19-23); the real-transpose layout replaces a zero scale by one.
+__global__ void fp6_scales_kernel(const unsigned* amax, int qc, int harness, uint16_t* s6)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= qc) return;
+    uint16_t sh = f2h(h2f((uint16_t)amax[c]) * (float)(1.0 / 28.0));
+    if (!harness && (sh & 0x7fffu) == 0) sh = 0x3c00u;
+    s6[scale_pos(c)] = sh;
+}
+
+// One thread per fragment owner of the FP6 planes.  `row` (0..qc) and `col` (0..k) index the [qc, k]
+// matrix the reference's prepacker works on.  In the harness layout that matrix is the flat [k, qc]
+// buffer re-read with row length k (weight_quant pybind.cpp:52-57 does not transpose): element (row, col)
+// is flat element row*k + col, normalised by the scale of *its* column in the [k, qc] view, while the
+// check weight multiplies by the scale of `row` (test.py:37-38).  Otherwise it is the true transpose.
+__global__ void fp6_pack_kernel(const uint16_t* w, int k, int n, int n4, int qc, int harness, const uint16_t* s6,
+                                uint32_t* plane2, uint32_t* plane4, uint16_t* w_ref, int* bad)
+{
+    const size_t owner = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t groups = qc / 64, owners = (size_t)(k / 16) * groups * 32;
+    if (owner >= owners) return;
+    const int t = (int)(owner & 31), l = t >> 2, i = t & 3;
+    const size_t g64 = (owner >> 5) % groups, kb = (owner >> 5) / groups;
+    uint32_t w2[2] = {0, 0}, w4[4];
+    bool any_bad = false;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+            const size_t row = 64 * g64 + 16 * j + l + 8 * (x >> 2);
+            const size_t col = 16 * kb + k_off(i, x & 3);
+            size_t src_k = col, src_n = row;                         // where the value comes from in w's FP6 slice
+            if (harness) {
+                const size_t flat = row * (size_t)k + col;
+                src_k = flat / qc;
+                src_n = flat % qc;
+            }
+            const float sn = h2f(s6[scale_pos(src_n)]);
+            uint16_t v = f2h(h2f(w[src_k * n + n4 + src_n]) / sn);
+            if (h2f((uint16_t)(v & 0x7fffu)) < 0.0625f) v = 0;       // |x| < 0.0625 -> +0 (test.py:25); a NaN fails the test
+            else if (h2f((uint16_t)(v & 0x7fffu)) > 28.0f) v = (uint16_t)((v & 0x8000u) | 0x4f00u);   // clamp to +-28
+            const uint32_t c = fp6_code(v);
+            any_bad |= c == 0xff;
+            if (w_ref) w_ref[col * n + n4 + row] = f2h(h2f(fp6_value(c)) * h2f(s6[scale_pos(row)]));
+            const int b = fp6_byte_of(x), hi = x >> 2;
+            word |= (c & 15u) << (28 - 4 * (2 * b + hi));
+            w2[j >> 1] |= ((c >> 4) & 3u) << (30 - 2 * (4 * b + 2 * (j & 1) + hi));
+        }
+        w4[j] = word;
+    }
+    uint4 v4 = {w4[0], w4[1], w4[2], w4[3]};
+    reinterpret_cast<uint4*>(plane4)[owner] = v4;
+    uint2 v2 = {w2[0], w2[1]};
+    reinterpret_cast<uint2*>(plane2)[owner] = v2;
+    if (any_bad) *bad = 1;
+}
+
+}  // namespace
+}  // namespace fp6m
+
+extern "C" int fp6m_pack_mixed_device(const void* w, int k, int n, int quant_cols, int group_size, int harness_layout,
+                                      void* B, void* s, void* w_ref, int dev, void* stream)
+{
+    using namespace fp6m;
+    if (!w || !B || !s) return FP6M_ERR_ARG;
+    const int qc = quant_cols == -1 ? 0 : quant_cols;
+    if (k <= 0 || n <= 0 || qc < 0 || qc > n || qc % 64 || (n - qc) % 64 || k % 64 || n % 8) return FP6M_ERR_SHAPE;
+    if (group_size != -1 && (group_size <= 0 || k % group_size || group_size % 16)) return FP6M_ERR_SHAPE;
+    if ((size_t)qc * sizeof(unsigned) + 64 > kPackTemp) return FP6M_ERR_SHAPE;
+    const int n4 = n - qc, g = group_size == -1 ? k : group_size, per_column = group_size == -1;
+    hipError_t e = hipSetDevice(dev);
+    if (e != hipSuccess) return hip_fail(e);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* wp = static_cast<const uint16_t*>(w);
+    uint16_t* sp = static_cast<uint16_t*>(s);
+    uint16_t* rp = static_cast<uint16_t*>(w_ref);
+    uint32_t* bp = static_cast<uint32_t*>(B);
+    int* bad = nullptr;
+    if (n4) {
+        hipLaunchKernelGGL(int4_scales_kernel, dim3((n4 + 255) / 256, k / g), dim3(256), 0, st, wp, k, n, n4, g, sp, per_column);
+        hipLaunchKernelGGL(int4_pack_kernel, dim3((n4 + kPackCols - 1) / kPackCols, k / 16), dim3(256), 0, st, wp, k, n, n4, g,
+                           sp, per_column, bp, rp);
+    }
+    if (qc) {
+        void* temp = nullptr;
+        const int rc = pack_temp(dev, &temp);
+        if (rc != FP6M_OK) return rc;
+        bad = static_cast<int*>(temp);                                   // [0]: range flag, [16..]: column maxima
+        unsigned* amax = static_cast<unsigned*>(temp) + 16;
+        e = hipMemsetAsync(temp, 0, 64 + (size_t)qc * sizeof(unsigned), st);
+        if (e != hipSuccess) return hip_fail(e);
+        uint16_t* s6 = sp + (per_column ? (size_t)n4 : (size_t)(k / g) * n4);
+        uint32_t* plane2 = bp + (size_t)k * n4 / 8;
+        uint32_t* plane4 = plane2 + (size_t)k * qc / 16;
+        hipLaunchKernelGGL(fp6_amax_kernel, dim3((qc + 63) / 64, (k + 63) / 64), dim3(256), 0, st, wp, k, n, n4, qc, amax);
+        hipLaunchKernelGGL(fp6_scales_kernel, dim3((qc + 63) / 64), dim3(64), 0, st, amax, qc, harness_layout, s6);
+        const size_t owners = (size_t)(k / 16) * (qc / 64) * 32;
+        hipLaunchKernelGGL(fp6_pack_kernel, dim3((unsigned)((owners + 255) / 256)), dim3(256), 0, st, wp, k, n, n4, qc,
+                           harness_layout, s6, plane2, plane4, rp, bad);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+    int host_bad = 0;
+    if (bad) {
+        // the range check of the FP6 cast is reported by value, so this call waits for its kernels
+        e = hipMemcpyAsync(&host_bad, bad, sizeof(int), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return hip_fail(e);
+    }
+    return host_bad ? FP6M_ERR_RANGE : FP6M_OK;
+}

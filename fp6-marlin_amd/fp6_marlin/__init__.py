@@ -20,10 +20,10 @@ try:
 except ImportError as e:  # pragma: no cover
     raise ImportError("fp6_marlin/_fp6m_torch.so is missing or does not load: build it with "
                       "`python fp6-marlin_amd/build.py`; there is no fallback implementation") from e
-from .cabi import init, workspace_elems
+from .cabi import init, workspace_elems, pack_mixed_weight_device
 from .layer import Layer, pack_mixed_weight, int4_quantize, int4_pack, permute_scales, unpack_to_fp16
 
-__all__ = ["prepacking", "quantize", "dequantize", "mul", "Layer", "pack_mixed_weight", "int4_quantize",
+__all__ = ["prepacking", "quantize", "dequantize", "mul", "Layer", "pack_mixed_weight", "pack_mixed_weight_device", "int4_quantize",
            "int4_pack", "permute_scales", "unpack_to_fp16", "init", "workspace_elems"]
 
 

@@ -28,6 +28,8 @@ lib.fp6m_strerror.argtypes = [_int]
 lib.fp6m_last_hip_error.restype = _int
 lib.fp6m_abi_version.restype = _int
 lib.fp6m_workspace_elems.restype = _sz
+lib.fp6m_pack_mixed_device.restype = _int
+lib.fp6m_pack_mixed_device.argtypes = [_vp, _int, _int, _int, _int, _int, _vp, _vp, _vp, _int, _vp]
 lib.fp6m_workspace_elems.argtypes = [_int, _int]
 lib.fp6m_init.argtypes = [_int]
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
@@ -144,6 +146,31 @@ def unpack_to_fp16(B, s, k, n, quant_cols=-1, group_size=-1):
     out = torch.empty((k, n), dtype=torch.float16)
     _raise_cpu(lib.fp6m_unpack_to_fp16(B.data_ptr(), s.data_ptr(), out.data_ptr(), k, n, quant_cols, group_size))
     return out
+
+
+def pack_mixed_weight_device(w, quant_cols=-1, group_size=-1, harness_layout=True, want_ref=True):
+    """Quantise and pack a CUDA float16 weight [k, n] on the GPU; same outputs, bit for bit, as the host path
+    (`layer.pack_mixed_weight`).  Returns (B int32 1-D, s float16 1-D, w_ref float16 [k, n] or None), all on
+    w's device."""
+    if not isinstance(w, torch.Tensor) or not w.is_cuda or w.dtype != torch.float16 or w.dim() != 2:
+        raise ValueError("w must be a 2-D CUDA float16 tensor")
+    w = w.contiguous()
+    k, n = w.shape
+    qc = 0 if quant_cols in (-1, 0) else int(quant_cols)
+    n4 = n - qc
+    words = k * n4 // 8 + k * qc * 3 // 16
+    nscale = (n4 if group_size == -1 else (k // group_size if group_size > 0 else 0) * n4) + qc
+    B = torch.empty(words, dtype=torch.int32, device=w.device)
+    s = torch.empty(nscale, dtype=torch.float16, device=w.device)
+    ref = torch.empty((k, n), dtype=torch.float16, device=w.device) if want_ref else None
+    with torch.cuda.device(w.device):
+        code = lib.fp6m_pack_mixed_device(w.data_ptr(), k, n, qc, int(group_size), int(bool(harness_layout)), B.data_ptr(),
+                                          s.data_ptr(), ref.data_ptr() if want_ref else None, w.device.index,
+                                          torch.cuda.current_stream().cuda_stream)
+    if code == ERR_HIP:
+        raise RuntimeError(f"fp6m_pack_mixed_device: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+    _raise_cpu(code)
+    return B, s, ref
 
 
 # ------------------------------------------------------------------------------------------ the GEMM

@@ -44,9 +44,17 @@ def pack_mixed_weight(w, quant_cols=-1, group_size=-1, harness_layout=True):
     FP6 path quantises the [k, nq] buffer as if it were [nq, k] (no transpose, pybind.cpp:52-57), so the
     FP6 part of ``w_ref`` is a reshuffle of ``w``.  ``harness_layout=False`` transposes first, so that
     ``w_ref`` approximates ``w`` column for column: use that for real models (``Layer.pack`` does).
+
+    A CUDA ``w`` is quantised and packed on the GPU (same bits; outputs stay on its device); a CPU ``w`` goes
+    through the host routines.
     """
     if w.dtype != torch.float16 or w.dim() != 2:
         raise ValueError("w must be a 2-D float16 tensor")
+    if w.is_cuda:
+        qc_dev = 0 if quant_cols in (-1, 0) else quant_cols
+        if qc_dev < 0 or qc_dev > w.shape[1] or qc_dev % 64:
+            raise ValueError("quant_cols must be -1 or a multiple of 64 not above n")
+        return cabi.pack_mixed_weight_device(w.detach(), quant_cols, group_size, harness_layout)
     w = w.detach().cpu().contiguous()
     k, n = w.shape
     qc = 0 if quant_cols in (-1, 0) else quant_cols
@@ -109,9 +117,11 @@ class Layer(nn.Module):
         self.register_buffer("workspace", torch.zeros(outfeatures // 128 * 16, dtype=torch.int32), persistent=False)
 
     def pack(self, linear):
-        """Quantise and pack ``linear`` (an ``nn.Linear`` or a float16 weight [outfeatures, infeatures])."""
+        """Quantise and pack ``linear`` (an ``nn.Linear`` or a float16 weight [outfeatures, infeatures]).
+        A weight that lives on a GPU is packed there (70B-size layers take milliseconds instead of the host
+        packer's seconds); the result is the same bit for bit."""
         w = linear.weight.data if isinstance(linear, nn.Module) else linear
-        w = w.detach().to(torch.float16).cpu().t().contiguous()      # [k, n]
+        w = w.detach().to(torch.float16).t().contiguous()            # [k, n], on the weight's device
         if tuple(w.shape) != (self.k, self.n):
             raise ValueError("weight shape does not match the layer")
         B, s, w_ref = pack_mixed_weight(w, self.quant_cols, self.groupsize, harness_layout=False)

@@ -136,6 +136,21 @@ int fp6m_permute_scales(const uint16_t* in, uint16_t* out, size_t n);
 int fp6m_unpack_to_fp16(const int32_t* B, const uint16_t* s, uint16_t* w_ref, size_t k, size_t n,
                         int quant_cols, int group_size);
 
+/* Weight preparation on the GPU: what the reference's harness does on the host with numpy and its CPU extension
+ * (gen_mixed_weight test.py:123-152 = gen_int4_weight test.py:85-121 + gen_fp6_weight test.py:13-58, i.e.
+ * weight_quantization_cpu pybind.cpp:42-59 and weight_prepacking_cpu pybind.cpp:18-31, + the scale permutation
+ * test.py:80-83), in one call on device memory, bit for bit.
+ *   w        device fp16 [k, n] row-major
+ *   B, s     device outputs in the wire format of fp6m_mul (sizes as for fp6m_unpack_to_fp16)
+ *   w_ref    optional device fp16 [k, n]: the dequantised weight the GEMM multiplies by (NULL to skip)
+ *   harness_layout  1 = the reference harness bit for bit (its FP6 path reads the flat [k, quant_cols] buffer as
+ *            [quant_cols, k] without transposing); 0 = quantise the true transpose (what Layer.pack uses)
+ * k % 64 == 0, quant_cols and n - quant_cols multiples of 64, group_size -1 or a divisor of k.
+ * Enqueued on `stream`; when quant_cols > 0 the call waits for its kernels, because the FP6 range check
+ * (FP6M_ERR_RANGE: a NaN weight or a zero-scale column in the harness layout) is reported by value. */
+int fp6m_pack_mixed_device(const void* w, int k, int n, int quant_cols, int group_size, int harness_layout,
+                           void* B, void* s, void* w_ref, int dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
