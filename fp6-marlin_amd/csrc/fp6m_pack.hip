@@ -29,18 +29,27 @@ __device__ __forceinline__ size_t scale_pos(size_t c) { return (c & ~size_t(31))
 
 // ---- INT4 region: columns [0, n4) of w
 
-// One thread per (group, column): s = max|w| * 2/15 (test.py:88-89).
+// One thread per (group, 8 adjacent columns), 16-byte loads: s = max|w| * 2/15 (test.py:88-89).  The maximum of
+// |x| is taken on the bit patterns (monotonic for binary16), two columns per 32-bit lane.
 __global__ void int4_scales_kernel(const uint16_t* w, int k, int n, int n4, int g, uint16_t* s, int per_column)
 {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x, gi = blockIdx.y;
-    if (c >= n4) return;
-    uint16_t amax = 0;
-    for (int r = gi * g; r < (gi + 1) * g; r++) {
-        const uint16_t a = w[(size_t)r * n + c] & 0x7fffu;
-        amax = a > amax ? a : amax;
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8, gi = blockIdx.y;
+    if (c >= n4) return;                                                // n4 is a multiple of 64
+    us2 m[4] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+    const uint16_t* src = w + (size_t)gi * g * n + c;
+#pragma unroll 4
+    for (int r = 0; r < g; r++, src += n) {
+        const uint4 v = *reinterpret_cast<const uint4*>(src);
+        const uint32_t q[4] = {v.x & 0x7fff7fffu, v.y & 0x7fff7fffu, v.z & 0x7fff7fffu, v.w & 0x7fff7fffu};
+#pragma unroll
+        for (int t = 0; t < 4; t++) m[t] = __builtin_elementwise_max(m[t], __builtin_bit_cast(us2, q[t]));
     }
-    const uint16_t sh = f2h(h2f(amax) * (float)(2.0 / 15.0));
-    s[per_column ? scale_pos(c) : (size_t)gi * n4 + c] = sh;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        const uint16_t sh = f2h(h2f(m[t >> 1][t & 1]) * (float)(2.0 / 15.0));
+        s[per_column ? scale_pos(c + t) : (size_t)gi * n4 + c + t] = sh;
+    }
 }
 
 // q = clamp(round(w / s) + 8, 0, 15) and the check weight (q - 8) * s (test.py:90-98).  The harness packs the
@@ -236,7 +245,7 @@ extern "C" int fp6m_pack_mixed_device(const void* w, int k, int n, int quant_col
     uint32_t* bp = static_cast<uint32_t*>(B);
     int* bad = nullptr;
     if (n4) {
-        hipLaunchKernelGGL(int4_scales_kernel, dim3((n4 + 255) / 256, k / g), dim3(256), 0, st, wp, k, n, n4, g, sp, per_column);
+        hipLaunchKernelGGL(int4_scales_kernel, dim3((n4 / 8 + 255) / 256, k / g), dim3(256), 0, st, wp, k, n, n4, g, sp, per_column);
         hipLaunchKernelGGL(int4_pack_kernel, dim3((n4 + kPackCols - 1) / kPackCols, k / 16), dim3(256), 0, st, wp, k, n, n4, g,
                            sp, per_column, bp, rp);
     }
