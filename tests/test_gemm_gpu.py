@@ -34,16 +34,19 @@ def problem(oracle, n, k, qc=-1, gs=-1, seed=0):
     return _cache[key]
 
 
-def run(oracle, m, n, k, thread_k=-1, thread_n=-1, qc=-1, gs=-1, seed=0, max_par=16, ksplit=None, sms=-1):
+def run(oracle, m, n, k, thread_k=-1, thread_n=-1, qc=-1, gs=-1, seed=0, max_par=16, ksplit=None, sms=-1, env=None):
     import fp6_marlin
-    print(f"case m={m} n={n} k={k} tk={thread_k} tn={thread_n} qc={qc} gs={gs} ksplit={ksplit} sms={sms}", flush=True)
+    print(f"case m={m} n={n} k={k} tk={thread_k} tn={thread_n} qc={qc} gs={gs} ksplit={ksplit} sms={sms} env={env}", flush=True)
+    env = dict(env or {})
     ref, B, s = problem(oracle, n, k, qc, gs, seed)
     g = torch.Generator().manual_seed(seed * 7919 + m)
     A = torch.randn((m, k), generator=g, dtype=torch.float32).half()
     C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())      # must be fully overwritten
     ws = torch.zeros(n // 128 * max_par, dtype=torch.int32, device=dev())
     if ksplit is not None:
-        os.environ["FP6M_KSPLIT"] = str(ksplit)
+        env["FP6M_KSPLIT"] = ksplit
+    for name, value in env.items():                                # the library reads its tuning knobs on every call
+        os.environ[name] = str(value)
     try:
         fp6_marlin.mul(A.to(dev()), B, C, s, ws, qc, thread_k, thread_n, sms, max_par, gs)
         torch.cuda.synchronize()
@@ -51,7 +54,8 @@ def run(oracle, m, n, k, thread_k=-1, thread_n=-1, qc=-1, gs=-1, seed=0, max_par
         fp6_marlin.mul(A.to(dev()), B, C2, s, ws, qc, thread_k, thread_n, sms, max_par, gs)
         torch.cuda.synchronize()
     finally:
-        os.environ.pop("FP6M_KSPLIT", None)
+        for name in env:
+            os.environ.pop(name, None)
     assert int(ws.abs().sum().item()) == 0, "workspace must be left zeroed"
     c = C.cpu().numpy()
     assert np.isfinite(c).all(), "C not fully written"
@@ -139,6 +143,25 @@ def test_forced_split_k_and_determinism(oracle):
     run(oracle, 16, 512, 2048, qc=256, sms=1)                       # `sms` caps the partners at one
 
 
+def test_shared_fragment_kernel(oracle):
+    """The kernel that large launches use (four row tiles share a tile's dequantised fragments; one or two
+    column tiles per workgroup), forced onto small problems: ragged row tiles, odd tile counts in both regions,
+    per-column and group scales, one to three k parts."""
+    for wn in (1, 2):
+        e = {"FP6M_WM": 1, "FP6M_WN": wn}
+        run(oracle, 256, 512, 1024, qc=256, ksplit=1, env=e)
+        run(oracle, 256, 512, 1024, qc=256, gs=128, ksplit=1, env=e)
+        run(oracle, 64, 768, 1024, qc=128, ksplit=1, env=e)
+        run(oracle, 100, 1024, 1280, qc=128, gs=128, env=e)
+        run(oracle, 33, 256, 512, qc=128, env=e)
+        run(oracle, 17, 256, 64, qc=-1, env=e)
+        run(oracle, 300, 2048, 2048, qc=256, gs=128, env=e)
+        run(oracle, 300, 2304, 2048, qc=384, gs=128, ksplit=3, env=e)
+        run(oracle, 520, 512, 512, qc=512, ksplit=2, env=e)            # all FP6
+        run(oracle, 1100, 256, 1024, qc=-1, gs=128, max_par=16, env=e)  # second launch of 76 rows
+    run(oracle, 1024, 768, 1024, qc=256, gs=128)                       # default dispatch stays on the other kernel
+
+
 def test_max_par_chunks_m(oracle):
     """m-tiles beyond max_par go to further launches (fp6_marlin_cuda_kernel.cu:917-948)."""
     run(oracle, 300, 512, 512, qc=256, max_par=2)
@@ -192,7 +215,8 @@ def test_baseline_full_sizes_against_unpacked_words(oracle):
     unpacker, which tests/test_cpu_routines.py pins bit for bit against the oracle's dequantised weight; the
     reference product is an fp32 matmul of A with it.  Also: linearity in A (C(a1 + a2) = C(a1) + C(a2))."""
     import fp6_marlin
-    cases = [(1, 4096, 22016), (1, 11008, 4096), (16, 8192, 57344), (1, 28672, 8192), (128, 8192, 8192), (1024, 8192, 8192)]
+    cases = [(1, 4096, 22016), (1, 11008, 4096), (16, 8192, 57344), (1, 28672, 8192), (128, 8192, 8192), (1024, 8192, 8192),
+             (1024, 8192, 16384)]                                      # the last two: shared-fragment kernel, one and two tiles
     qc, gs = 256, 128
     g = torch.Generator().manual_seed(11)
     for m, k, n in cases:
