@@ -269,6 +269,58 @@ def one_shape(args):
     print(json.dumps(row), flush=True)
 
 
+def fused_bench(args):
+    """`--fused m,k,n[,quant_cols,group_size]`: `mul_fused` (activation gather, output scatter, bias, residual in
+    the call) against the same work done around `mul` with torch kernels; every variant replayed from a HIP
+    graph over rotated weights."""
+    import torch
+    import fp6_marlin
+    v = [int(x) for x in args.fused.split(",")]
+    m, k, n = v[:3]
+    qc, gs = (v[3] if len(v) > 3 else 256), (v[4] if len(v) > 4 else 128)
+    gen = torch.Generator().manual_seed(0)
+    fp6_marlin.init(0)
+    copies = max(2, min(24, int(640e6 // weight_bytes(k, n, qc, gs)) + 1))
+    probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
+    a_cols = torch.randperm(k, generator=gen).to(torch.int32).cuda()
+    c_cols = torch.randperm(n, generator=gen).to(torch.int32).cuda()
+    inv = torch.argsort(c_cols.long())
+    bias = torch.randn(n, generator=gen).half().cuda()
+    res = torch.randn((m, n), generator=gen).half().cuda()
+    out = torch.empty((m, n), dtype=torch.half, device="cuda")
+    a_l = a_cols.long()
+
+    def plain(i):
+        probs[i % copies].run(fp6_marlin.mul)
+
+    def fused(**kw):
+        def f(i):
+            p = probs[i % copies]
+            fp6_marlin.mul_fused(p.A, p.B, p.C, p.s, p.ws, p.qc if p.qc else -1, p.gs, **kw)
+        return f
+
+    def around(i):                                                      # the same result with separate kernels
+        p = probs[i % copies]
+        ag = torch.index_select(p.A, 1, a_l)
+        fp6_marlin.mul(ag, p.B, p.C, p.s, p.ws, p.qc if p.qc else -1, -1, -1, -1, 16, p.gs)
+        torch.index_select(p.C, 1, inv, out=out)
+        out.add_(bias).add_(res)
+
+    variants = {"mul": plain, "fused_scatter": fused(c_cols=c_cols), "fused_gather": fused(a_cols=a_cols),
+                "fused_bias_residual": fused(bias=bias, residual=res),
+                "fused_all": fused(a_cols=a_cols, c_cols=c_cols, bias=bias, residual=res), "torch_kernels_around_mul": around}
+    row = {"fused": f"m={m} {k}x{n} qc={qc} gs={gs}"}
+    iters = copies * max(1, 100 // copies)
+    for name, f in variants.items():
+        for i in range(4):
+            f(i)
+        torch.cuda.synchronize()
+        fn, calls = graphed(torch, f, copies, iters)
+        _, ev = time_region(torch, fn, calls)
+        row[name + "_us"] = round(ev / iters * 1e6, 2)
+    print(json.dumps(row), flush=True)
+
+
 def pack_bench(args):
     """`--pack k,n[,quant_cols,group_size]`: on-GPU weight preparation (fp16 [k, n] -> B, s) against the host
     packers on the box's cores.  Algorithmic bytes: the fp16 weight read once, the packed words and scales
@@ -329,6 +381,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
     ap.add_argument("--shape", type=str, default=None, help="m,k,n[,quant_cols,group_size]: measure one shape")
+    ap.add_argument("--fused", type=str, default=None, help="m,k,n[,quant_cols,group_size]: time mul_fused against mul + torch kernels")
     ap.add_argument("--pack", type=str, default=None, help="k,n[,quant_cols,group_size]: time the on-GPU weight packer")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -345,6 +398,8 @@ def main():
         one_shape(args)
     elif args.pack:
         pack_bench(args)
+    elif args.fused:
+        fused_bench(args)
     else:
         headline(args)
 

@@ -57,6 +57,11 @@ struct GemmArgs {
     // m <= 16 kernel: the FP6 and the INT4 region are covered by separate ranges of workgroups
     int ks6, ks4;             // k parts (workgroups) per tile group, per region
     int groups6, groups4;     // tile groups (WN adjacent tiles) per region
+    // optional epilogue work (fp6m_mul_fused); `fused` is set when any of the three is
+    const int32_t* c_cols;    // column of C that packed column j goes to
+    const uint16_t* bias;     // fp16 [n], indexed by C column
+    const uint16_t* residual; // fp16 [m, n], same rows as C
+    int fused;
 #ifdef FP6M_TIMELINE
     unsigned long long* timeline;   // 8 realtime-clock stamps per workgroup (performance debugging builds only)
 #endif
@@ -90,6 +95,31 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int total)
 {
     const int q = total >> 3, r = total & 7, x = b & 7;
     return x * q + (x < r ? x : r) + (b >> 3);
+}
+
+// Epilogue of fp6m_mul_fused for two adjacent packed columns of one row: C[row, c_cols[col]] =
+// fp16(v + bias[c_cols[col]] + residual[row, c_cols[col]]), everything added in fp32 and rounded once.
+// Map entries are clamped to the row so that a bad map cannot write outside C.
+__device__ __forceinline__ void store_fused(const GemmArgs& p, size_t row, int col, float v0, float v1)
+{
+    int c0 = col, c1 = col + 1;
+    if (p.c_cols) {
+        c0 = p.c_cols[col];
+        c1 = p.c_cols[col + 1];
+        c0 = c0 < 0 ? 0 : (c0 >= p.n ? p.n - 1 : c0);
+        c1 = c1 < 0 ? 0 : (c1 >= p.n ? p.n - 1 : c1);
+    }
+    if (p.bias) {
+        v0 += (float)__builtin_bit_cast(_Float16, p.bias[c0]);
+        v1 += (float)__builtin_bit_cast(_Float16, p.bias[c1]);
+    }
+    const size_t r = row * (size_t)p.n;
+    if (p.residual) {
+        v0 += (float)__builtin_bit_cast(_Float16, p.residual[r + c0]);
+        v1 += (float)__builtin_bit_cast(_Float16, p.residual[r + c1]);
+    }
+    p.C[r + c0] = __builtin_bit_cast(uint16_t, (_Float16)v0);
+    p.C[r + c1] = __builtin_bit_cast(uint16_t, (_Float16)v1);
 }
 
 // ------------------------------------------------------------------------------------------------ tile bookkeeping
@@ -480,6 +510,10 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
     }
     uint16_t* c_out = p.C + ti.col0 + 2 * lane;
     auto store_row = [&](int m, float v0, float v1) {
+        if (p.fused) {
+            store_fused(p, (size_t)m, ti.col0 + 2 * lane, v0 * s0, v1 * s1);
+            return;
+        }
         h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
         *reinterpret_cast<h2*>(c_out + (size_t)m * p.n) = o;
     };
@@ -982,6 +1016,10 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     }
     uint16_t* c_out = p.C + (size_t)row0 * p.n + ti.col0 + 2 * lane;
     auto store_row = [&](int row, float v0, float v1) {
+        if (p.fused) {
+            store_fused(p, (size_t)(row0 + row), ti.col0 + 2 * lane, v0 * s0, v1 * s1);
+            return;
+        }
         h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
         *reinterpret_cast<h2*>(c_out + (size_t)row * p.n) = o;
     };
@@ -1462,6 +1500,22 @@ __global__ __launch_bounds__(512, 2) void gemm_wm_kernel(const GemmArgs p)
                          reinterpret_cast<int*>(smem + wm_lds<WN>() - 64) + grp, valid);
 }
 
+// Activation gather of fp6m_mul_fused: out[r, kk] = A[r, a_cols[kk]] (map entries clamped to the row).  One
+// thread per pair of output elements; the m x k result is what the GEMM kernels then stream as their A.
+__global__ __launch_bounds__(256) void gather_a_kernel(const uint16_t* __restrict__ A, int lda,
+                                                      const int32_t* __restrict__ a_cols, uint16_t* __restrict__ out,
+                                                      int k)
+{
+    const int kk = 2 * (blockIdx.x * 256 + threadIdx.x);
+    if (kk >= k) return;
+    const size_t row = blockIdx.y;
+    int c0 = a_cols[kk], c1 = a_cols[kk + 1];
+    c0 = c0 < 0 ? 0 : (c0 >= lda ? lda - 1 : c0);
+    c1 = c1 < 0 ? 0 : (c1 >= lda ? lda - 1 : c1);
+    const uint32_t v = (uint32_t)A[row * lda + c0] | ((uint32_t)A[row * lda + c1] << 16);
+    *reinterpret_cast<uint32_t*>(out + row * k + kk) = v;
+}
+
 // ------------------------------------------------------------------------------------------------ host
 
 thread_local int g_last_hip_error = 0;
@@ -1469,7 +1523,9 @@ thread_local int g_last_hip_error = 0;
 struct DeviceScratch {
     float* ptr = nullptr;
     int cus = 0;
+    uint16_t* gathered = nullptr;   // gathered activations of fp6m_mul_fused (kGatherBytes, on first use)
 };
+constexpr size_t kGatherBytes = size_t(64) << 20;
 constexpr int kMaxDevices = 64;
 DeviceScratch g_scratch[kMaxDevices];
 std::mutex g_scratch_mutex;
@@ -1500,6 +1556,23 @@ int ensure_scratch(int dev, DeviceScratch** out)
         d.cus = cus > 0 ? cus : 256;
     }
     *out = &d;
+    return FP6M_OK;
+}
+
+// The buffer the gathered activations of fp6m_mul_fused go through: allocated on the first call that gathers.
+int ensure_gather_buffer(int dev, DeviceScratch* d)
+{
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (d->gathered) return FP6M_OK;
+    int prev = 0;
+    hipError_t e = hipGetDevice(&prev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) return hip_fail(e);
+    void* mem = nullptr;
+    e = hipMalloc(&mem, kGatherBytes);
+    if (prev != dev) (void)hipSetDevice(prev);
+    if (e != hipSuccess) return hip_fail(e);
+    d->gathered = static_cast<uint16_t*>(mem);
     return FP6M_OK;
 }
 
@@ -1580,11 +1653,23 @@ int fp6m_init(int dev)
     return fp6m::ensure_scratch(dev, &d);
 }
 
-int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
-             void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
-             int quant_cols, int group_size)
+}  // extern "C"
+
+namespace fp6m {
+
+// Optional work around the GEMM (fp6m_mul_fused); all null / zero for fp6m_mul.
+struct Fusion {
+    const int32_t* a_cols = nullptr;
+    int lda = 0;
+    const int32_t* c_cols = nullptr;
+    const uint16_t* bias = nullptr;
+    const uint16_t* residual = nullptr;
+};
+
+int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+               void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
+               int quant_cols, int group_size, const Fusion& fu)
 {
-    using namespace fp6m;
     if (prob_m < 0 || prob_n < 0 || prob_k < 0) return FP6M_ERR_ARG;
 
     // Tile-shape arguments are validated the way the reference does it
@@ -1627,6 +1712,10 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     a.qc = qc;
     a.tiles6 = qc / kTileN;
     a.tiles = prob_n / kTileN;
+    a.c_cols = fu.c_cols;
+    a.bias = fu.bias;
+    a.residual = nullptr;
+    a.fused = fu.c_cols || fu.bias || fu.residual;
 #ifdef FP6M_TIMELINE
     a.timeline = nullptr;
     if (const char* e = getenv("FP6M_TIMELINE_PTR")) a.timeline = reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0));
@@ -1653,12 +1742,27 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
     const int units = g128 ? prob_k / 128 : prob_k / 64;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (fu.a_cols) {
+        const long long launch_rows = prob_m < (long long)rows_per_tile * max_par ? prob_m : (long long)rows_per_tile * max_par;
+        if ((size_t)launch_rows * prob_k * sizeof(uint16_t) > kGatherBytes) return FP6M_ERR_ARG;
+        if (int rc = ensure_gather_buffer(dev, scratch)) return rc;
+    }
     for (int mt0 = 0; mt0 < mtiles_total; mt0 += max_par) {
         const int mtiles = mtiles_total - mt0 < max_par ? mtiles_total - mt0 : max_par;
         const int rows0 = mt0 * rows_per_tile;
-        a.A = static_cast<const uint16_t*>(A) + (size_t)rows0 * prob_k;
         a.C = static_cast<uint16_t*>(C) + (size_t)rows0 * prob_n;
+        a.residual = fu.residual ? fu.residual + (size_t)rows0 * prob_n : nullptr;
         a.m = prob_m - rows0 < mtiles * rows_per_tile ? prob_m - rows0 : mtiles * rows_per_tile;
+        if (fu.a_cols) {
+            // the launch's rows of A, gathered into the per-device buffer (stream order keeps the launches apart)
+            dim3 ggrid((unsigned)((prob_k / 2 + 255) / 256), (unsigned)a.m);
+            hipLaunchKernelGGL(gather_a_kernel, ggrid, dim3(256), 0, st,
+                               static_cast<const uint16_t*>(A) + (size_t)rows0 * fu.lda, fu.lda, fu.a_cols,
+                               scratch->gathered, prob_k);
+            a.A = scratch->gathered;
+        } else {
+            a.A = static_cast<const uint16_t*>(A) + (size_t)rows0 * prob_k;
+        }
 
         const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
         const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
@@ -1748,6 +1852,33 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
         if (e != hipSuccess) return hip_fail(e);
     }
     return FP6M_OK;
+}
+
+}  // namespace fp6m
+
+extern "C" {
+
+int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+             void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
+             int quant_cols, int group_size)
+{
+    return fp6m::mul_common(A, B, C, s, prob_m, prob_n, prob_k, workspace, dev, stream, thread_k, thread_n, sms, max_par,
+                            quant_cols, group_size, fp6m::Fusion{});
+}
+
+int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+                   void* workspace, int dev, void* stream, int sms, int max_par, int quant_cols, int group_size,
+                   const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual)
+{
+    fp6m::Fusion fu;
+    fu.a_cols = a_cols;
+    fu.lda = lda;
+    fu.c_cols = c_cols;
+    fu.bias = static_cast<const uint16_t*>(bias);
+    fu.residual = static_cast<const uint16_t*>(residual);
+    if (a_cols ? lda <= 0 : lda != prob_k) return FP6M_ERR_ARG;
+    return fp6m::mul_common(A, B, C, s, prob_m, prob_n, prob_k, workspace, dev, stream, -1, -1, sms, max_par, quant_cols,
+                            group_size, fu);
 }
 
 }  // extern "C"

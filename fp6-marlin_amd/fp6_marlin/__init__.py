@@ -8,7 +8,8 @@ Same surface as liuchuan22/FP6-Marlin's ``fp6_marlin`` package (fp6_marlin/__ini
     mul(A, B, C, s, workspace, quant_cols=-1, thread_k=-1, thread_n=-1, sms=-1, max_par=16)
 
 plus what the reference keeps in its test harness or lacks: ``Layer`` (pack / forward), the INT4
-quantiser and packer, the scale permutation, the mixed-weight assembler and ``group_size=128`` scales.
+quantiser and packer, the scale permutation, the mixed-weight assembler, ``group_size=128`` scales and
+``mul_fused`` (activation gather, output column scatter, bias and residual inside the GEMM call).
 Everything is computed by ``libfp6m.so`` (C ABI in include/fp6m.h: host packers in C++, GEMM in
 hand-written HIP for gfx950).  The four reference entry points go through ``_fp6m_torch``, a thin
 PyTorch-ROCm C++ extension over that C ABI; ``fp6_marlin.cabi`` binds the same ABI with ctypes.
@@ -20,11 +21,11 @@ try:
 except ImportError as e:  # pragma: no cover
     raise ImportError("fp6_marlin/_fp6m_torch.so is missing or does not load: build it with "
                       "`python fp6-marlin_amd/build.py`; there is no fallback implementation") from e
-from .cabi import init, workspace_elems, pack_mixed_weight_device
+from .cabi import init, workspace_elems, pack_mixed_weight_device, mul_fused, check_column_map
 from .layer import Layer, pack_mixed_weight, int4_quantize, int4_pack, permute_scales, unpack_to_fp16
 
 __all__ = ["prepacking", "quantize", "dequantize", "mul", "Layer", "pack_mixed_weight", "pack_mixed_weight_device", "int4_quantize",
-           "int4_pack", "permute_scales", "unpack_to_fp16", "init", "workspace_elems"]
+           "int4_pack", "permute_scales", "unpack_to_fp16", "init", "workspace_elems", "mul_fused", "check_column_map"]
 
 
 def prepacking(fp6_tensor):

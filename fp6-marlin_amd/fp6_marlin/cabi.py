@@ -33,6 +33,8 @@ lib.fp6m_pack_mixed_device.argtypes = [_vp, _int, _int, _int, _int, _int, _vp, _
 lib.fp6m_workspace_elems.argtypes = [_int, _int]
 lib.fp6m_init.argtypes = [_int]
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
+lib.fp6m_mul_fused.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _vp, _vp,
+                               _vp, _vp]
 lib.fp6m_fp6_quantize.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_fp6_prepack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_fp6_dequant.argtypes = [_vp, _vp, _sz, _sz, _vp]
@@ -40,7 +42,7 @@ lib.fp6m_int4_quantize.argtypes = [_vp, _sz, _sz, _int, _vp, _vp, _vp]
 lib.fp6m_int4_pack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_permute_scales.argtypes = [_vp, _vp, _sz]
 lib.fp6m_unpack_to_fp16.argtypes = [_vp, _vp, _vp, _sz, _sz, _int, _int]
-for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
+for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
            lib.fp6m_int4_quantize, lib.fp6m_int4_pack, lib.fp6m_permute_scales, lib.fp6m_unpack_to_fp16):
     _f.restype = _int
 
@@ -222,3 +224,70 @@ def mul(A, B, C, s, workspace, quant_cols=-1, thread_k=-1, thread_n=-1, sms=-1, 
         raise RuntimeError(f"No kernel implementation for thread_k={thread_k}, thread_n={thread_n}.")
     if code != OK:
         raise RuntimeError(f"fp6m_mul: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+
+
+def check_column_map(cols, size, permutation=False):
+    """Validate an int32 CUDA map for `mul_fused` on the host side (one device sync): entries inside
+    [0, size), and a permutation if asked.  Do it once per map, not per call."""
+    if not isinstance(cols, torch.Tensor) or not cols.is_cuda or cols.dtype != torch.int32 or cols.dim() != 1:
+        raise ValueError("a column map must be a 1-D CUDA int32 tensor")
+    if cols.numel() and (int(cols.min()) < 0 or int(cols.max()) >= size):
+        raise ValueError(f"column map entries must lie in [0, {size})")
+    if permutation and (cols.numel() != size or int(torch.unique(cols).numel()) != size):
+        raise ValueError(f"column map must be a permutation of 0..{size - 1}")
+    return cols
+
+
+def mul_fused(A, B, C, s, workspace, quant_cols=-1, group_size=-1, a_cols=None, c_cols=None, bias=None, residual=None,
+              sms=-1, max_par=16):
+    """`mul` with the reorders and additions around it folded into the launch (no counterpart in the reference,
+    whose harness leaves them to the caller: the FP6 columns of its packed weight sit at the tail, test.py:123-152):
+
+        C[:, c_cols] = fp16(A[:, a_cols] @ dequant(B) * s + bias[c_cols] + residual[:, c_cols])
+
+    a_cols int32 [k] (columns of A, which may then be wider than k), c_cols int32 [n] permutation, bias float16 [n],
+    residual float16 [m, n] (may be C).  Maps are trusted here: run `check_column_map` on them once."""
+    tensors = [("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)]
+    tensors += [(nm, t) for nm, t in (("a_cols", a_cols), ("c_cols", c_cols), ("bias", bias), ("residual", residual))
+                if t is not None]
+    for name, t in tensors:
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise RuntimeError(f"{name} must be a tensor on the GPU")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+        if t.device != A.device:
+            raise RuntimeError("all operands must live on the same device")
+    if A.dtype != torch.float16 or C.dtype != torch.float16 or s.dtype != torch.float16:
+        raise RuntimeError("A, C and s must be float16")
+    if B.element_size() != 4 or workspace.element_size() != 4:
+        raise RuntimeError("B must be int32 (or another 4-byte type) and workspace a 4-byte type")
+    if A.dim() != 2 or C.dim() != 2 or C.shape[0] != A.shape[0]:
+        raise RuntimeError("A must be [m, lda] and C [m, n]")
+    m, lda = A.shape
+    n = C.shape[1]
+    k = lda if a_cols is None else a_cols.numel()
+    for name, t, numel in (("a_cols", a_cols, k), ("c_cols", c_cols, n)):
+        if t is not None and (t.dtype != torch.int32 or t.numel() != numel):
+            raise RuntimeError(f"{name} must be int32 with {numel} entries")
+    if bias is not None and (bias.dtype != torch.float16 or bias.numel() != n):
+        raise RuntimeError(f"bias must be float16 with {n} entries")
+    if residual is not None and (residual.dtype != torch.float16 or tuple(residual.shape) != (m, n)):
+        raise RuntimeError("residual must be float16 [m, n]")
+    if workspace.numel() < n // 128 * max_par:
+        raise RuntimeError(f"workspace must be of size at least {n // 128 * max_par}.")
+    qc = 0 if quant_cols in (-1, 0) else quant_cols
+    n4 = n - qc
+    if k % 32 == 0 and 0 <= qc <= n:
+        need_b = k * n4 // 8 + k * qc * 3 // 16
+        need_s = (n4 if group_size == -1 else (k // 128) * n4) + qc
+        if B.numel() < need_b or s.numel() != need_s:
+            raise RuntimeError(f"B must hold {need_b} words and s {need_s} scales for this problem")
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(A.device):
+        code = lib.fp6m_mul_fused(A.data_ptr(), lda, B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k,
+                                  workspace.data_ptr(), A.device.index, torch.cuda.current_stream().cuda_stream, sms,
+                                  max_par, quant_cols, group_size, ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual))
+    if code == ERR_PROB_SHAPE:
+        raise RuntimeError(f"Problem (m={m}, n={n}, k={k}) not compatible with the tile shape.")
+    if code != OK:
+        raise RuntimeError(f"fp6m_mul_fused: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")

@@ -73,6 +73,28 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
              void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
              int quant_cols, int group_size);
 
+/*
+ * The GEMM with the reordering and the additions around it folded in.  No counterpart in the reference: its
+ * harness packs a weight whose FP6 columns already sit at the tail (gen_mixed_weight, test.py:123-152) and
+ * leaves the matching reorder of the output columns (and, for selected input channels, of the activations) and
+ * any bias / residual addition to separate kernels of the caller.
+ *   A, lda    device fp16 [m, lda] row-major.  Without a_cols, lda must equal prob_k.
+ *   a_cols    device int32 [prob_k] or NULL: row kk of the packed weight multiplies column a_cols[kk] of A
+ *             (0 <= a_cols[kk] < lda).  The gathered rows pass through a 64 MiB per-device buffer that the first
+ *             such call allocates; min(prob_m, 64 * max_par) * prob_k * 2 bytes must fit (else FP6M_ERR_ARG).
+ *   c_cols    device int32 [prob_n] or NULL: packed column j (INT4 columns first, then the FP6 columns) is written
+ *             to column c_cols[j] of C; must be a permutation of 0 .. prob_n-1.
+ *   bias      device fp16 [prob_n] or NULL, indexed by C column.
+ *   residual  device fp16 [prob_m, prob_n] or NULL, laid out like C; may be C itself (in-place accumulation).
+ *   C[r, c_cols[j]] = fp16(acc[r, j] * scale[j] + bias[c_cols[j]] + residual[r, c_cols[j]]): the additions are in
+ *   fp32 and the result is rounded once.  With all four NULL the result equals fp6m_mul's bit for bit.
+ * Map entries out of range are clamped on the device (wrong values, no fault); validate maps once on the host.
+ * Other arguments as for fp6m_mul (tile shapes are always automatic).
+ */
+int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+                   void* workspace, int dev, void* stream, int sms, int max_par, int quant_cols, int group_size,
+                   const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual);
+
 /* Minimum workspace length in 4-byte elements: n / 128 * max_par (fp6_marlin/fp6_marlin_cuda.cpp:62-63). */
 size_t fp6m_workspace_elems(int prob_n, int max_par);
 

@@ -1,0 +1,166 @@
+"""GPU tests of `mul_fused` (C ABI fp6m_mul_fused): the activation gather, the output column scatter and the
+bias / residual additions around the GEMM.  The reference has no such entry; what pins it here:
+
+* with nothing to add, the scattered result is the plain `mul` result bit for bit (C_fused[:, c_cols] == C);
+* a gathered A equals `mul` on the materialised A[:, a_cols] bit for bit;
+* bias / residual: fp16(x + bias + residual) where x is recovered exactly from a bias-free run whose outputs are
+  integers (A and the dequantised weight are chosen so that every product sum is a small integer, hence exact in
+  fp16 and fp32), and, on random data, the oracle's fp32 product plus the additions within the GEMM tolerance
+  (mean |d| / mean |ref| <= 1e-3).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from oracle import fp6m_oracle
+    return fp6m_oracle
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def packed(oracle, k, n, qc, gs, seed=0):
+    rng = np.random.default_rng(seed)
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float16)
+    ref, b, s = oracle.gen_mixed_weight(w, qc, gs, strict=False)
+    return ref, torch.from_numpy(b).to(dev()), torch.from_numpy(s).to(dev())
+
+
+def plain(fp6_marlin, A, B, s, n, qc, gs):
+    C = torch.full((A.shape[0], n), float("nan"), dtype=torch.half, device=dev())
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+    fp6_marlin.cabi.mul(A, B, C, s, ws, qc, -1, -1, -1, 16, gs)
+    torch.cuda.synchronize()
+    assert int(ws.abs().sum()) == 0
+    return C
+
+
+@pytest.mark.parametrize("m", [1, 16, 48, 200, 1100])
+def test_scatter_and_gather_are_exact_reorders(oracle, m):
+    import fp6_marlin
+    k, n, qc, gs = 1024, 768, 256, 128
+    print(f"case fused reorder m={m}", flush=True)
+    ref, B, s = packed(oracle, k, n, qc, gs)
+    g = torch.Generator().manual_seed(m)
+    lda = k + 64
+    A_wide = torch.randn((m, lda), generator=g).half().to(dev())
+    a_cols = torch.randperm(lda, generator=g)[:k].to(torch.int32).to(dev())
+    c_cols = torch.randperm(n, generator=g).to(torch.int32).to(dev())
+    fp6_marlin.check_column_map(a_cols, lda)
+    fp6_marlin.check_column_map(c_cols, n, permutation=True)
+    A = A_wide[:, a_cols.long()].contiguous()
+    want = plain(fp6_marlin, A, B, s, n, qc, gs)
+
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+    for use_a, use_c in ((False, True), (True, False), (True, True), (False, False)):
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        fp6_marlin.mul_fused(A_wide if use_a else A, B, C, s, ws, qc, gs, a_cols=a_cols if use_a else None,
+                             c_cols=c_cols if use_c else None)
+        torch.cuda.synchronize()
+        got = C[:, c_cols.long()] if use_c else C
+        assert torch.equal(got, want), (use_a, use_c)
+        assert int(ws.abs().sum()) == 0
+    err = oracle.rel_err(want.cpu().numpy(), oracle.matmul_ref(A.cpu().numpy(), ref))
+    assert err <= TOL
+
+
+@pytest.mark.parametrize("m", [3, 16, 40, 130])
+def test_bias_and_residual_round_once(oracle, m):
+    """Integer-valued products: the bias-free output x is exact, so the fused result must be fp16(x + b + r)
+    with one rounding, bit for bit."""
+    import fp6_marlin
+    k, n, qc, gs = 256, 512, 128, -1
+    print(f"case fused bias m={m}", flush=True)
+    rng = np.random.default_rng(5)
+    # weights on both grids: INT4 codes times scale 1 -> integers in [-8, 7]; FP6 values {0, +-1, +-2, +-3, +-4}
+    w = rng.integers(-4, 5, (k, n)).astype(np.float16)
+    w[:, :n - qc] = rng.integers(-7, 8, (k, n - qc))
+    w[0, :n - qc] = 7.5                                               # max |w| = 7.5 -> INT4 scale 2 * 7.5 / 15 = 1
+    w[0, n - qc:] = 28.0                                              # max |w| = 28 per column -> FP6 scale 1
+    ref, b, s = oracle.gen_mixed_weight(w, qc, gs, strict=False)
+    B, sd = torch.from_numpy(b).to(dev()), torch.from_numpy(s).to(dev())
+    g = torch.Generator().manual_seed(m)
+    A = torch.randint(-1, 2, (m, k), generator=g).half().to(dev())
+    x = plain(fp6_marlin, A, B, sd, n, qc, gs)
+    x_ref = A.float().cpu().numpy() @ ref.astype(np.float32)
+    assert np.array_equal(x.float().cpu().numpy(), x_ref.astype(np.float16).astype(np.float32))
+    assert np.abs(x_ref).max() < 2048                                 # integers below 2048: exact in fp16
+
+    bias = (torch.randn(n, generator=g) * 3).half().to(dev())
+    res = (torch.randn((m, n), generator=g) * 5).half().to(dev())
+    c_cols = torch.randperm(n, generator=g).to(torch.int32).to(dev())
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+    for use_b, use_r, use_c in ((True, False, False), (False, True, False), (True, True, False), (True, True, True)):
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        fp6_marlin.mul_fused(A, B, C, sd, ws, qc, gs, c_cols=c_cols if use_c else None, bias=bias if use_b else None,
+                             residual=res if use_r else None)
+        torch.cuda.synchronize()
+        xs = torch.empty_like(x)
+        if use_c:
+            xs[:, c_cols.long()] = x
+        else:
+            xs = x
+        want = xs.float() + (bias.float() if use_b else 0) + (res.float() if use_r else 0)
+        assert torch.equal(C, want.half()), (use_b, use_r, use_c)
+    # in place: residual is C itself
+    C = res.clone()
+    fp6_marlin.mul_fused(A, B, C, sd, ws, qc, gs, residual=C)
+    torch.cuda.synchronize()
+    assert torch.equal(C, (x.float() + res.float()).half())
+
+
+def test_fused_on_random_data_against_oracle(oracle):
+    import fp6_marlin
+    for m, k, n, qc, gs in ((1, 2048, 1024, 256, 128), (16, 1024, 1536, 512, -1), (300, 1024, 1024, 256, 128)):
+        print(f"case fused random m={m} k={k} n={n}", flush=True)
+        ref, B, s = packed(oracle, k, n, qc, gs, seed=m)
+        g = torch.Generator().manual_seed(m)
+        A = torch.randn((m, k), generator=g).half()
+        a_cols = torch.randperm(k, generator=g).to(torch.int32)
+        c_cols = torch.randperm(n, generator=g).to(torch.int32)
+        bias = torch.randn(n, generator=g).half()
+        res = torch.randn((m, n), generator=g).half()
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+        fp6_marlin.mul_fused(A.to(dev()), B, C, s, ws, qc, gs, a_cols=a_cols.to(dev()), c_cols=c_cols.to(dev()),
+                             bias=bias.to(dev()), residual=res.to(dev()))
+        torch.cuda.synchronize()
+        prod = oracle.matmul_ref(A[:, a_cols.long()].numpy(), ref).astype(np.float32)
+        want = np.empty_like(prod)
+        want[:, c_cols.numpy()] = prod
+        want = want + bias.float().numpy() + res.float().numpy()
+        assert oracle.rel_err(C.cpu().numpy(), want) <= TOL
+
+
+def test_fused_argument_errors():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import fp6_marlin
+    m, k, n = 4, 256, 256
+    A = torch.zeros((m, k), dtype=torch.half, device=dev())
+    B = torch.zeros(k * n // 8, dtype=torch.int32, device=dev())
+    s = torch.ones(n, dtype=torch.half, device=dev())
+    C = torch.zeros((m, n), dtype=torch.half, device=dev())
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+    with pytest.raises(RuntimeError):
+        fp6_marlin.mul_fused(A, B, C, s, ws, c_cols=torch.zeros(n - 1, dtype=torch.int32, device=dev()))
+    with pytest.raises(RuntimeError):
+        fp6_marlin.mul_fused(A, B, C, s, ws, bias=torch.zeros(n, dtype=torch.float32, device=dev()))
+    with pytest.raises(RuntimeError):
+        fp6_marlin.mul_fused(A, B, C, s, ws, residual=torch.zeros((m + 1, n), dtype=torch.half, device=dev()))
+    with pytest.raises(ValueError):
+        fp6_marlin.check_column_map(torch.full((n,), n, dtype=torch.int32, device=dev()), n)
+    with pytest.raises(ValueError):
+        fp6_marlin.check_column_map(torch.zeros(n, dtype=torch.int32, device=dev()), n, permutation=True)
+    fp6_marlin.mul_fused(A, B, C, s, ws)                               # nothing to fuse: plain GEMM
+    torch.cuda.synchronize()
+    assert float(C.abs().sum()) == 0
