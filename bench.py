@@ -321,6 +321,55 @@ def fused_bench(args):
     print(json.dumps(row), flush=True)
 
 
+def rows_bench(args):
+    """`--rows m,k,n[,quant_rows]`: the row-mixed GEMM (`mul_rows`: INT4 rows and FP6 rows of every column in one
+    launch) against what the column-mix entry needs for the same result (one `mul` per row range and an addition),
+    both replayed from HIP graphs over rotated weights.  Bytes: INT4 words + FP6 planes + scales, read once."""
+    import torch
+    import fp6_marlin
+    v = [int(x) for x in args.rows.split(",")]
+    m, k, n = v[:3]
+    qr = v[3] if len(v) > 3 else 256
+    k4 = k - qr
+    gen = torch.Generator().manual_seed(0)
+    fp6_marlin.init(0)
+    words4, words6, ns4 = k4 * n // 8, qr * n * 3 // 16, (k4 // 128) * n
+    nbytes = 4 * (words4 + words6) + 2 * (ns4 + n)
+    copies = max(2, min(24, int(640e6 // nbytes) + 1))
+    Bs = [torch.randint(-2 ** 31, 2 ** 31 - 1, (words4 + words6,), generator=gen, dtype=torch.int64).to(torch.int32).cuda()
+          for _ in range(copies)]
+    ss = [(torch.rand(ns4 + n, generator=gen) * 0.01 + 0.001).half().cuda() for _ in range(copies)]
+    parts = [(b[:words4].clone(), b[words4:].clone(), x[:ns4].clone(), x[ns4:].clone()) for b, x in zip(Bs, ss)]
+    A = torch.randn((m, k), generator=gen).half().cuda()
+    A4, A6 = A[:, :k4].contiguous(), A[:, k4:].contiguous()
+    C, C4, C6 = (torch.zeros((m, n), dtype=torch.half, device="cuda") for _ in range(3))
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device="cuda")
+
+    def one(i):
+        fp6_marlin.mul_rows(A, Bs[i % copies], C, ss[i % copies], ws, qr)
+
+    def two(i):
+        b4, b6, s4, s6 = parts[i % copies]
+        fp6_marlin.mul(A4, b4, C4, s4, ws, -1, -1, -1, -1, 16, 128)
+        fp6_marlin.mul(A6, b6, C6, s6, ws, n, -1, -1, -1, 16, -1)
+        torch.add(C4, C6, out=C)
+
+    row = {"rows": f"m={m} {k}x{n} quant_rows={qr}", "weight_bytes": nbytes}
+    iters = copies * max(1, 100 // copies)
+    for name, f in (("mul_rows", one), ("two_mul_and_add", two)):
+        for i in range(4):
+            f(i)
+        torch.cuda.synchronize()
+        fn, calls = graphed(torch, f, copies, iters)
+        _, ev = time_region(torch, fn, calls)
+        row[name + "_us"] = round(ev / iters * 1e6, 2)
+    t = row["mul_rows_us"] * 1e-6
+    row["weight_GBs"] = round(nbytes / t / 1e9, 1)
+    row["hbm_frac"] = round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)
+    row["TFLOPs"] = round(2 * m * k * n / t / 1e12, 2)
+    print(json.dumps(row), flush=True)
+
+
 def pack_bench(args):
     """`--pack k,n[,quant_cols,group_size]`: on-GPU weight preparation (fp16 [k, n] -> B, s) against the host
     packers on the box's cores.  Algorithmic bytes: the fp16 weight read once, the packed words and scales
@@ -382,6 +431,7 @@ def main():
     ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
     ap.add_argument("--shape", type=str, default=None, help="m,k,n[,quant_cols,group_size]: measure one shape")
     ap.add_argument("--fused", type=str, default=None, help="m,k,n[,quant_cols,group_size]: time mul_fused against mul + torch kernels")
+    ap.add_argument("--rows", type=str, default=None, help="m,k,n[,quant_rows]: time the row-mixed GEMM against two mul calls and an addition")
     ap.add_argument("--pack", type=str, default=None, help="k,n[,quant_cols,group_size]: time the on-GPU weight packer")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -400,6 +450,8 @@ def main():
         pack_bench(args)
     elif args.fused:
         fused_bench(args)
+    elif args.rows:
+        rows_bench(args)
     else:
         headline(args)
 

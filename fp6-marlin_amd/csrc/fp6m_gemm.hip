@@ -57,6 +57,9 @@ struct GemmArgs {
     // m <= 16 kernel: the FP6 and the INT4 region are covered by separate ranges of workgroups
     int ks6, ks4;             // k parts (workgroups) per tile group, per region
     int groups6, groups4;     // tile groups (WN adjacent tiles) per region
+    // row mix (fp6m_mul_rows): rows [0, k4) of every column are INT4 with group scales, rows [k4, k) FP6.  The
+    // k slices of a tile (parts x waves) are numbered INT4 first: slices [0, slices4) cover the INT4 rows.
+    int k4, slices4;          // 0 = column mix
     // optional epilogue work (fp6m_mul_fused); `fused` is set when any of the three is
     const int32_t* c_cols;    // column of C that packed column j goes to
     const uint16_t* bias;     // fp16 [n], indexed by C column
@@ -130,7 +133,25 @@ struct TileInfo {
     int tcol;                // tile index inside its region
     int region_n;            // columns of the region
     int col0;                // first column of the tile in C
+    int a_step0;             // k step of A that step 0 of the wave's weight segment multiplies (row mix: k4 / 32)
 };
+
+// Row mix: slice `sl` of the `nsl` slices of a tile -> its segment (ti.fp6, ti.a_step0) and its steps there.
+__device__ __forceinline__ void row_mix_slice(const GemmArgs& p, int sl, int nsl, TileInfo& ti, int& begin, int& end)
+{
+    ti.fp6 = sl >= p.slices4;
+    if (!ti.fp6) {
+        const int units = p.k4 / 128;
+        begin = (int)((long long)units * sl / p.slices4) * 4;
+        end = (int)((long long)units * (sl + 1) / p.slices4) * 4;
+        ti.a_step0 = 0;
+    } else {
+        const int units = (p.k - p.k4) / 64, s6 = sl - p.slices4, n6 = nsl - p.slices4;
+        begin = (int)((long long)units * s6 / n6) * 2;
+        end = (int)((long long)units * (s6 + 1) / n6) * 2;
+        ti.a_step0 = p.k4 / 32;
+    }
+}
 
 __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 {
@@ -143,6 +164,7 @@ __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
     t.tcol = t.fp6 ? t.tile : t.tile - p.tiles6;
     t.region_n = t.fp6 ? p.qc : p.n4;
     t.col0 = (t.fp6 ? p.n4 : 0) + t.tcol * kTileN;
+    t.a_step0 = 0;
     return t;
 }
 
@@ -323,7 +345,7 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const bool a_active = a_m < AROWS && ti.mtile * 16 + a_m < p.m;
     const uint32_t va = (uint32_t)(a_active ? a_m : 0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3));
     const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)ti.mtile * 16 * p.k) +
-                                  (size_t)step_begin * 64;
+                                  (size_t)(ti.a_step0 + step_begin) * 64;
     const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
     const uint32_t vgs = 4 * lane;
     constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;        // 256-byte slabs of group scales: 2 suffice up to depth 5
@@ -483,8 +505,11 @@ constexpr int wave_lds_bytes(int d4, int d6, int arows)
 template <int WN, int WK>
 __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti, bool tile_valid, int wn, int wk,
                                           int ks, int slot_base, int* counter, f4 (&acc)[1][8],
-                                          bool per_column_scale, unsigned char* smem, int wave_lds, int* flag)
+                                          bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
+                                          int first_fp6 = WK)
 {
+    // first_fp6: row mix only -- k slices first_fp6 .. WK-1 of this workgroup hold FP6 rows, whose sums take the
+    // FP6 column scale here (the INT4 slices are already scaled by their group scales)
     constexpr int RMAX = (16 + WK - 1) / WK;                             // rows one wave finishes
     constexpr int PCHUNK = 32 / RMAX;                                    // parts whose loads are in flight together
     typedef float f2 __attribute__((ext_vector_type(2)));
@@ -508,6 +533,13 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
         s0 = (float)sv[0];
         s1 = (float)sv[1];
     }
+    float x0 = 1.0f, x1 = 1.0f;                                          // FP6 column scales of a row mix
+    if (tile_valid && first_fp6 < WK) {
+        const int nr = ti.tcol * kTileN + 2 * lane;
+        const h2 sv = *reinterpret_cast<const h2*>(p.s_fp6 + (nr & ~31) + scale_slot(nr & 31));
+        x0 = (float)sv[0];
+        x1 = (float)sv[1];
+    }
     uint16_t* c_out = p.C + ti.col0 + 2 * lane;
     auto store_row = [&](int m, float v0, float v1) {
         if (p.fused) {
@@ -530,8 +562,8 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
             for (int j = 0; j < WK; j++) {
                 const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + (j * WN + wn) * wave_lds) +
                                                           m * kRedStride + 2 * lane);
-                v0[r] += v[0];
-                v1[r] += v[1];
+                v0[r] += j >= first_fp6 ? v[0] * x0 : v[0];
+                v1[r] += j >= first_fp6 ? v[1] * x1 : v[1];
             }
         }
     }
@@ -630,8 +662,11 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     constexpr int unit_steps = G128 ? 4 : 2;
     const int units = p.k / (32 * unit_steps);
     const int kp = ti.part * WK + wk, kparts = ks * WK;
-    const int step_begin = (int)((long long)units * kp / kparts) * unit_steps;
-    const int step_end = (int)((long long)units * (kp + 1) / kparts) * unit_steps;
+    int step_begin = (int)((long long)units * kp / kparts) * unit_steps;
+    int step_end = (int)((long long)units * (kp + 1) / kparts) * unit_steps;
+    ti.a_step0 = 0;
+    const bool region6 = ti.fp6;                                         // the workgroup's column region
+    if (p.k4) row_mix_slice(p, kp, kparts, ti, step_begin, step_end);    // per wave: INT4 or FP6 rows of the tile
 
     f4 acc[1][8];
 #pragma unroll
@@ -645,10 +680,10 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     }
     FP6M_MARK(p, 2);
     // scratch slots: FP6 groups first (groups6 * ks6 slots), then INT4 groups; counters likewise
-    const int slot_base = ti.fp6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
-    int* counter = p.counters + (ti.fp6 ? group : p.groups6 + group);
-    wg_finish<WN, WK>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, ti.fp6 || !G128, smem, kWaveLds,
-                      reinterpret_cast<int*>(smem + NW * kWaveLds));
+    const int slot_base = region6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
+    int* counter = p.counters + (region6 ? group : p.groups6 + group);
+    wg_finish<WN, WK>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+                      reinterpret_cast<int*>(smem + NW * kWaveLds), p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
 }
 
@@ -811,7 +846,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
                  (kAOff + 1024 * mb) % 4096;
     }
     const unsigned char* base_a = uniform_ptr(reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
-                                              (size_t)step_begin * 64 - 4096);
+                                              (size_t)(ti.a_step0 + step_begin) * 64 - 4096);
     const unsigned char* base_gs =
         uniform_ptr(reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN));
     const uint32_t vgs = 4 * lane;
@@ -997,7 +1032,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
 template <int MB, int WK = kWaves>
 __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, f4 (&acc)[MB][8],
                                              bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
-                                             bool valid = true)
+                                             bool valid = true, int first_fp6 = WK)
 {
     constexpr int RMAX = 16 / WK, PCHUNK = 32 / RMAX;                // parts whose loads are in flight together
     typedef float f2 __attribute__((ext_vector_type(2)));
@@ -1013,6 +1048,13 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
         const h2 sv = *reinterpret_cast<const h2*>(sp + (nr & ~31) + scale_slot(nr & 31));
         s0 = (float)sv[0];
         s1 = (float)sv[1];
+    }
+    float x0 = 1.0f, x1 = 1.0f;                                      // row mix: FP6 column scales of slices >= first_fp6
+    if (first_fp6 < WK) {
+        const int nr = ti.tcol * kTileN + 2 * lane;
+        const h2 sv = *reinterpret_cast<const h2*>(p.s_fp6 + (nr & ~31) + scale_slot(nr & 31));
+        x0 = (float)sv[0];
+        x1 = (float)sv[1];
     }
     uint16_t* c_out = p.C + (size_t)row0 * p.n + ti.col0 + 2 * lane;
     auto store_row = [&](int row, float v0, float v1) {
@@ -1044,8 +1086,8 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
                 for (int j = 0; j < WK; j++) {
                     const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + j * wave_lds) +
                                                               m * kRedStride + 2 * lane);
-                    v0 += v[0];
-                    v1 += v[1];
+                    v0 += j >= first_fp6 ? v[0] * x0 : v[0];
+                    v1 += j >= first_fp6 ? v[1] * x1 : v[1];
                 }
                 if (ks == 1) {
                     store_row(row, v0, v1);
@@ -1123,10 +1165,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_mb_kernel(const GemmArgs p)
     __shared__ __attribute__((aligned(16))) unsigned char smem[kWaves * kWaveLds + 16];
 
     FP6M_MARK(p, 0);
-    const TileInfo ti = locate_tile(p);
+    TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int step_begin, step_end;
     wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
+    if (p.k4) row_mix_slice(p, ti.part * kWaves + wave, p.ksplit * kWaves, ti, step_begin, step_end);
 
     f4 acc[MB][8];
 #pragma unroll
@@ -1141,8 +1184,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_mb_kernel(const GemmArgs p)
             stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
     }
     FP6M_MARK(p, 2);
-    wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, ti.fp6 || !G128, smem, kWaveLds,
-                     reinterpret_cast<int*>(smem + kWaves * kWaveLds));
+    wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+                     reinterpret_cast<int*>(smem + kWaves * kWaveLds), true, p.k4 ? p.slices4 - ti.part * kWaves : kWaves);
     FP6M_MARK(p, 7);
 }
 
@@ -1252,7 +1295,7 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
         va[mb] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3)) + 4096 - 1024 * mb;
     }
     const unsigned char* base_a = uniform_ptr(reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
-                                              (size_t)step_begin * 64 - 4096);
+                                              (size_t)(ti.a_step0 + step_begin) * 64 - 4096);
     const unsigned char* base_gs =
         uniform_ptr(reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN));
     const uint32_t vgs = 4 * lane;
@@ -1467,6 +1510,7 @@ __global__ __launch_bounds__(512, 2) void gemm_wm_kernel(const GemmArgs p)
     ti.tcol = tcol;
     ti.tile = ti.fp6 ? tcol : p.tiles6 + tcol;
     ti.col0 = (ti.fp6 ? p.n4 : 0) + tcol * kTileN;
+    ti.a_step0 = 0;
 
     // k slices: part-major, then wk; every wave of the workgroup runs the longest slice's step count
     constexpr int unit_steps = G128 ? 4 : 2;
@@ -1664,6 +1708,7 @@ struct Fusion {
     const int32_t* c_cols = nullptr;
     const uint16_t* bias = nullptr;
     const uint16_t* residual = nullptr;
+    int quant_rows = 0;              // > 0: row mix (fp6m_mul_rows), the last quant_rows rows of k are FP6
 };
 
 int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
@@ -1674,16 +1719,22 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
 
     // Tile-shape arguments are validated the way the reference does it
     // (fp6_marlin_cuda_kernel.cu:890-905, 933-944) even though they do not pick a kernel here.
-    if (thread_k == -1 || thread_n == -1) {
-        thread_k = prob_m <= 16 ? 128 : 64;
-        thread_n = prob_m <= 16 ? 128 : 256;
+    if (fu.quant_rows > 0) {
+        // the row mix is no reference path: its own rule is whole 128-column tiles (and, below, whole k units)
+        if (prob_n % kTileN) return FP6M_ERR_PROB_SHAPE;
+        if (prob_m == 0 || prob_n == 0) return FP6M_OK;
+    } else {
+        if (thread_k == -1 || thread_n == -1) {
+            thread_k = prob_m <= 16 ? 128 : 64;
+            thread_n = prob_m <= 16 ? 128 : 256;
+        }
+        if (thread_k <= 0 || thread_n <= 0) return FP6M_ERR_KERN_SHAPE;
+        if (prob_n % thread_n != 0 || prob_k % thread_k != 0) return FP6M_ERR_PROB_SHAPE;
+        if (prob_m == 0 || prob_n == 0 || prob_k == 0) return FP6M_OK;
+        const bool small_tile = thread_k == 128 && thread_n == 128;
+        const bool large_tile = thread_k == 64 && thread_n == 256;
+        if (!(large_tile || (small_tile && prob_m <= 16))) return FP6M_ERR_KERN_SHAPE;
     }
-    if (thread_k <= 0 || thread_n <= 0) return FP6M_ERR_KERN_SHAPE;
-    if (prob_n % thread_n != 0 || prob_k % thread_k != 0) return FP6M_ERR_PROB_SHAPE;
-    if (prob_m == 0 || prob_n == 0 || prob_k == 0) return FP6M_OK;
-    const bool small_tile = thread_k == 128 && thread_n == 128;
-    const bool large_tile = thread_k == 64 && thread_n == 256;
-    if (!(large_tile || (small_tile && prob_m <= 16))) return FP6M_ERR_KERN_SHAPE;
 
     if (!A || !B || !C || !s || !workspace) return FP6M_ERR_ARG;
     if (max_par <= 0) return FP6M_ERR_ARG;
@@ -1692,8 +1743,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     const int n4 = prob_n - qc;
     if (n4 % kTileN || qc % kTileN) return FP6M_ERR_PROB_SHAPE;
     if (group_size != -1 && group_size != 128) return FP6M_ERR_ARG;
+    const bool row_mix = fu.quant_rows > 0;
+    const int k4 = prob_k - fu.quant_rows;                            // row mix: INT4 rows
+    if (row_mix) {
+        if (qc != 0 || group_size != 128 || fu.quant_rows >= prob_k) return FP6M_ERR_ARG;
+        if (k4 % 128 || fu.quant_rows % 64) return FP6M_ERR_PROB_SHAPE;
+    }
     const bool g128 = group_size == 128 && n4 > 0;
-    if (g128 && prob_k % 128) return FP6M_ERR_PROB_SHAPE;
+    if (g128 && prob_k % 128 && !row_mix) return FP6M_ERR_PROB_SHAPE;
 
     DeviceScratch* scratch = nullptr;
     if (int rc = ensure_scratch(dev, &scratch)) return rc;
@@ -1712,6 +1769,16 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.qc = qc;
     a.tiles6 = qc / kTileN;
     a.tiles = prob_n / kTileN;
+    a.k4 = 0;
+    a.slices4 = 0;
+    if (row_mix) {
+        // every tile spans all n columns of both segments: INT4 words of rows [0, k4), then the FP6 planes of the rest
+        a.b_fp6_2 = a.b_int4 + (size_t)k4 * prob_n / 8;
+        a.b_fp6_4 = a.b_fp6_2 + (size_t)fu.quant_rows * prob_n / 16;
+        a.s_fp6 = a.s_int4 + (size_t)(k4 / 128) * prob_n;
+        a.qc = prob_n;
+        a.k4 = k4;
+    }
     a.c_cols = fu.c_cols;
     a.bias = fu.bias;
     a.residual = nullptr;
@@ -1736,6 +1803,17 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     const long long weights = (long long)prob_n * prob_k;
     bool shared_frags = rows_per_launch >= 1024 && weights >= (64LL << 20);
     if (const char* e = getenv("FP6M_WM")) shared_frags = prob_m > 16 && atoi(e) != 0;   // tuning/testing override
+    if (row_mix) shared_frags = false;                                // its waves run in lock step on one segment
+    // Row mix: the kWaves * ks slices of a tile are dealt to the two segments in proportion to their cost (an FP6
+    // step costs about two INT4 steps), at least one each.
+    auto deal_slices = [&](int total) {
+        const long long c4 = k4 / 32, c6 = 2LL * (fu.quant_rows / 32);
+        long long n6 = (total * c6 + (c4 + c6) / 2) / (c4 + c6);
+        if (n6 > fu.quant_rows / 64) n6 = fu.quant_rows / 64;
+        if (n6 > total - 1) n6 = total - 1;
+        if (n6 < 1) n6 = 1;
+        return (int)(total - n6);
+    };
     if (shared_frags) mb = 4;
     const int rows_per_tile = 16 * mb;
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
@@ -1821,6 +1899,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.ks6 = (int)(2 * ks <= ks_k ? 2 * ks : (ks > ks_k ? ks : ks_k));
             if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
             a.ksplit = a.ks4;
+            if (row_mix) {
+                a.ks6 = 0;                                            // no FP6 column region: groups6 is 0
+                a.slices4 = deal_slices(a.ks4 * cfg.wk);
+            }
             dim3 grid((unsigned)(a.groups6 * a.ks6 + a.groups4 * a.ks4), 1);
             if (getenv("FP6M_VERBOSE"))
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u\n", a.m, prob_n,
@@ -1841,6 +1923,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (ks < 1) ks = 1;
             while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
             a.ksplit = (int)ks;
+            if (row_mix) a.slices4 = deal_slices(a.ksplit * kWaves);
             dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
             if (getenv("FP6M_VERBOSE"))
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d grid=%ux%u\n", a.m, prob_n, prob_k, mb, mtiles,
@@ -1879,6 +1962,22 @@ int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s
     if (a_cols ? lda <= 0 : lda != prob_k) return FP6M_ERR_ARG;
     return fp6m::mul_common(A, B, C, s, prob_m, prob_n, prob_k, workspace, dev, stream, -1, -1, sms, max_par, quant_cols,
                             group_size, fu);
+}
+
+int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+                  void* workspace, int dev, void* stream, int sms, int max_par, int quant_rows, const int32_t* a_cols,
+                  const int32_t* c_cols, const void* bias, const void* residual)
+{
+    fp6m::Fusion fu;
+    fu.a_cols = a_cols;
+    fu.lda = lda;
+    fu.c_cols = c_cols;
+    fu.bias = static_cast<const uint16_t*>(bias);
+    fu.residual = static_cast<const uint16_t*>(residual);
+    fu.quant_rows = quant_rows;
+    if (quant_rows <= 0) return FP6M_ERR_ARG;
+    if (a_cols ? lda <= 0 : lda != prob_k) return FP6M_ERR_ARG;
+    return fp6m::mul_common(A, B, C, s, prob_m, prob_n, prob_k, workspace, dev, stream, -1, -1, sms, max_par, -1, 128, fu);
 }
 
 }  // extern "C"

@@ -35,6 +35,7 @@ lib.fp6m_init.argtypes = [_int]
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
 lib.fp6m_mul_fused.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _vp, _vp,
                                _vp, _vp]
+lib.fp6m_mul_rows.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _vp, _vp, _vp, _vp]
 lib.fp6m_fp6_quantize.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_fp6_prepack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_fp6_dequant.argtypes = [_vp, _vp, _sz, _sz, _vp]
@@ -42,7 +43,7 @@ lib.fp6m_int4_quantize.argtypes = [_vp, _sz, _sz, _int, _vp, _vp, _vp]
 lib.fp6m_int4_pack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_permute_scales.argtypes = [_vp, _vp, _sz]
 lib.fp6m_unpack_to_fp16.argtypes = [_vp, _vp, _vp, _sz, _sz, _int, _int]
-for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
+for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
            lib.fp6m_int4_quantize, lib.fp6m_int4_pack, lib.fp6m_permute_scales, lib.fp6m_unpack_to_fp16):
     _f.restype = _int
 
@@ -238,15 +239,7 @@ def check_column_map(cols, size, permutation=False):
     return cols
 
 
-def mul_fused(A, B, C, s, workspace, quant_cols=-1, group_size=-1, a_cols=None, c_cols=None, bias=None, residual=None,
-              sms=-1, max_par=16):
-    """`mul` with the reorders and additions around it folded into the launch (no counterpart in the reference,
-    whose harness leaves them to the caller: the FP6 columns of its packed weight sit at the tail, test.py:123-152):
-
-        C[:, c_cols] = fp16(A[:, a_cols] @ dequant(B) * s + bias[c_cols] + residual[:, c_cols])
-
-    a_cols int32 [k] (columns of A, which may then be wider than k), c_cols int32 [n] permutation, bias float16 [n],
-    residual float16 [m, n] (may be C).  Maps are trusted here: run `check_column_map` on them once."""
+def _mul_extended(A, B, C, s, workspace, quant_cols, group_size, quant_rows, a_cols, c_cols, bias, residual, sms, max_par):
     tensors = [("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)]
     tensors += [(nm, t) for nm, t in (("a_cols", a_cols), ("c_cols", c_cols), ("bias", bias), ("residual", residual))
                 if t is not None]
@@ -275,19 +268,64 @@ def mul_fused(A, B, C, s, workspace, quant_cols=-1, group_size=-1, a_cols=None, 
         raise RuntimeError("residual must be float16 [m, n]")
     if workspace.numel() < n // 128 * max_par:
         raise RuntimeError(f"workspace must be of size at least {n // 128 * max_par}.")
-    qc = 0 if quant_cols in (-1, 0) else quant_cols
-    n4 = n - qc
-    if k % 32 == 0 and 0 <= qc <= n:
-        need_b = k * n4 // 8 + k * qc * 3 // 16
-        need_s = (n4 if group_size == -1 else (k // 128) * n4) + qc
-        if B.numel() < need_b or s.numel() != need_s:
-            raise RuntimeError(f"B must hold {need_b} words and s {need_s} scales for this problem")
+    if quant_rows:
+        k4 = k - quant_rows
+        if quant_rows < 0 or k4 <= 0:
+            raise RuntimeError("quant_rows must be positive and below k")
+        if k4 % 128 == 0 and quant_rows % 64 == 0:
+            need_b, need_s = k4 * n // 8 + quant_rows * n * 3 // 16, (k4 // 128) * n + n
+            if B.numel() < need_b or s.numel() != need_s:
+                raise RuntimeError(f"B must hold {need_b} words and s {need_s} scales for this problem")
+    else:
+        qc = 0 if quant_cols in (-1, 0) else quant_cols
+        n4 = n - qc
+        if k % 32 == 0 and 0 <= qc <= n:
+            need_b = k * n4 // 8 + k * qc * 3 // 16
+            need_s = (n4 if group_size == -1 else (k // 128) * n4) + qc
+            if B.numel() < need_b or s.numel() != need_s:
+                raise RuntimeError(f"B must hold {need_b} words and s {need_s} scales for this problem")
     ptr = lambda t: None if t is None else t.data_ptr()
     with torch.cuda.device(A.device):
-        code = lib.fp6m_mul_fused(A.data_ptr(), lda, B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k,
-                                  workspace.data_ptr(), A.device.index, torch.cuda.current_stream().cuda_stream, sms,
-                                  max_par, quant_cols, group_size, ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual))
+        stream = torch.cuda.current_stream().cuda_stream
+        if quant_rows:
+            name = "fp6m_mul_rows"
+            code = lib.fp6m_mul_rows(A.data_ptr(), lda, B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k,
+                                     workspace.data_ptr(), A.device.index, stream, sms, max_par, quant_rows,
+                                     ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual))
+        else:
+            name = "fp6m_mul_fused"
+            code = lib.fp6m_mul_fused(A.data_ptr(), lda, B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k,
+                                      workspace.data_ptr(), A.device.index, stream, sms, max_par, quant_cols, group_size,
+                                      ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual))
     if code == ERR_PROB_SHAPE:
         raise RuntimeError(f"Problem (m={m}, n={n}, k={k}) not compatible with the tile shape.")
     if code != OK:
-        raise RuntimeError(f"fp6m_mul_fused: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+        raise RuntimeError(f"{name}: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+
+
+def mul_fused(A, B, C, s, workspace, quant_cols=-1, group_size=-1, a_cols=None, c_cols=None, bias=None, residual=None,
+              sms=-1, max_par=16):
+    """`mul` with the reorders and additions around it folded into the launch (no counterpart in the reference,
+    whose harness leaves them to the caller: the FP6 columns of its packed weight sit at the tail, test.py:123-152):
+
+        C[:, c_cols] = fp16(A[:, a_cols] @ dequant(B) * s + bias[c_cols] + residual[:, c_cols])
+
+    a_cols int32 [k] (columns of A, which may then be wider than k), c_cols int32 [n] permutation, bias float16 [n],
+    residual float16 [m, n] (may be C).  Maps are trusted here: run `check_column_map` on them once."""
+    _mul_extended(A, B, C, s, workspace, quant_cols, group_size, 0, a_cols, c_cols, bias, residual, sms, max_par)
+
+
+def mul_rows(A, B, C, s, workspace, quant_rows, a_cols=None, c_cols=None, bias=None, residual=None, sms=-1, max_par=16):
+    """The GEMM for a weight mixed along k instead of n: the last `quant_rows` rows (input channels) of every
+    column are FP6 with one scale per column, the rows before them INT4 with one scale per 128 rows and column.
+    Both segments of a column tile accumulate into the same output tile inside one launch.  (The reference mixes
+    along n only, fp6_marlin_cuda_kernel.cu:308-337; the same result there takes two `mul` calls and an addition.)
+
+        B = INT4 words of rows [0, k - quant_rows) || FP6 2-bit plane of the last rows || their 4-bit plane
+        s = INT4 group scales [(k - quant_rows) / 128, n] || FP6 column scales [n] (permuted order)
+
+    (k - quant_rows) % 128 == 0, quant_rows % 64 == 0, n % 128 == 0.  The optional arguments are those of
+    `mul_fused`; `a_cols` is how arbitrary input channels get to the FP6 tail."""
+    if int(quant_rows) <= 0:
+        raise RuntimeError("quant_rows must be positive and below k")
+    _mul_extended(A, B, C, s, workspace, -1, 128, int(quant_rows), a_cols, c_cols, bias, residual, sms, max_par)

@@ -87,6 +87,22 @@ def pack_mixed_weight(w, quant_cols=-1, group_size=-1, harness_layout=True):
             torch.cat(parts_ref, dim=1).contiguous())
 
 
+def pack_row_mix_weight(w, quant_rows):
+    """Quantise and pack a float16 weight ``w`` [k, n] for ``mul_rows``: the last ``quant_rows`` rows (input
+    channels) go to FP6 with one scale per column, the rows before them to INT4 with one scale per 128 rows and
+    column.  Returns ``(B, s, w_ref)`` like ``pack_mixed_weight``; both segments use its routines (on the GPU for
+    a CUDA ``w``), the FP6 one in the layout that quantises each column by its own scale."""
+    if w.dtype != torch.float16 or w.dim() != 2:
+        raise ValueError("w must be a 2-D float16 tensor")
+    k, n = w.shape
+    k4 = k - quant_rows
+    if quant_rows <= 0 or k4 <= 0 or k4 % 128 or quant_rows % 64 or n % 128:
+        raise ValueError("need 0 < quant_rows < k, (k - quant_rows) % 128 == 0, quant_rows % 64 == 0 and n % 128 == 0")
+    b4, s4, r4 = pack_mixed_weight(w[:k4].contiguous(), -1, 128)
+    b6, s6, r6 = pack_mixed_weight(w[k4:].contiguous(), n, -1, harness_layout=False)
+    return torch.cat([b4, b6]).contiguous(), torch.cat([s4, s6]).contiguous(), torch.cat([r4, r6], dim=0).contiguous()
+
+
 class Layer(nn.Module):
     """Linear layer ``y = x @ W`` with W [infeatures, outfeatures] stored as mixed INT4 / FP6.
 

@@ -95,6 +95,23 @@ int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s
                    void* workspace, int dev, void* stream, int sms, int max_par, int quant_cols, int group_size,
                    const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual);
 
+/*
+ * The GEMM for a weight mixed along k instead of n: the last quant_rows rows (input channels) of every column are
+ * FP6 e3m2 with one scale per column, the prob_k - quant_rows rows before them INT4 with one scale per 128 rows and
+ * column.  Both segments of a column tile accumulate into the same output tile inside one launch.  No counterpart
+ * in the reference, which splits the columns between the two formats (fp6_marlin_cuda_kernel.cu:308-337); there the
+ * same result takes two launches on the two row ranges and an addition.
+ *   B   INT4 words of rows [0, prob_k - quant_rows) (fp6m_int4_pack of that [rows, n] block) || FP6 2-bit plane ||
+ *       FP6 4-bit plane of the last quant_rows rows (fp6m_fp6_prepack of that [quant_rows, n] block)
+ *   s   INT4 scales [(prob_k - quant_rows) / 128, n] in natural column order || FP6 scales [n] in the permuted
+ *       order of fp6m_permute_scales
+ * (prob_k - quant_rows) % 128, quant_rows % 64 or prob_n % 128 != 0 -> FP6M_ERR_PROB_SHAPE.
+ * lda, a_cols, c_cols, bias, residual as for fp6m_mul_fused (a_cols is how arbitrary input channels reach the tail).
+ */
+int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+                  void* workspace, int dev, void* stream, int sms, int max_par, int quant_rows, const int32_t* a_cols,
+                  const int32_t* c_cols, const void* bias, const void* residual);
+
 /* Minimum workspace length in 4-byte elements: n / 128 * max_par (fp6_marlin/fp6_marlin_cuda.cpp:62-63). */
 size_t fp6m_workspace_elems(int prob_n, int max_par);
 

@@ -266,6 +266,21 @@ def gen_mixed_weight(w, quant_cols=-1, group_size=-1, strict=True):
             np.concatenate([s1.reshape(-1), s2.reshape(-1)]))
 
 
+def gen_row_mix_weight(w, quant_rows):
+    """Operands of the row-mixed GEMM (no counterpart in the reference; a composition of its harness routines):
+    rows [0, k - quant_rows) through gen_int4_weight with 128-row groups (test.py:85-121), the last quant_rows
+    rows through gen_fp6_weight (test.py:13-58), both over all n columns.
+    B = INT4 words || FP6 words, s = INT4 group scales || FP6 scales, w_ref = the two check weights stacked."""
+    k, n = w.shape
+    k4 = k - quant_rows
+    assert 0 < k4 < k and k4 % 128 == 0 and quant_rows % 64 == 0 and n % 128 == 0
+    r1, b1, s1 = gen_int4_weight(np.ascontiguousarray(w[:k4]), 128)
+    r2, b2, s2 = gen_fp6_weight(np.ascontiguousarray(w[k4:]), False)
+    return (np.ascontiguousarray(np.concatenate([r1, r2], axis=0)),
+            np.concatenate([b1.reshape(-1), b2.reshape(-1)]),
+            np.concatenate([s1.reshape(-1), s2.reshape(-1)]))
+
+
 def matmul_ref(a, w_ref):
     """test.py:165-167 in fp32 (fp16 inputs are exact in fp32; fp64 accumulate)."""
     return (np.asarray(a, dtype=np.float64) @ np.asarray(w_ref, dtype=np.float64)).astype(np.float32)
