@@ -338,6 +338,54 @@ int fp6m_permute_scales(const uint16_t* in, uint16_t* out, size_t n)
     return FP6M_OK;
 }
 
+namespace {
+
+// One plane (rows x cols weights, `words` 32-bit words per lane and k-block) between the reference's granule order
+// [k-block][64-column group][owner 4 l + i] and the gfx950 one [tile][k-block][lane 16 i + 8 sigma + l].
+void repack_plane(const uint32_t* in, uint32_t* out, size_t rows, size_t cols, int words, bool to_gfx950)
+{
+    const size_t kblocks = rows / 16, tiles = cols / 128;
+    parallel_chunks(kblocks, 1, [=](size_t kb0, size_t kb1) {
+        for (size_t kb = kb0; kb < kb1; kb++)
+            for (size_t t = 0; t < tiles; t++)
+                for (int lane = 0; lane < 64; lane++) {
+                    const int i = lane >> 4, sigma = (lane >> 3) & 1, l = lane & 7;
+                    const size_t ref = ((kb * (cols / 64) + 2 * t + sigma) * 32 + 4 * l + i) * words;
+                    const size_t nat = ((t * kblocks + kb) * 64 + lane) * words;
+                    for (int w = 0; w < words; w++) {
+                        if (to_gfx950) out[nat + w] = in[ref + w];
+                        else out[ref + w] = in[nat + w];
+                    }
+                }
+    });
+}
+
+}  // namespace
+
+int fp6m_repack_gfx950(const int32_t* in, int32_t* out, size_t k, size_t n, int quant_cols, int quant_rows, int to_gfx950)
+{
+    if (!in || !out || in == out) return FP6M_ERR_ARG;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(in);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(out);
+    size_t rows4, cols4, rows6, cols6;                                // the INT4 block and the FP6 block
+    if (quant_rows > 0) {
+        if ((size_t)quant_rows >= k) return FP6M_ERR_ARG;
+        rows4 = k - (size_t)quant_rows, cols4 = n, rows6 = (size_t)quant_rows, cols6 = n;
+    } else {
+        const size_t qc = quant_cols <= 0 ? 0 : (size_t)quant_cols;
+        if (qc > n) return FP6M_ERR_ARG;
+        rows4 = k, cols4 = n - qc, rows6 = k, cols6 = qc;
+    }
+    if (rows4 % 16 || rows6 % 16 || cols4 % 128 || cols6 % 128) return FP6M_ERR_SHAPE;
+    const size_t words4 = rows4 * cols4 / 8, words2 = rows6 * cols6 / 16;
+    if (cols4) repack_plane(src, dst, rows4, cols4, 4, to_gfx950 != 0);
+    if (cols6) {
+        repack_plane(src + words4, dst + words4, rows6, cols6, 2, to_gfx950 != 0);
+        repack_plane(src + words4 + words2, dst + words4 + words2, rows6, cols6, 4, to_gfx950 != 0);
+    }
+    return FP6M_OK;
+}
+
 int fp6m_unpack_to_fp16(const int32_t* B, const uint16_t* s, uint16_t* w_ref, size_t k, size_t n,
                         int quant_cols, int group_size)
 {

@@ -60,6 +60,9 @@ struct GemmArgs {
     // row mix (fp6m_mul_rows): rows [0, k4) of every column are INT4 with group scales, rows [k4, k) FP6.  The
     // k slices of a tile (parts x waves) are numbered INT4 first: slices [0, slices4) cover the INT4 rows.
     int k4, slices4;          // 0 = column mix
+    // weight planes in the gfx950 order (fp6m_repack_gfx950): [tile][k-block][MFMA lane] instead of the reference's
+    // [k-block][64-column group][fragment owner]
+    int native;
     // optional epilogue work (fp6m_mul_fused); `fused` is set when any of the three is
     const int32_t* c_cols;    // column of C that packed column j goes to
     const uint16_t* bias;     // fp16 [n], indexed by C column
@@ -151,6 +154,31 @@ __device__ __forceinline__ void row_mix_slice(const GemmArgs& p, int sl, int nsl
         end = (int)((long long)units * (s6 + 1) / n6) * 2;
         ti.a_step0 = p.k4 / 32;
     }
+}
+
+// Where a tile's packed words sit.  Reference order: a k-block (16 rows of k) is one row of region_n * 8 bytes
+// (4-bit plane / INT4; half that for the 2-bit plane) in which the tile owns 1 KiB (512 B), lane granules in
+// fragment-owner order.  gfx950 order: the tile's k-blocks follow each other, lane granules in MFMA lane order.
+struct PlaneGeometry {
+    size_t row4, row2;       // bytes from one k-block of the tile to the next
+    size_t tile4, tile2;     // byte offset of the tile's first k-block
+};
+__device__ __forceinline__ PlaneGeometry plane_geometry(const GemmArgs& p, const TileInfo& ti)
+{
+    PlaneGeometry g;
+    if (p.native) {
+        const size_t kblocks = (size_t)(p.k4 ? (ti.fp6 ? p.k - p.k4 : p.k4) : p.k) / 16;
+        g.row4 = 1024;
+        g.row2 = 512;
+        g.tile4 = (size_t)ti.tcol * kblocks * 1024;
+        g.tile2 = (size_t)ti.tcol * kblocks * 512;
+    } else {
+        g.row4 = (size_t)ti.region_n * 8;
+        g.row2 = (size_t)ti.region_n * 4;
+        g.tile4 = (size_t)ti.tcol * 1024;
+        g.tile2 = (size_t)ti.tcol * 512;
+    }
+    return g;
 }
 
 __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
@@ -334,12 +362,13 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     // ---- fetch side (lane = position in the slot).  Uniform 64-bit bases advance on the scalar unit;
     // each lane only contributes a constant 32-bit offset.
     const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
-    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const PlaneGeometry geo = plane_geometry(p, ti);
+    const size_t row4 = geo.row4, row2 = geo.row2;
     const unsigned char* base4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
-                                 (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4;
+                                 geo.tile4 + (size_t)(2 * step_begin) * row4;
     const int lg = lane & 31;
     const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
-    const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + (size_t)ti.tcol * 512 +
+    const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + geo.tile2 +
                                  (size_t)(2 * step_begin) * row2;
     const int a_m = lane >> 2;
     const bool a_active = a_m < AROWS && ti.mtile * 16 + a_m < p.m;
@@ -370,7 +399,7 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     };
 
     // ---- read side (lane = MFMA identity)
-    const int owner = 32 * sigma + 4 * l + i;
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;   // whose granule of the k-block this lane needs
     const uint32_t ring_lds = lds_addr(ring);
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
     const int gr2 = owner >> 1;
@@ -826,14 +855,16 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     // scalar base, so that the lane offsets stay non-negative.  The FP6 2-bit plane (8 bytes per lane and
     // k-block, already in owner order in memory) skips LDS: it is loaded into registers two steps ahead,
     // alternating between two register sets, which keeps an FP6 slot as small as an INT4 one.
-    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const PlaneGeometry geo = plane_geometry(p, ti);
+    const size_t row4 = geo.row4, row2 = geo.row2;
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;      // whose granule of the k-block this lane needs
     const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
     const uint32_t v4b = v4 + (uint32_t)row4 - 1024;
     const unsigned char* base4 = uniform_ptr(reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
-                                             (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4);
-    const uint32_t v2 = (uint32_t)(32 * sigma + 4 * l + i) * 8, v2b = v2 + (uint32_t)row2;
+                                             geo.tile4 + (size_t)(2 * step_begin) * row4);
+    const uint32_t v2 = (uint32_t)owner * 8, v2b = v2 + (uint32_t)row2;
     const unsigned char* base2 = uniform_ptr(reinterpret_cast<const unsigned char*>(p.b_fp6_2) +
-                                             (size_t)ti.tcol * 512 + (size_t)(2 * step_begin) * row2);
+                                             geo.tile2 + (size_t)(2 * step_begin) * row2);
     u2 tq[2][2];                                          // [register set][k-block]
     const int a_m = lane >> 2;
     const int tile_row0 = ti.mtile * 16 * MB;
@@ -880,7 +911,6 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     };
 
     // ---- read side
-    const int owner = 32 * sigma + 4 * l + i;
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
     uint32_t rda[4];
 #pragma unroll
@@ -1276,15 +1306,16 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
 
     // ---- fetch side: wave 0 and 1 of the slice fetch the two k-blocks of the words, wave 2 the 2-bit plane,
     // wave 3 the group scales; every wave its own four blocks of A
-    const size_t row4 = (size_t)ti.region_n * 8, row2 = (size_t)ti.region_n * 4;
+    const PlaneGeometry geo = plane_geometry(p, ti);
+    const size_t row4 = geo.row4, row2 = geo.row2;
     const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
     const uint32_t v4b = v4 + (uint32_t)row4 - 1024;
     const unsigned char* base4 = uniform_ptr(reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
-                                             (size_t)ti.tcol * 1024 + (size_t)(2 * step_begin) * row4);
+                                             geo.tile4 + (size_t)(2 * step_begin) * row4);
     const int lg = lane & 31;
     const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
     const unsigned char* base2 = uniform_ptr(reinterpret_cast<const unsigned char*>(p.b_fp6_2) +
-                                             (size_t)ti.tcol * 512 + (size_t)(2 * step_begin) * row2);
+                                             geo.tile2 + (size_t)(2 * step_begin) * row2);
     const int a_m = lane >> 2;
     const int tile_row0 = ti.mtile * 16 * MB;
     uint32_t va[MB];
@@ -1342,7 +1373,7 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
     };
 
     // ---- read side
-    const int owner = 32 * sigma + 4 * l + i;
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;      // whose granule of the k-block this lane needs
     const uint32_t rd4 = slice_lds + w_off + (owner ^ ((owner >> 4) & 3)) * 16 + 4 * j;
     const int gr2 = owner >> 1;
     const uint32_t rd2 = slice_lds + w_off + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8 + 4 * (j >> 1);
@@ -1709,6 +1740,7 @@ struct Fusion {
     const uint16_t* bias = nullptr;
     const uint16_t* residual = nullptr;
     int quant_rows = 0;              // > 0: row mix (fp6m_mul_rows), the last quant_rows rows of k are FP6
+    bool native = false;             // weight planes in the gfx950 order (FP6M_LAYOUT_GFX950)
 };
 
 int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
@@ -1779,6 +1811,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         a.qc = prob_n;
         a.k4 = k4;
     }
+    a.native = fu.native;
     a.c_cols = fu.c_cols;
     a.bias = fu.bias;
     a.residual = nullptr;
@@ -1951,9 +1984,11 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
 
 int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
                    void* workspace, int dev, void* stream, int sms, int max_par, int quant_cols, int group_size,
-                   const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual)
+                   const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual, int flags)
 {
     fp6m::Fusion fu;
+    if (flags & ~FP6M_LAYOUT_GFX950) return FP6M_ERR_ARG;
+    fu.native = (flags & FP6M_LAYOUT_GFX950) != 0;
     fu.a_cols = a_cols;
     fu.lda = lda;
     fu.c_cols = c_cols;
@@ -1966,9 +2001,11 @@ int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s
 
 int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
                   void* workspace, int dev, void* stream, int sms, int max_par, int quant_rows, const int32_t* a_cols,
-                  const int32_t* c_cols, const void* bias, const void* residual)
+                  const int32_t* c_cols, const void* bias, const void* residual, int flags)
 {
     fp6m::Fusion fu;
+    if (flags & ~FP6M_LAYOUT_GFX950) return FP6M_ERR_ARG;
+    fu.native = (flags & FP6M_LAYOUT_GFX950) != 0;
     fu.a_cols = a_cols;
     fu.lda = lda;
     fu.c_cols = c_cols;

@@ -34,8 +34,10 @@ lib.fp6m_workspace_elems.argtypes = [_int, _int]
 lib.fp6m_init.argtypes = [_int]
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
 lib.fp6m_mul_fused.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _vp, _vp,
-                               _vp, _vp]
-lib.fp6m_mul_rows.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _vp, _vp, _vp, _vp]
+                               _vp, _vp, _int]
+lib.fp6m_repack_gfx950.argtypes = [_vp, _vp, _sz, _sz, _int, _int, _int]
+lib.fp6m_mul_rows.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _vp, _vp, _vp, _vp,
+                              _int]
 lib.fp6m_fp6_quantize.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_fp6_prepack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_fp6_dequant.argtypes = [_vp, _vp, _sz, _sz, _vp]
@@ -43,7 +45,7 @@ lib.fp6m_int4_quantize.argtypes = [_vp, _sz, _sz, _int, _vp, _vp, _vp]
 lib.fp6m_int4_pack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_permute_scales.argtypes = [_vp, _vp, _sz]
 lib.fp6m_unpack_to_fp16.argtypes = [_vp, _vp, _vp, _sz, _sz, _int, _int]
-for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
+for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_repack_gfx950, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
            lib.fp6m_int4_quantize, lib.fp6m_int4_pack, lib.fp6m_permute_scales, lib.fp6m_unpack_to_fp16):
     _f.restype = _int
 
@@ -239,7 +241,14 @@ def check_column_map(cols, size, permutation=False):
     return cols
 
 
-def _mul_extended(A, B, C, s, workspace, quant_cols, group_size, quant_rows, a_cols, c_cols, bias, residual, sms, max_par):
+LAYOUT_GFX950 = 1
+
+
+def _mul_extended(A, B, C, s, workspace, quant_cols, group_size, quant_rows, a_cols, c_cols, bias, residual, sms, max_par,
+                  layout="reference"):
+    if layout not in ("reference", "gfx950"):
+        raise ValueError("layout must be 'reference' or 'gfx950'")
+    flags = LAYOUT_GFX950 if layout == "gfx950" else 0
     tensors = [("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)]
     tensors += [(nm, t) for nm, t in (("a_cols", a_cols), ("c_cols", c_cols), ("bias", bias), ("residual", residual))
                 if t is not None]
@@ -291,12 +300,12 @@ def _mul_extended(A, B, C, s, workspace, quant_cols, group_size, quant_rows, a_c
             name = "fp6m_mul_rows"
             code = lib.fp6m_mul_rows(A.data_ptr(), lda, B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k,
                                      workspace.data_ptr(), A.device.index, stream, sms, max_par, quant_rows,
-                                     ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual))
+                                     ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual), flags)
         else:
             name = "fp6m_mul_fused"
             code = lib.fp6m_mul_fused(A.data_ptr(), lda, B.data_ptr(), C.data_ptr(), s.data_ptr(), m, n, k,
                                       workspace.data_ptr(), A.device.index, stream, sms, max_par, quant_cols, group_size,
-                                      ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual))
+                                      ptr(a_cols), ptr(c_cols), ptr(bias), ptr(residual), flags)
     if code == ERR_PROB_SHAPE:
         raise RuntimeError(f"Problem (m={m}, n={n}, k={k}) not compatible with the tile shape.")
     if code != OK:
@@ -304,18 +313,20 @@ def _mul_extended(A, B, C, s, workspace, quant_cols, group_size, quant_rows, a_c
 
 
 def mul_fused(A, B, C, s, workspace, quant_cols=-1, group_size=-1, a_cols=None, c_cols=None, bias=None, residual=None,
-              sms=-1, max_par=16):
+              sms=-1, max_par=16, layout="reference"):
     """`mul` with the reorders and additions around it folded into the launch (no counterpart in the reference,
     whose harness leaves them to the caller: the FP6 columns of its packed weight sit at the tail, test.py:123-152):
 
         C[:, c_cols] = fp16(A[:, a_cols] @ dequant(B) * s + bias[c_cols] + residual[:, c_cols])
 
     a_cols int32 [k] (columns of A, which may then be wider than k), c_cols int32 [n] permutation, bias float16 [n],
-    residual float16 [m, n] (may be C).  Maps are trusted here: run `check_column_map` on them once."""
-    _mul_extended(A, B, C, s, workspace, quant_cols, group_size, 0, a_cols, c_cols, bias, residual, sms, max_par)
+    residual float16 [m, n] (may be C).  Maps are trusted here: run `check_column_map` on them once.
+    layout="gfx950": B went through `repack_gfx950`."""
+    _mul_extended(A, B, C, s, workspace, quant_cols, group_size, 0, a_cols, c_cols, bias, residual, sms, max_par, layout)
 
 
-def mul_rows(A, B, C, s, workspace, quant_rows, a_cols=None, c_cols=None, bias=None, residual=None, sms=-1, max_par=16):
+def mul_rows(A, B, C, s, workspace, quant_rows, a_cols=None, c_cols=None, bias=None, residual=None, sms=-1, max_par=16,
+             layout="reference"):
     """The GEMM for a weight mixed along k instead of n: the last `quant_rows` rows (input channels) of every
     column are FP6 with one scale per column, the rows before them INT4 with one scale per 128 rows and column.
     Both segments of a column tile accumulate into the same output tile inside one launch.  (The reference mixes
@@ -328,4 +339,53 @@ def mul_rows(A, B, C, s, workspace, quant_rows, a_cols=None, c_cols=None, bias=N
     `mul_fused`; `a_cols` is how arbitrary input channels get to the FP6 tail."""
     if int(quant_rows) <= 0:
         raise RuntimeError("quant_rows must be positive and below k")
-    _mul_extended(A, B, C, s, workspace, -1, 128, int(quant_rows), a_cols, c_cols, bias, residual, sms, max_par)
+    _mul_extended(A, B, C, s, workspace, -1, 128, int(quant_rows), a_cols, c_cols, bias, residual, sms, max_par, layout)
+
+
+def _plane_views(B, k, n, quant_cols, quant_rows):
+    """(offset, rows, cols, words per lane) of the planes inside a B buffer."""
+    if quant_rows:
+        rows4, cols4, rows6, cols6 = k - quant_rows, n, quant_rows, n
+    else:
+        qc = 0 if quant_cols in (-1, 0) else quant_cols
+        rows4, cols4, rows6, cols6 = k, n - qc, k, qc
+    if rows4 <= 0 or rows4 % 16 or rows6 % 16 or cols4 % 128 or cols6 % 128 or cols4 < 0:
+        raise ValueError("regions must have whole 128-column tiles and 16-row k-blocks")
+    words4, words2 = rows4 * cols4 // 8, rows6 * cols6 // 16
+    if B.numel() != words4 + 3 * words2:
+        raise ValueError(f"B must hold {words4 + 3 * words2} words")
+    planes = [(0, rows4, cols4, 4)] if cols4 else []
+    if cols6:
+        planes += [(words4, rows6, cols6, 2), (words4 + words2, rows6, cols6, 4)]
+    return planes
+
+
+def repack_gfx950(B, k, n, quant_cols=-1, quant_rows=0, to_gfx950=True):
+    """Reorder the packed words of `B` (int32 1-D, on any device) between the reference's order and the gfx950
+    one, in which every 128-column tile is one sequential stream in MFMA lane order (see fp6m_repack_gfx950 in
+    include/fp6m.h, which this mirrors with tensor permutes so that it runs where the tensor lives).  Lossless;
+    `to_gfx950=False` is the inverse.  Scales do not change."""
+    if B.dtype != torch.int32 or B.dim() != 1:
+        raise ValueError("B must be a 1-D int32 tensor")
+    out = torch.empty_like(B)
+    for off, rows, cols, words in _plane_views(B, k, n, quant_cols, quant_rows):
+        size = rows * cols // 32 * words
+        kb, tiles = rows // 16, cols // 128
+        src = B[off:off + size]
+        if to_gfx950:        # [kb][tile][sigma][l][i][w] -> [tile][kb][i][sigma][l][w]
+            out[off:off + size] = src.view(kb, tiles, 2, 8, 4, words).permute(1, 0, 4, 2, 3, 5).reshape(-1)
+        else:
+            out[off:off + size] = src.view(tiles, kb, 4, 2, 8, words).permute(1, 0, 3, 4, 2, 5).reshape(-1)
+    return out
+
+
+def repack_gfx950_host(B, k, n, quant_cols=-1, quant_rows=0, to_gfx950=True):
+    """The same conversion through the C ABI's host routine (CPU tensors)."""
+    if B.dtype != torch.int32 or B.dim() != 1 or B.is_cuda:
+        raise ValueError("B must be a 1-D int32 CPU tensor")
+    B = B.contiguous()
+    out = torch.empty_like(B)
+    _plane_views(B, k, n, quant_cols, quant_rows)
+    qc = 0 if quant_cols in (-1, 0) else quant_cols
+    _raise_cpu(lib.fp6m_repack_gfx950(B.data_ptr(), out.data_ptr(), k, n, qc, quant_rows, int(bool(to_gfx950))))
+    return out

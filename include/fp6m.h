@@ -74,6 +74,21 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
              int quant_cols, int group_size);
 
 /*
+ * The packed words in the order this GPU's kernels would choose, next to the reference's.  Same bits; what moves is
+ * the 16-byte (4-bit plane, INT4 words) or 8-byte (2-bit plane) granule that one lane consumes per k-block of 16 rows:
+ *   reference  [k-block][64-column group g][fragment owner t = 4 l + i]          (weight_prepacking.cpp:123-177,
+ *              test.py:60-79: mma.m16n8k16 lane order, a tile's k-blocks a whole matrix row apart)
+ *   gfx950     [128-column tile][k-block][MFMA lane 16 i + 8 (g & 1) + l]        (v_mfma_f32_16x16x32_f16 operand
+ *              order: a tile's packed words form one sequential stream and lanes read them in lane order)
+ * fp6m_repack_gfx950 converts a whole B buffer (INT4 words || FP6 2-bit plane || FP6 4-bit plane; the column mix of
+ * fp6m_mul when quant_rows == 0, else the row mix of fp6m_mul_rows with quant_cols ignored) either way on the host;
+ * to_gfx950 = 0 is the exact inverse.  Scales are not affected.  Column counts of each region must be multiples of 128,
+ * row counts multiples of 16 -> else FP6M_ERR_SHAPE.  in and out must not overlap.
+ */
+#define FP6M_LAYOUT_GFX950 1
+int fp6m_repack_gfx950(const int32_t* in, int32_t* out, size_t k, size_t n, int quant_cols, int quant_rows, int to_gfx950);
+
+/*
  * The GEMM with the reordering and the additions around it folded in.  No counterpart in the reference: its
  * harness packs a weight whose FP6 columns already sit at the tail (gen_mixed_weight, test.py:123-152) and
  * leaves the matching reorder of the output columns (and, for selected input channels, of the activations) and
@@ -90,10 +105,11 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
  *   fp32 and the result is rounded once.  With all four NULL the result equals fp6m_mul's bit for bit.
  * Map entries out of range are clamped on the device (wrong values, no fault); validate maps once on the host.
  * Other arguments as for fp6m_mul (tile shapes are always automatic).
+ *   flags     0, or FP6M_LAYOUT_GFX950 when B went through fp6m_repack_gfx950.
  */
 int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
                    void* workspace, int dev, void* stream, int sms, int max_par, int quant_cols, int group_size,
-                   const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual);
+                   const int32_t* a_cols, const int32_t* c_cols, const void* bias, const void* residual, int flags);
 
 /*
  * The GEMM for a weight mixed along k instead of n: the last quant_rows rows (input channels) of every column are
@@ -106,11 +122,12 @@ int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s
  *   s   INT4 scales [(prob_k - quant_rows) / 128, n] in natural column order || FP6 scales [n] in the permuted
  *       order of fp6m_permute_scales
  * (prob_k - quant_rows) % 128, quant_rows % 64 or prob_n % 128 != 0 -> FP6M_ERR_PROB_SHAPE.
- * lda, a_cols, c_cols, bias, residual as for fp6m_mul_fused (a_cols is how arbitrary input channels reach the tail).
+ * lda, a_cols, c_cols, bias, residual, flags as for fp6m_mul_fused (a_cols is how arbitrary input channels reach the
+ * tail).
  */
 int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
                   void* workspace, int dev, void* stream, int sms, int max_par, int quant_rows, const int32_t* a_cols,
-                  const int32_t* c_cols, const void* bias, const void* residual);
+                  const int32_t* c_cols, const void* bias, const void* residual, int flags);
 
 /* Minimum workspace length in 4-byte elements: n / 128 * max_par (fp6_marlin/fp6_marlin_cuda.cpp:62-63). */
 size_t fp6m_workspace_elems(int prob_n, int max_par);
