@@ -67,6 +67,10 @@ class Problem:
     def run(self, mul):
         mul(self.A, self.B, self.C, self.s, self.ws, self.qc if self.qc else -1, -1, -1, -1, 16, self.gs)
 
+    def run_gfx950(self, mul_fused):
+        """The same words read in the gfx950 order (random bits either way: the timing is what matters here)."""
+        mul_fused(self.A, self.B, self.C, self.s, self.ws, self.qc if self.qc else -1, self.gs, layout="gfx950")
+
     def run_fp16(self, torch):
         torch.matmul(self.A, self.W16, out=self.C)
 
@@ -218,7 +222,7 @@ def traffic_probe():
           [p.bytes for p in probs[0]], flush=True)
 
 
-def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100):
+def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100, layout="reference"):
     """One (m, k, n) GEMM against fp16 torch.matmul (hipBLASLt), both replayed from HIP graphs that walk
     over > 512 MB of distinct weights."""
     nbytes = weight_bytes(k, n, qc, gs)
@@ -228,7 +232,10 @@ def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100
            for _ in range(max(2, min(copies, int(640e6 // (2 * k * n)) + 1)))]
 
     def f(i):
-        probs[i % copies].run(fp6_marlin.mul)
+        if layout == "gfx950":
+            probs[i % copies].run_gfx950(fp6_marlin.mul_fused)
+        else:
+            probs[i % copies].run(fp6_marlin.mul)
 
     def f16(i):
         torch.matmul(probs[0].A, w16[i % len(w16)], out=probs[0].C)
@@ -243,7 +250,7 @@ def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100
     fn16, calls16 = graphed(torch, f16, len(w16), iters16)
     _, ev16 = time_region(torch, fn16, calls16)
     t, t16 = ev / iters, ev16 / iters16
-    row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "us": round(t * 1e6, 2),
+    row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "layout": layout, "us": round(t * 1e6, 2),
            "weight_GBs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
            "TFLOPs": round(2 * m * k * n / t / 1e12, 2), "mfma_frac": round(2 * m * k * n / t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
            "fp16_us": round(t16 * 1e6, 2), "speedup_vs_fp16": round(t16 / t, 2)}
@@ -260,7 +267,7 @@ def one_shape(args):
     m, k, n = v[:3]
     qc, gs = (v[3] if len(v) > 3 else 256), (v[4] if len(v) > 4 else 128)
     fp6_marlin.init(0)
-    row = measure_shape(torch, fp6_marlin, torch.Generator().manual_seed(0), "shape", m, k, n, qc, gs)
+    row = measure_shape(torch, fp6_marlin, torch.Generator().manual_seed(0), "shape", m, k, n, qc, gs, layout=args.layout)
     bound = "mfma" if m >= 128 else "hbm"
     row["roofline"] = ({"bound": "mfma", "achieved": row["TFLOPs"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": row["mfma_frac"]} if bound == "mfma" else
@@ -430,6 +437,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", type=str, default=None, help="write the per-shape table of all configs to this file")
     ap.add_argument("--shape", type=str, default=None, help="m,k,n[,quant_cols,group_size]: measure one shape")
+    ap.add_argument("--layout", type=str, default="reference", choices=["reference", "gfx950"],
+                    help="word order of the packed weight for --shape (gfx950: after repack_gfx950)")
     ap.add_argument("--fused", type=str, default=None, help="m,k,n[,quant_cols,group_size]: time mul_fused against mul + torch kernels")
     ap.add_argument("--rows", type=str, default=None, help="m,k,n[,quant_rows]: time the row-mixed GEMM against two mul calls and an addition")
     ap.add_argument("--pack", type=str, default=None, help="k,n[,quant_cols,group_size]: time the on-GPU weight packer")
