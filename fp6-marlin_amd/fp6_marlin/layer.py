@@ -104,49 +104,99 @@ def pack_row_mix_weight(w, quant_rows):
 
 
 class Layer(nn.Module):
-    """Linear layer ``y = x @ W`` with W [infeatures, outfeatures] stored as mixed INT4 / FP6.
+    """Linear layer ``y = x @ W (+ bias)`` with W [infeatures, outfeatures] stored as mixed INT4 / FP6.
 
-    Buffers (all on the module's device):
+    Buffers (all on the module's device; ``B``, ``s``, ``meta`` and, if used, ``c_cols`` / ``bias`` are saved):
       ``B``          int32 1-D, the wire format of ``mul``
       ``s``          float16 1-D: INT4 scales (per column in the reference's permuted order, or
                      [infeatures/128, outfeatures-quant_cols] in natural column order when
                      ``groupsize=128``) followed by the FP6 per-column scales (permuted order)
-      ``workspace``  int32 zeros, outfeatures // 128 * 16
+      ``meta``       int32 [6]: format version, infeatures, outfeatures, quant_cols, groupsize, word order
+                     (0 reference, 1 gfx950); a checkpoint whose ``meta`` differs from the layer's is refused
+      ``workspace``  int32 zeros, outfeatures // 128 * 16 (not saved)
 
-    ``quant_cols`` output features, the *last* ones, are kept in FP6.  To protect arbitrary "significant"
-    output channels, permute the columns of W so they come last (and un-permute y).
+    Which output features are kept in FP6: by default the *last* ``quant_cols`` ones (what the reference's
+    harness does after moving its chosen columns to the tail, test.py:123-152).  With ``fp6_channels`` (indices
+    of ``quant_cols`` output features) ``pack`` moves those columns to the tail itself and ``forward`` writes
+    every result column back to its own place inside the GEMM (``mul_fused``), so callers see W's own order.
+    ``layout="gfx950"`` stores the packed words as per-tile sequential streams (``repack_gfx950``).
     """
 
-    def __init__(self, infeatures, outfeatures, groupsize=-1, quant_cols=-1):
+    FORMAT_VERSION = 1
+
+    def __init__(self, infeatures, outfeatures, groupsize=-1, quant_cols=-1, fp6_channels=None, bias=False,
+                 layout="reference"):
         super().__init__()
         if groupsize not in (-1, 128):
             raise ValueError("Only groupsize -1 and 128 are supported.")
+        if layout not in ("reference", "gfx950"):
+            raise ValueError("layout must be 'reference' or 'gfx950'")
         qc = 0 if quant_cols in (-1, 0) else quant_cols
         if infeatures % 128 or outfeatures % 128 or qc % 128 or qc > outfeatures:
             raise ValueError("infeatures, outfeatures and quant_cols must be multiples of 128")
-        self.k, self.n, self.groupsize, self.quant_cols = infeatures, outfeatures, groupsize, quant_cols
+        self.k, self.n, self.groupsize, self.quant_cols, self.layout = infeatures, outfeatures, groupsize, quant_cols, layout
         n4 = outfeatures - qc
         words = infeatures * n4 // 8 + infeatures * qc * 3 // 16
         nscale = (n4 if groupsize == -1 else infeatures // 128 * n4) + qc
         self.register_buffer("B", torch.empty(words, dtype=torch.int32))
         self.register_buffer("s", torch.empty(nscale, dtype=torch.float16))
+        self.register_buffer("meta", torch.tensor([self.FORMAT_VERSION, infeatures, outfeatures, qc, groupsize,
+                                                   int(layout == "gfx950")], dtype=torch.int32))
         self.register_buffer("workspace", torch.zeros(outfeatures // 128 * 16, dtype=torch.int32), persistent=False)
+        if fp6_channels is not None:
+            picked = torch.as_tensor(fp6_channels, dtype=torch.int64).reshape(-1)
+            if picked.numel() != qc or picked.unique().numel() != qc or (qc and (picked.min() < 0 or picked.max() >= outfeatures)):
+                raise ValueError("fp6_channels must name quant_cols distinct output features")
+            keep = torch.ones(outfeatures, dtype=torch.bool)
+            keep[picked] = False
+            # packed column j holds output feature c_cols[j]: the others in order, then the chosen ones
+            self.register_buffer("c_cols", torch.cat([torch.nonzero(keep).reshape(-1), picked]).to(torch.int32))
+        else:
+            self.c_cols = None
+        if bias:
+            self.register_buffer("bias", torch.zeros(outfeatures, dtype=torch.float16))
+        else:
+            self.bias = None
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        meta = state_dict.get(prefix + "meta")
+        if meta is not None and not torch.equal(meta.cpu().to(torch.int32), self.meta.cpu()):
+            raise RuntimeError(f"{prefix}: checkpoint format {meta.tolist()} does not match this layer {self.meta.tolist()} "
+                               "(version, infeatures, outfeatures, quant_cols, groupsize, word order)")
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def pack(self, linear):
         """Quantise and pack ``linear`` (an ``nn.Linear`` or a float16 weight [outfeatures, infeatures]).
         A weight that lives on a GPU is packed there (70B-size layers take milliseconds instead of the host
-        packer's seconds); the result is the same bit for bit."""
+        packer's seconds); the result is the same bit for bit.  Returns the dequantised weight [k, n] in W's own
+        column order."""
         w = linear.weight.data if isinstance(linear, nn.Module) else linear
         w = w.detach().to(torch.float16).t().contiguous()            # [k, n], on the weight's device
         if tuple(w.shape) != (self.k, self.n):
             raise ValueError("weight shape does not match the layer")
+        if self.c_cols is not None:
+            w = w[:, self.c_cols.long().to(w.device)].contiguous()
         B, s, w_ref = pack_mixed_weight(w, self.quant_cols, self.groupsize, harness_layout=False)
+        if self.layout == "gfx950":
+            B = cabi.repack_gfx950(B, self.k, self.n, self.quant_cols)
         self.B.copy_(B)
         self.s.copy_(s)
+        if self.bias is not None and isinstance(linear, nn.Module) and getattr(linear, "bias", None) is not None:
+            self.bias.copy_(linear.bias.data.detach().to(torch.float16))
+        if self.c_cols is not None:
+            own = torch.empty_like(w_ref)
+            own[:, self.c_cols.long().to(w_ref.device)] = w_ref
+            w_ref = own
         return w_ref
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """y = x @ W (+ bias) (+ residual, float16 of y's shape), as one GEMM call."""
         x2 = x.reshape(-1, x.shape[-1]).to(torch.float16).contiguous()
         out = torch.empty((x2.shape[0], self.n), dtype=torch.float16, device=x2.device)
-        cabi.mul(x2, self.B, out, self.s, self.workspace, self.quant_cols, -1, -1, -1, 16, self.groupsize)
+        if self.c_cols is None and self.bias is None and residual is None and self.layout == "reference":
+            cabi.mul(x2, self.B, out, self.s, self.workspace, self.quant_cols, -1, -1, -1, 16, self.groupsize)
+        else:
+            res = None if residual is None else residual.reshape(-1, self.n).to(torch.float16).contiguous()
+            cabi.mul_fused(x2, self.B, out, self.s, self.workspace, self.quant_cols, self.groupsize, c_cols=self.c_cols,
+                           bias=self.bias, residual=res, layout=self.layout)
         return out.reshape(x.shape[:-1] + (self.n,))

@@ -265,3 +265,34 @@ def test_layer_forward(oracle):
     assert y.shape == (2, 5, 768)
     y_ref = (x.reshape(-1, 1024).float() @ w_ref.float()).reshape(2, 5, 768)
     assert oracle.rel_err(y.numpy(), y_ref.numpy()) <= TOL
+
+
+def test_layer_with_chosen_fp6_channels_bias_residual_and_checkpoint(oracle):
+    """FP6 on arbitrary output features, results in the linear layer's own order, bias and residual in the call,
+    both word orders; state_dict round trip and the refusal of a checkpoint of another format."""
+    import fp6_marlin
+    torch.manual_seed(2)
+    k, n, qc = 512, 768, 128
+    lin = torch.nn.Linear(k, n, bias=True).half()
+    picked = torch.randperm(n)[:qc]
+    x = torch.randn((3, 4, k), dtype=torch.half)
+    res = torch.randn((3, 4, n), dtype=torch.half)
+    outs = []
+    for layout in ("reference", "gfx950"):
+        layer = fp6_marlin.Layer(k, n, groupsize=128, quant_cols=qc, fp6_channels=picked, bias=True, layout=layout)
+        w_ref = layer.pack(lin)
+        # the check weight comes back in the linear layer's own column order (a wrong order would give ~1.4 here)
+        err = (w_ref.float() - lin.weight.data.t().float()).abs().mean(0) / lin.weight.data.t().float().abs().mean(0)
+        assert err.max() < 0.3
+        layer = layer.to(dev())
+        y = layer(x.to(dev()), residual=res.to(dev())).cpu()
+        y_ref = (x.reshape(-1, k).float() @ w_ref.float() + lin.bias.data.float()).reshape(3, 4, n) + res.float()
+        assert oracle.rel_err(y.numpy(), y_ref.numpy()) <= TOL
+        outs.append(y)
+        clone = fp6_marlin.Layer(k, n, groupsize=128, quant_cols=qc, fp6_channels=picked, bias=True, layout=layout)
+        clone.load_state_dict(layer.state_dict())
+        assert torch.equal(clone.to(dev())(x.to(dev()), residual=res.to(dev())).cpu(), y)
+        other = fp6_marlin.Layer(k, n, groupsize=-1, quant_cols=qc, fp6_channels=picked, bias=True, layout=layout)
+        with pytest.raises(RuntimeError, match="does not match"):
+            other.load_state_dict(layer.state_dict())
+    assert torch.equal(outs[0], outs[1])
