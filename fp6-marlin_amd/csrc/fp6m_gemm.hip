@@ -32,7 +32,6 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 256;        // four wavefronts
 constexpr int kWaves = 4;
 constexpr int kTileN = 128;          // columns per tile
 constexpr int kRedStride = kTileN + 4;                       // floats per row of the reduction slab
@@ -198,13 +197,13 @@ __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 
 // k range of one wave in steps of 32 (two k-blocks).  Units of two steps (four with group scales) keep
 // every wave's step count even and group-aligned.
-template <bool G128>
+template <bool G128, int WK = kWaves>
 __device__ __forceinline__ void wave_k_range(const GemmArgs& p, int part, int wave, int& begin, int& end)
 {
     constexpr int unit_steps = G128 ? 4 : 2;
     const int units = p.k / (32 * unit_steps);
-    const int nwaves = p.ksplit * kWaves;
-    const int wv = part * kWaves + wave;
+    const int nwaves = p.ksplit * WK;
+    const int wv = part * WK + wave;
     begin = (int)((long long)units * wv / nwaves) * unit_steps;
     end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
 }
@@ -1188,18 +1187,21 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
     return max3(d4 * (2048 + mb * 1024) + scale_slab_bytes(d4), d6 * (2048 + mb * 1024), 16 * kRedStride * 4);
 }
 
-template <bool G128, int MB, int D4, int D6>
-__global__ __launch_bounds__(kThreads, 2) void gemm_mb_kernel(const GemmArgs p)
+// WK = k slices (waves) per workgroup: four, or eight (one workgroup per CU, two waves per SIMD) for grids that
+// would otherwise leave every SIMD a single wave.
+template <bool G128, int MB, int D4, int D6, int WK>
+__global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
 {
     constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kWaves * kWaveLds + 16];
+    static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];
 
     FP6M_MARK(p, 0);
     TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int step_begin, step_end;
-    wave_k_range<G128>(p, ti.part, wave, step_begin, step_end);
-    if (p.k4) row_mix_slice(p, ti.part * kWaves + wave, p.ksplit * kWaves, ti, step_begin, step_end);
+    wave_k_range<G128, WK>(p, ti.part, wave, step_begin, step_end);
+    if (p.k4) row_mix_slice(p, ti.part * WK + wave, p.ksplit * WK, ti, step_begin, step_end);
 
     f4 acc[MB][8];
 #pragma unroll
@@ -1214,8 +1216,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_mb_kernel(const GemmArgs p)
             stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
     }
     FP6M_MARK(p, 2);
-    wg_finish_mb<MB>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
-                     reinterpret_cast<int*>(smem + kWaves * kWaveLds), true, p.k4 ? p.slices4 - ti.part * kWaves : kWaves);
+    wg_finish_mb<MB, WK>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+                         reinterpret_cast<int*>(smem + WK * kWaveLds), true, p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
 }
 
@@ -1693,12 +1695,19 @@ inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, d
 }
 
 template <int MB, int D4, int D6>
-void launch_mb(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
+void launch_mb(const GemmArgs& a, bool g128, int wk, dim3 grid, hipStream_t stream)
 {
-    if (g128)
-        hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6>), grid, dim3(kThreads), 0, stream, a);
-    else
-        hipLaunchKernelGGL((gemm_mb_kernel<false, MB, D4, D6>), grid, dim3(kThreads), 0, stream, a);
+    if (wk == 8) {
+        if (g128)
+            hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6, 8>), grid, dim3(512), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gemm_mb_kernel<false, MB, D4, D6, 8>), grid, dim3(512), 0, stream, a);
+    } else {
+        if (g128)
+            hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6, 4>), grid, dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gemm_mb_kernel<false, MB, D4, D6, 4>), grid, dim3(256), 0, stream, a);
+    }
 }
 
 void launch_wm(const GemmArgs& a, bool g128, int wn, dim3 grid, hipStream_t stream)
@@ -1956,13 +1965,17 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (ks < 1) ks = 1;
             while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
             a.ksplit = (int)ks;
-            if (row_mix) a.slices4 = deal_slices(a.ksplit * kWaves);
+            // A grid of at most one workgroup per CU would leave every SIMD a single wave: give the workgroup eight
+            // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
+            int wk = base * ks <= scratch->cus && units / 16 >= ks ? 8 : kWaves;
+            if (const char* e = getenv("FP6M_WK")) wk = atoi(e) == 8 ? 8 : kWaves;   // tuning/testing override
+            if (row_mix) a.slices4 = deal_slices(a.ksplit * wk);
             dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
             if (getenv("FP6M_VERBOSE"))
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d grid=%ux%u\n", a.m, prob_n, prob_k, mb, mtiles,
-                        a.ksplit, grid.x, grid.y);
-            if (mb == 2) launch_mb<2, 4, 3>(a, g128, grid, st);
-            else launch_mb<4, 3, 3>(a, g128, grid, st);
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d k slices %d grid=%ux%u\n", a.m, prob_n, prob_k,
+                        mb, mtiles, a.ksplit, wk, grid.x, grid.y);
+            if (mb == 2) launch_mb<2, 4, 3>(a, g128, wk, grid, st);
+            else launch_mb<4, 3, 3>(a, g128, wk, grid, st);
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return hip_fail(e);

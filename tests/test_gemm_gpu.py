@@ -162,6 +162,19 @@ def test_shared_fragment_kernel(oracle):
     run(oracle, 1024, 768, 1024, qc=256, gs=128)                       # default dispatch stays on the other kernel
 
 
+def test_eight_k_slices_per_workgroup(oracle):
+    """The m > 16 kernel with eight waves (k slices) per workgroup, which small grids on long k pick by themselves
+    (here: 8192 x 512 at m = 40), forced on and off on ragged shapes."""
+    for wk in (8, 4):
+        e = {"FP6M_WK": wk}
+        for m in (17, 32, 33, 64, 100, 200):
+            run(oracle, m, 512, 1024, qc=256, gs=128, env=e)
+        run(oracle, 48, 768, 512, qc=128, env=e)
+        run(oracle, 70, 256, 64, qc=-1, env=e)                          # one k unit: seven idle slices
+        run(oracle, 130, 512, 2048, qc=256, ksplit=3, env=e)
+    run(oracle, 40, 512, 8192, qc=256, gs=128)
+
+
 def test_max_par_chunks_m(oracle):
     """m-tiles beyond max_par go to further launches (fp6_marlin_cuda_kernel.cu:917-948)."""
     run(oracle, 300, 512, 512, qc=256, max_par=2)

@@ -90,5 +90,5 @@ def test_mfma_loops_keep_accumulators_in_place(asm):
                 last = n
         moved = [l for l in ins[first:last] if l.startswith("v_accvgpr")]
         assert not moved, f"{name}: accumulator copies between MFMAs: {moved[:4]}"
-    assert seen == 8        # (group scales or not) x (MB 2, 4) and x (one or two tiles per workgroup)
+    assert seen == 12       # (group scales or not) x ((MB 2, 4) x (4, 8 k slices) + (one, two tiles per workgroup))
     assert not re.findall(r"\.vgpr_spill_count:\s+[1-9]", asm), "a kernel spills VGPRs"
