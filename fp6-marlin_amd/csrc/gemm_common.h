@@ -1,0 +1,308 @@
+// Shared pieces of the GEMM kernels (fp6m_gemm.hip): argument block, tile bookkeeping, the fused store, direct-to-LDS
+// load and s_waitcnt helpers, and the register-level dequantisers.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "fp6m.h"
+#include "fp6m_layout.h"
+
+namespace fp6m {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWaves = 4;
+constexpr int kTileN = 128;          // columns per tile
+constexpr int kRedStride = kTileN + 4;                       // floats per row of the reduction slab
+constexpr size_t kScratchBytes = size_t(64) << 20;           // per-device partial-sum scratch
+constexpr size_t kPackTempBytes = size_t(1) << 20;           // + the packer's flag and per-column maxima
+
+struct GemmArgs {
+    const uint16_t* A;
+    const uint32_t* b_int4;   // INT4 words
+    const uint32_t* b_fp6_2;  // FP6 2-bit plane
+    const uint32_t* b_fp6_4;  // FP6 4-bit plane
+    uint16_t* C;
+    const uint16_t* s_int4;   // per-column (permuted order) or [k/128][n4] group scales
+    const uint16_t* s_fp6;    // per-column (permuted order)
+    float* scratch;
+    int* counters;
+    int m, n, k;
+    int n4, qc;               // columns in the INT4 / FP6 region
+    int tiles6;               // FP6 tiles come first in the tile list
+    int tiles;                // all tiles
+    int ksplit;               // workgroups per (tile, m-tile)
+    // m <= 16 kernel: the FP6 and the INT4 region are covered by separate ranges of workgroups
+    int ks6, ks4;             // k parts (workgroups) per tile group, per region
+    int groups6, groups4;     // tile groups (WN adjacent tiles) per region
+    // row mix (fp6m_mul_rows): rows [0, k4) of every column are INT4 with group scales, rows [k4, k) FP6.  The
+    // k slices of a tile (parts x waves) are numbered INT4 first: slices [0, slices4) cover the INT4 rows.
+    int k4, slices4;          // 0 = column mix
+    // weight planes in the gfx950 order (fp6m_repack_gfx950): [tile][k-block][MFMA lane] instead of the reference's
+    // [k-block][64-column group][fragment owner]
+    int native;
+    // optional epilogue work (fp6m_mul_fused); `fused` is set when any of the three is
+    const int32_t* c_cols;    // column of C that packed column j goes to
+    const uint16_t* bias;     // fp16 [n], indexed by C column
+    const uint16_t* residual; // fp16 [m, n], same rows as C
+    int fused;
+#ifdef FP6M_TIMELINE
+    unsigned long long* timeline;   // 8 realtime-clock stamps per workgroup (performance debugging builds only)
+#endif
+};
+
+#ifdef FP6M_TIMELINE
+#define FP6M_MARK(p, i)                                                                            \
+    do {                                                                                           \
+        if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0 && (p).timeline) /* uniform branch */ \
+            (p).timeline[(size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#else
+#define FP6M_MARK(p, i) do { } while (0)
+#endif
+
+// ------------------------------------------------------------------------------------------------ bit tricks
+
+__device__ __forceinline__ h2 as_h2(uint32_t v) { return __builtin_bit_cast(h2, v); }
+
+__device__ __forceinline__ h8 join(h2 a, h2 b, h2 c, h2 d)
+{
+    h8 v;
+    v[0] = a[0]; v[1] = a[1]; v[2] = b[0]; v[3] = b[1];
+    v[4] = c[0]; v[5] = c[1]; v[6] = d[0]; v[7] = d[1];
+    return v;
+}
+
+// Workgroup b of a 1-D grid runs on XCD b % 8.  Renumber so that every XCD sees a contiguous range of
+// logical ids: workgroups that share a tile (adjacent logical ids) then share an L2.
+__device__ __forceinline__ int xcd_contiguous_id(int b, int total)
+{
+    const int q = total >> 3, r = total & 7, x = b & 7;
+    return x * q + (x < r ? x : r) + (b >> 3);
+}
+
+// Epilogue of fp6m_mul_fused for two adjacent packed columns of one row: C[row, c_cols[col]] =
+// fp16(v + bias[c_cols[col]] + residual[row, c_cols[col]]), everything added in fp32 and rounded once.
+// Map entries are clamped to the row so that a bad map cannot write outside C.
+__device__ __forceinline__ void store_fused(const GemmArgs& p, size_t row, int col, float v0, float v1)
+{
+    int c0 = col, c1 = col + 1;
+    if (p.c_cols) {
+        c0 = p.c_cols[col];
+        c1 = p.c_cols[col + 1];
+        c0 = c0 < 0 ? 0 : (c0 >= p.n ? p.n - 1 : c0);
+        c1 = c1 < 0 ? 0 : (c1 >= p.n ? p.n - 1 : c1);
+    }
+    if (p.bias) {
+        v0 += (float)__builtin_bit_cast(_Float16, p.bias[c0]);
+        v1 += (float)__builtin_bit_cast(_Float16, p.bias[c1]);
+    }
+    const size_t r = row * (size_t)p.n;
+    if (p.residual) {
+        v0 += (float)__builtin_bit_cast(_Float16, p.residual[r + c0]);
+        v1 += (float)__builtin_bit_cast(_Float16, p.residual[r + c1]);
+    }
+    p.C[r + c0] = __builtin_bit_cast(uint16_t, (_Float16)v0);
+    p.C[r + c1] = __builtin_bit_cast(uint16_t, (_Float16)v1);
+}
+
+// ------------------------------------------------------------------------------------------------ tile bookkeeping
+
+struct TileInfo {
+    int tile, part, mtile;   // tile in the [FP6 | INT4] tile list, k partner index, m-tile
+    bool fp6;
+    int tcol;                // tile index inside its region
+    int region_n;            // columns of the region
+    int col0;                // first column of the tile in C
+    int a_step0;             // k step of A that step 0 of the wave's weight segment multiplies (row mix: k4 / 32)
+};
+
+// Row mix: slice `sl` of the `nsl` slices of a tile -> its segment (ti.fp6, ti.a_step0) and its steps there.
+__device__ __forceinline__ void row_mix_slice(const GemmArgs& p, int sl, int nsl, TileInfo& ti, int& begin, int& end)
+{
+    ti.fp6 = sl >= p.slices4;
+    if (!ti.fp6) {
+        const int units = p.k4 / 128;
+        begin = (int)((long long)units * sl / p.slices4) * 4;
+        end = (int)((long long)units * (sl + 1) / p.slices4) * 4;
+        ti.a_step0 = 0;
+    } else {
+        const int units = (p.k - p.k4) / 64, s6 = sl - p.slices4, n6 = nsl - p.slices4;
+        begin = (int)((long long)units * s6 / n6) * 2;
+        end = (int)((long long)units * (s6 + 1) / n6) * 2;
+        ti.a_step0 = p.k4 / 32;
+    }
+}
+
+// Where a tile's packed words sit.  Reference order: a k-block (16 rows of k) is one row of region_n * 8 bytes
+// (4-bit plane / INT4; half that for the 2-bit plane) in which the tile owns 1 KiB (512 B), lane granules in
+// fragment-owner order.  gfx950 order: the tile's k-blocks follow each other, lane granules in MFMA lane order.
+struct PlaneGeometry {
+    size_t row4, row2;       // bytes from one k-block of the tile to the next
+    size_t tile4, tile2;     // byte offset of the tile's first k-block
+};
+__device__ __forceinline__ PlaneGeometry plane_geometry(const GemmArgs& p, const TileInfo& ti)
+{
+    PlaneGeometry g;
+    if (p.native) {
+        const size_t kblocks = (size_t)(p.k4 ? (ti.fp6 ? p.k - p.k4 : p.k4) : p.k) / 16;
+        g.row4 = 1024;
+        g.row2 = 512;
+        g.tile4 = (size_t)ti.tcol * kblocks * 1024;
+        g.tile2 = (size_t)ti.tcol * kblocks * 512;
+    } else {
+        g.row4 = (size_t)ti.region_n * 8;
+        g.row2 = (size_t)ti.region_n * 4;
+        g.tile4 = (size_t)ti.tcol * 1024;
+        g.tile2 = (size_t)ti.tcol * 512;
+    }
+    return g;
+}
+
+__device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
+{
+    TileInfo t;
+    const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    t.tile = logical / p.ksplit;
+    t.part = logical - t.tile * p.ksplit;
+    t.mtile = blockIdx.y;
+    t.fp6 = t.tile < p.tiles6;
+    t.tcol = t.fp6 ? t.tile : t.tile - p.tiles6;
+    t.region_n = t.fp6 ? p.qc : p.n4;
+    t.col0 = (t.fp6 ? p.n4 : 0) + t.tcol * kTileN;
+    t.a_step0 = 0;
+    return t;
+}
+
+// k range of one wave in steps of 32 (two k-blocks).  Units of two steps (four with group scales) keep
+// every wave's step count even and group-aligned.
+template <bool G128, int WK = kWaves>
+__device__ __forceinline__ void wave_k_range(const GemmArgs& p, int part, int wave, int& begin, int& end)
+{
+    constexpr int unit_steps = G128 ? 4 : 2;
+    const int units = p.k / (32 * unit_steps);
+    const int nwaves = p.ksplit * WK;
+    const int wv = part * WK + wave;
+    begin = (int)((long long)units * wv / nwaves) * unit_steps;
+    end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
+}
+
+// ------------------------------------------------------------------------------------------------ loads, waits, dequantisers
+
+#define FP6M_AS1 __attribute__((address_space(1)))
+#define FP6M_AS3 __attribute__((address_space(3)))
+
+__device__ __forceinline__ void dma16(const void* gsrc, unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 0);
+}
+// Same, with the non-temporal hint: for the packed words, which are read exactly once.
+__device__ __forceinline__ void dma16_stream(const void* gsrc, unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 2);
+}
+__device__ __forceinline__ void dma4(const void* gsrc, unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 4, 0, 0);
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* ptr) { return (uint32_t)(uintptr_t)(const FP6M_AS3 void*)ptr; }
+
+// Direct-to-LDS loads in their scalar-base form: global address = sbase + voff + OFF, LDS address =
+// M0 + OFF + 16 * lane.  The immediate moves both sides, so loads whose LDS targets lie within 4 KiB of
+// each other share one M0 value (the global side is compensated in voff or sbase) and no vector address
+// arithmetic is left in the loop.  One wait state separates the M0 write from its first use.
+// The "s" operands below must live in SGPRs: values are made wave-uniform explicitly where they are
+// created (a no-op when the compiler already knows it).
+__device__ __forceinline__ uint32_t uniform32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename T>
+__device__ __forceinline__ const T* uniform_ptr(const T* ptr)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const T*>(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ void set_m0(uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_base) : "memory");
+}
+template <int OFF, bool STREAM>
+__device__ __forceinline__ void dma16_m0(const void* sbase, uint32_t voff)
+{
+    static_assert(OFF >= 0 && OFF < 4096, "13-bit signed immediate");
+    if constexpr (STREAM)
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2 nt" : : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+    else
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+}
+__device__ __forceinline__ void dma4_m0(const void* sbase, uint32_t voff)
+{
+    asm volatile("global_load_lds_dword %0, %1" : : "v"(voff), "s"(sbase) : "memory");
+}
+template <int MB, int A_OFF, int I = 0>
+__device__ __forceinline__ void dma_a_blocks(uint32_t slot_lds, const void* sbase_a, const uint32_t (&voff)[MB])
+{
+    if constexpr (I < MB) {
+        constexpr int lds_off = A_OFF + 1024 * I;
+        if constexpr (lds_off % 4096 == 0) set_m0(slot_lds + lds_off);
+        dma16_m0<lds_off % 4096, false>(sbase_a, voff[I]);
+        dma_a_blocks<MB, A_OFF, I + 1>(slot_lds, sbase_a, voff);
+    }
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt = [3:0] and [15:14]).
+constexpr int vmcnt_only(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+// A value the optimiser must treat as an unknown VGPR: keeps bit masks in registers so that
+// (x & mask) | magic selects the three-operand v_and_or_b32 (VOP3 cannot take literals on gfx9).
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+struct DequantConsts {
+    uint32_t lo, hi, ex;          // INT4 nibble masks and the 1024.0 magic
+    uint32_t top2, exp_man;       // FP6 plane mask and the s00eeemm field mask
+};
+
+__device__ __forceinline__ void dequant_int4_fast(uint32_t q, const DequantConsts& k, h2 (&r)[4])
+{
+    const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+    const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+    const uint32_t q8 = q >> 8;
+    r[0] = as_h2((q & k.lo) | k.ex) - bias_lo;
+    r[1] = __builtin_elementwise_fma(as_h2((q & k.hi) | k.ex), mul_hi, bias_hi);
+    r[2] = as_h2((q8 & k.lo) | k.ex) - bias_lo;
+    r[3] = __builtin_elementwise_fma(as_h2((q8 & k.hi) | k.ex), mul_hi, bias_hi);
+}
+
+typedef short s2 __attribute__((ext_vector_type(2)));
+
+// FP6 without the multiply by 4096 (the MFMA keeps fp16 sub-normal inputs; 4096 goes into the epilogue
+// scale).  p holds four bytes `s eee mm xx`, MSB first e1 e3 e0 e2; an arithmetic shift right by two of
+// each 16-bit half moves eee mm under the sign and the mask 0x9f00 clears the sign copies and the low byte.
+__device__ __forceinline__ void dequant_fp6_fast(uint32_t q2, uint32_t q4, const DequantConsts& k, h2 (&r)[4])
+{
+    const s2 two = {2, 2};
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const uint32_t lo = half == 0 ? (q4 >> 2) : (q4 << 2);
+        const uint32_t hi = half == 0 ? q2 : (q2 << 2);
+        const uint32_t p = (hi & k.top2) | (lo & ~k.top2);                       // v_bfi_b32
+        const uint32_t p8 = p << 8;
+        r[2 * half + 0] = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p) >> two) & k.exp_man);
+        r[2 * half + 1] = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p8) >> two) & k.exp_man);
+    }
+}
+
+// s_waitcnt immediate that waits for lgkmcnt <= n only.
+constexpr int lgkmcnt_only(int n) { return 15 | (3 << 14) | (7 << 4) | ((n & 15) << 8); }
+
+}  // namespace fp6m

@@ -1,0 +1,403 @@
+// gemm_m16_kernel: the m <= 16 (decode) kernel of fp6m_gemm.hip.
+#pragma once
+#include "gemm_common.h"
+
+namespace fp6m {
+
+// ------------------------------------------------------------------------------------------------ m <= 16: LDS-ring kernel
+//
+// Every wave keeps a private ring of DEPTH slots in LDS.  A slot is one k step (32 rows of k) of its
+// tile: the packed words (2 x 1 KiB 4-bit/INT4, + 2 x 512 B FP6 2-bit) and the 16 x 32 fp16 activation
+// block (1 KiB).  Slots are filled by direct-to-LDS global loads (no VGPR staging): lane L's data lands
+// at slot + 16 L, so the *global* granule each lane fetches is permuted (inside aligned 64-byte quads,
+// which keeps the loads coalesced) to obtain a layout that the permuted reads hit without bank
+// conflicts.  The loads of step s + DEPTH - 1 are issued before step s is consumed; `s_waitcnt vmcnt`
+// with a constant count is the only synchronisation in the loop.  LDS reads are inline asm so that
+// the compiler does not serialise them behind every outstanding direct-to-LDS load.
+
+struct StepRegs {
+    u4 q0, q1;          // 4-bit plane / INT4 words of the two k-blocks
+    u2 t0, t1;          // FP6 2-bit plane
+    uint32_t a[4];      // activations in MFMA operand order
+};
+
+// AROWS = rows of A a slot holds (4 or 16): 64 bytes per row and step.
+template <bool FP6, bool G128, int DEPTH, int AROWS>
+__device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
+                                            int step_begin, int step_end, f4 (&acc)[1][8])
+{
+    static_assert(DEPTH >= 3, "needs two steps of look-ahead");
+    constexpr bool kGroup = G128 && !FP6;                 // group scales apply to INT4 tiles only
+    constexpr int kAOff = FP6 ? 3072 : 2048;
+    constexpr int kSlot = kAOff + AROWS * 64;
+    constexpr int kOps = FP6 ? 4 : 3;                     // direct-to-LDS loads per step
+    constexpr int kReads = FP6 ? 8 : 6;                   // LDS reads per step
+    constexpr int kUnroll = kGroup ? 4 : 2;               // steps per loop trip (step counts are multiples of it)
+    const int lane = threadIdx.x & 63;
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+
+    DequantConsts kc;
+    kc.lo = vgpr_const(0x000f000fu);
+    kc.hi = vgpr_const(0x00f000f0u);
+    kc.ex = vgpr_const(0x64006400u);
+    kc.top2 = vgpr_const(0xc0c0c0c0u);
+    kc.exp_man = vgpr_const(0x9f009f00u);
+
+    // ---- fetch side (lane = position in the slot).  Uniform 64-bit bases advance on the scalar unit;
+    // each lane only contributes a constant 32-bit offset.
+    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
+    const PlaneGeometry geo = plane_geometry(p, ti);
+    const size_t row4 = geo.row4, row2 = geo.row2;
+    const unsigned char* base4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                                 geo.tile4 + (size_t)(2 * step_begin) * row4;
+    const int lg = lane & 31;
+    const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
+    const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + geo.tile2 +
+                                 (size_t)(2 * step_begin) * row2;
+    const int a_m = lane >> 2;
+    const bool a_active = a_m < AROWS && ti.mtile * 16 + a_m < p.m;
+    const uint32_t va = (uint32_t)(a_active ? a_m : 0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3));
+    const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)ti.mtile * 16 * p.k) +
+                                  (size_t)(ti.a_step0 + step_begin) * 64;
+    const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
+    const uint32_t vgs = 4 * lane;
+    constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;        // 256-byte slabs of group scales: 2 suffice up to depth 5
+    unsigned char* gs_ring = ring + DEPTH * kSlot;
+
+    int issued = step_begin;                              // next step to fetch (clamped at the last one)
+    const int last = step_end - 1;
+    auto issue = [&](int slot) {
+        unsigned char* dst = ring + slot * kSlot;
+        dma16_stream(base4 + v4, dst);
+        dma16_stream(base4 + row4 + v4, dst + 1024);
+        if (FP6) dma16_stream(base2 + v2, dst + 2048);
+        if (a_active) dma16(base_a + va, dst + kAOff);
+        if (kGroup && (issued & 3) == 0)
+            dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & kScaleMask) * 256);
+        if (issued < last) {                              // uniform: pointers move on the scalar unit
+            issued++;
+            base4 += 2 * row4;
+            base2 += 2 * row2;
+            base_a += 64;
+        }
+    };
+
+    // ---- read side (lane = MFMA identity)
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;   // whose granule of the k-block this lane needs
+    const uint32_t ring_lds = lds_addr(ring);
+    const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
+    const int gr2 = owner >> 1;
+    const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
+    const int ar = c & (AROWS - 1);                       // rows beyond AROWS re-read a valid row; their sums are never stored
+    uint32_t rda[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * ar + (d ^ ((ar >> 2) & 3))) * 16 + 4 * i;
+    const int q = i;                                      // result side: quarter of the column slots
+    const uint32_t rdgs = lds_addr(gs_ring) + (64 * (q >> 1) + 4 * (q & 1)) * 2;
+
+    // kReads LDS reads of one step, not waited for.
+    auto fetch = [&](StepRegs& r, int slot) {
+        const uint32_t so = slot * kSlot;
+        if (FP6) {
+            asm volatile(
+                "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
+                "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
+                : "=&v"(r.q0), "=&v"(r.q1), "=&v"(r.t0), "=&v"(r.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
+        } else {
+            asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
+                         : "=&v"(r.q0), "=&v"(r.q1) : "v"(rd4 + so) : "memory");
+        }
+        asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7"
+                     : "=&v"(r.a[0]), "=&v"(r.a[1]), "=&v"(r.a[2]), "=&v"(r.a[3])
+                     : "v"(rda[0] + so), "v"(rda[1] + so), "v"(rda[2] + so), "v"(rda[3] + so) : "memory");
+    };
+    // After the counter wait, the registers of `r` hold their data: make every later use depend on it.
+    auto settle = [&](StepRegs& r) {
+        asm volatile("" : "+v"(r.q0), "+v"(r.q1), "+v"(r.a[0]), "+v"(r.a[1]), "+v"(r.a[2]), "+v"(r.a[3]));
+        if (FP6) asm volatile("" : "+v"(r.t0), "+v"(r.t1));
+    };
+    auto compute = [&](const StepRegs& r, f4 (&dst)[8], bool fresh) {
+        const h8 av = __builtin_bit_cast(h8, u4{r.a[0], r.a[1], r.a[2], r.a[3]});
+        const f4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            h2 r0[4], r1[4];
+            if (FP6) {
+                dequant_fp6_fast(r.t0[j >> 1] << (4 * (j & 1)), r.q0[j], kc, r0);
+                dequant_fp6_fast(r.t1[j >> 1] << (4 * (j & 1)), r.q1[j], kc, r1);
+            } else {
+                dequant_int4_fast(r.q0[j], kc, r0);
+                dequant_int4_fast(r.q1[j], kc, r1);
+            }
+            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
+            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
+            dst[2 * j + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, fresh ? zero : dst[2 * j + 0], 0, 0, 0);
+            dst[2 * j + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, fresh ? zero : dst[2 * j + 1], 0, 0, 0);
+        }
+    };
+
+    // Pipeline: while step s is being computed, the LDS reads of step s+1 are in flight and the
+    // direct-to-LDS loads of steps s+2 .. s+DEPTH-1 are outstanding.
+    int slot_in = 0;
+#pragma unroll 1
+    for (int d = 0; d < DEPTH - 1; d++) {
+        issue(slot_in);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    }
+    StepRegs regs[2];
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+    FP6M_MARK(p, 1);
+    fetch(regs[0], 0);
+    int slot_rd = 1;                                      // slot of the step whose LDS reads come next
+    f4 grp[8];
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s += kUnroll) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            issue(slot_in);
+            slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));   // step s+u+1 has landed
+            fetch(regs[(u + 1) & 1], slot_rd);
+            slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
+            __builtin_amdgcn_s_waitcnt(lgkmcnt_only(kReads));             // reads of step s+u (older) are done
+            settle(regs[u & 1]);
+            if (kGroup)
+                compute(regs[u & 1], grp, u == 0);
+            else
+                compute(regs[u & 1], acc[0], false);
+        }
+        if (kGroup) {
+            // end of a 128-row group: fold it into the running sum with its scales (fp32)
+            const uint32_t ga = rdgs + ((s >> 2) & kScaleMask) * 256;
+            u2 sv[8];
+            asm volatile(
+                "ds_read_b64 %0, %8\n\tds_read_b64 %1, %8 offset:16\n\tds_read_b64 %2, %8 offset:32\n\t"
+                "ds_read_b64 %3, %8 offset:48\n\tds_read_b64 %4, %8 offset:64\n\tds_read_b64 %5, %8 offset:80\n\t"
+                "ds_read_b64 %6, %8 offset:96\n\tds_read_b64 %7, %8 offset:112\n\ts_waitcnt lgkmcnt(0)"
+                : "=&v"(sv[0]), "=&v"(sv[1]), "=&v"(sv[2]), "=&v"(sv[3]), "=&v"(sv[4]), "=&v"(sv[5]), "=&v"(sv[6]),
+                  "=&v"(sv[7])
+                : "v"(ga) : "memory");
+            settle(regs[0]);                              // lgkmcnt(0) also completed the look-ahead reads
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const h2 lo = as_h2(sv[t][0]), hi = as_h2(sv[t][1]);
+                acc[0][t][0] += (float)lo[0] * grp[t][0];
+                acc[0][t][1] += (float)lo[1] * grp[t][1];
+                acc[0][t][2] += (float)hi[0] * grp[t][2];
+                acc[0][t][3] += (float)hi[1] * grp[t][3];
+            }
+        }
+    }
+    // Redundant tail prefetches and look-ahead reads may still be in flight; the epilogue reuses the ring.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    settle(regs[0]);
+    if (FP6) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[0][t] *= 4096.0f;  // the deferred e3m2 exponent re-bias
+    }
+}
+
+// LDS per wave: the larger of an INT4 ring (D4 slots + the group-scale slabs) and an FP6 ring (D6
+// slots), and at least the 16 x 128 fp32 row slab of the epilogue.
+constexpr int scale_slab_bytes(int depth) { return depth <= 5 ? 512 : 1024; }
+constexpr int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
+constexpr int wave_lds_bytes(int d4, int d6, int arows)
+{
+    return max3(d4 * (2048 + arows * 64) + scale_slab_bytes(d4), d6 * (3072 + arows * 64), 16 * kRedStride * 4);
+}
+
+// The m <= 16 kernel.
+//
+// A workgroup is WN x WK waves: WN adjacent 128-column tiles (one per wave column, so the workgroup
+// reads WN KiB contiguous runs of every k-block row) times WK consecutive slices of the workgroup's
+// k range.  Waves never synchronise in the main loop.  Epilogue: every wave turns its MFMA fragments
+// into fp32 rows in its own drained ring, one barrier, then wave (wn, wk) sums rows wk, wk+WK, ... of
+// tile wn over the WK slices (fixed order) with lane L owning columns 2L, 2L+1.  With one k part per
+// tile group it scales and writes C; otherwise it publishes the rows with agent-scope stores, the
+// workgroup bumps the group's counter, and the workgroup that arrives last sums all parts in part order.
+template <int WN, int WK>
+__device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti, bool tile_valid, int wn, int wk,
+                                          int ks, int slot_base, int* counter, f4 (&acc)[1][8],
+                                          bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
+                                          int first_fp6 = WK)
+{
+    // first_fp6: row mix only -- k slices first_fp6 .. WK-1 of this workgroup hold FP6 rows, whose sums take the
+    // FP6 column scale here (the INT4 slices are already scaled by their group scales)
+    constexpr int RMAX = (16 + WK - 1) / WK;                             // rows one wave finishes
+    constexpr int PCHUNK = 32 / RMAX;                                    // parts whose loads are in flight together
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15, q = lane >> 4;
+    const int wave = wk * WN + wn;
+    if (tile_valid) {
+        float* mine = reinterpret_cast<float*>(smem + wave * wave_lds) + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[0][t];
+    }
+    __syncthreads();
+    FP6M_MARK(p, 3);
+
+    const int nrows = p.m < 16 ? p.m : 16;
+    float s0 = 1.0f, s1 = 1.0f;
+    if (tile_valid && per_column_scale) {
+        const uint16_t* sp = ti.fp6 ? p.s_fp6 : p.s_int4;
+        const int nr = ti.tcol * kTileN + 2 * lane;                      // even column inside the region
+        const h2 sv = *reinterpret_cast<const h2*>(sp + (nr & ~31) + scale_slot(nr & 31));
+        s0 = (float)sv[0];
+        s1 = (float)sv[1];
+    }
+    float x0 = 1.0f, x1 = 1.0f;                                          // FP6 column scales of a row mix
+    if (tile_valid && first_fp6 < WK) {
+        const int nr = ti.tcol * kTileN + 2 * lane;
+        const h2 sv = *reinterpret_cast<const h2*>(p.s_fp6 + (nr & ~31) + scale_slot(nr & 31));
+        x0 = (float)sv[0];
+        x1 = (float)sv[1];
+    }
+    uint16_t* c_out = p.C + ti.col0 + 2 * lane;
+    auto store_row = [&](int m, float v0, float v1) {
+        if (p.fused) {
+            store_fused(p, (size_t)m, ti.col0 + 2 * lane, v0 * s0, v1 * s1);
+            return;
+        }
+        h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
+        *reinterpret_cast<h2*>(c_out + (size_t)m * p.n) = o;
+    };
+
+    // Sum of the WK slices of my rows.
+    float v0[RMAX], v1[RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+        v0[r] = 0.f;
+        v1[r] = 0.f;
+        const int m = wk + r * WK;
+        if (tile_valid && m < nrows) {
+#pragma unroll
+            for (int j = 0; j < WK; j++) {
+                const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + (j * WN + wn) * wave_lds) +
+                                                          m * kRedStride + 2 * lane);
+                v0[r] += j >= first_fp6 ? v[0] * x0 : v[0];
+                v1[r] += j >= first_fp6 ? v[1] * x1 : v[1];
+            }
+        }
+    }
+    if (ks == 1) {
+#pragma unroll
+        for (int r = 0; r < RMAX; r++)
+            if (tile_valid && wk + r * WK < nrows) store_row(wk + r * WK, v0[r], v1[r]);
+        return;
+    }
+
+    // Publish.  A slot holds [WN tiles][16 rows][128 columns] fp32; 8-byte agent-scope accesses.
+    constexpr size_t kSlotU64 = (size_t)WN * 16 * kTileN / 2;
+    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) + (size_t)slot_base * kSlotU64 +
+                                (size_t)wn * (16 * kTileN / 2) + lane;
+    unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+        const int m = wk + r * WK;
+        if (tile_valid && m < nrows) {
+            const f2 v = {v0[r], v1[r]};
+            __hip_atomic_store(my + m * (kTileN / 2), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");               // my stores have completed
+    __syncthreads();
+    FP6M_MARK(p, 4);
+    if (threadIdx.x == 0) {
+        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = (seen == ks - 1);
+    }
+    __syncthreads();
+    FP6M_MARK(p, 5);
+    if (!*flag) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+    for (int r = 0; r < RMAX; r++) {
+        v0[r] = 0.f;
+        v1[r] = 0.f;
+    }
+    for (int pp = 0; pp < ks; pp += PCHUNK) {
+        unsigned long long t[PCHUNK][RMAX];
+#pragma unroll
+        for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                const int m = wk + r * WK;
+                t[u][r] = 0;
+                if (tile_valid && m < nrows && pp + u < ks)
+                    t[u][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + m * (kTileN / 2), __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+        for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                const f2 v = __builtin_bit_cast(f2, t[u][r]);
+                v0[r] += v[0];
+                v1[r] += v[1];
+            }
+    }
+#pragma unroll
+    for (int r = 0; r < RMAX; r++)
+        if (tile_valid && wk + r * WK < nrows) store_row(wk + r * WK, v0[r], v1[r]);
+    FP6M_MARK(p, 6);
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <bool G128, int AROWS, int WN, int WK, int D4, int D6>
+// second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
+__global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArgs p)
+{
+    constexpr int NW = WN * WK;
+    constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);
+    __shared__ __attribute__((aligned(16))) unsigned char smem[NW * kWaveLds + 16];
+
+    FP6M_MARK(p, 0);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
+    const int wn = wave % WN, wk = wave / WN;
+    const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int wgs6 = p.groups6 * p.ks6;                                  // the FP6 region's workgroups come first
+    TileInfo ti;
+    ti.fp6 = logical < wgs6;
+    const int local = ti.fp6 ? logical : logical - wgs6;
+    const int groups = ti.fp6 ? p.groups6 : p.groups4;
+    const int ks = ti.fp6 ? p.ks6 : p.ks4;
+    ti.part = local / groups;                                            // part-major: neighbours share k, adjoin in n
+    const int group = local - ti.part * groups;
+    ti.tcol = group * WN + wn;
+    ti.region_n = ti.fp6 ? p.qc : p.n4;
+    const bool tile_valid = ti.tcol * kTileN < ti.region_n;
+    ti.tile = ti.fp6 ? ti.tcol : p.tiles6 + ti.tcol;
+    ti.mtile = 0;
+    ti.col0 = (ti.fp6 ? p.n4 : 0) + ti.tcol * kTileN;
+
+    constexpr int unit_steps = G128 ? 4 : 2;
+    const int units = p.k / (32 * unit_steps);
+    const int kp = ti.part * WK + wk, kparts = ks * WK;
+    int step_begin = (int)((long long)units * kp / kparts) * unit_steps;
+    int step_end = (int)((long long)units * (kp + 1) / kparts) * unit_steps;
+    ti.a_step0 = 0;
+    const bool region6 = ti.fp6;                                         // the workgroup's column region
+    if (p.k4) row_mix_slice(p, kp, kparts, ti, step_begin, step_end);    // per wave: INT4 or FP6 rows of the tile
+
+    f4 acc[1][8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[0][t] = f4{0.f, 0.f, 0.f, 0.f};
+    unsigned char* ring = smem + wave * kWaveLds;
+    if (tile_valid && step_begin < step_end) {
+        if (ti.fp6)
+            stream_tile<true, G128, D6, AROWS>(p, ti, ring, step_begin, step_end, acc);
+        else
+            stream_tile<false, G128, D4, AROWS>(p, ti, ring, step_begin, step_end, acc);
+    }
+    FP6M_MARK(p, 2);
+    // scratch slots: FP6 groups first (groups6 * ks6 slots), then INT4 groups; counters likewise
+    const int slot_base = region6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
+    int* counter = p.counters + (region6 ? group : p.groups6 + group);
+    wg_finish<WN, WK>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+                      reinterpret_cast<int*>(smem + NW * kWaveLds), p.k4 ? p.slices4 - ti.part * WK : WK);
+    FP6M_MARK(p, 7);
+}
+
+}  // namespace fp6m

@@ -1,0 +1,513 @@
+// gemm_mb_kernel: the 16 < m kernel of fp6m_gemm.hip (private rings, MB 16-row blocks per wave, asm MFMAs).
+#pragma once
+#include "gemm_common.h"
+
+namespace fp6m {
+
+// ------------------------------------------------------------------------------------------------ 16 < m: ring kernel with MB row blocks
+//
+// Same ring and lane routing as the m <= 16 kernel, but a slot carries MB blocks of 16 rows of A (1 KiB
+// each) and every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per
+// 16*MB rows.  A workgroup is one tile x four k slices; blockIdx.y walks the row tiles.  Group scales are
+// applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more
+// registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
+// the number of direct-to-LDS loads per step is constant) and never stored.
+
+struct WeightRegs {
+    u4 q0, q1;
+};
+
+template <int N>
+struct Int {
+    static constexpr int value = N;
+};
+
+template <int OFF>
+__device__ __forceinline__ void lds_read_a4(uint32_t (&a)[4], const uint32_t (&addr)[4])
+{
+    asm volatile(
+        "ds_read_b32 %0, %4 offset:%8\n\tds_read_b32 %1, %5 offset:%8\n\t"
+        "ds_read_b32 %2, %6 offset:%8\n\tds_read_b32 %3, %7 offset:%8"
+        : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3])
+        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "n"(OFF) : "memory");
+}
+
+// acc += w (16 columns x 32 k) * a (16 rows x 32 k), in place.  Written as asm so that the accumulator
+// stays in one VGPR quad for the whole loop (the builtin let the allocator rotate the accumulators
+// through copies) and the MFMAs keep their place between the LDS reads.  The hazards the compiler would pad for are handled
+// here: an MFMA must not read a VGPR in the two wait states after a VALU wrote it (register copies the
+// allocator places in front of the asm count), hence the s_nop; the loop never reads an accumulator
+// except as the addend of the same MFMA a full step later; the wait states before the first VALU read
+// of a result follow the loop.
+template <bool FIRST>
+__device__ __forceinline__ void mfma_acc(f4& acc, const h8& w, const h8& a)
+{
+    if constexpr (FIRST)
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
+    else
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
+}
+
+// Two of the four h2 a packed word expands to (half 0: fragment columns +0, half 1: columns +8).
+template <bool FP6>
+__device__ __forceinline__ void dequant_half(uint32_t q2, uint32_t q4, int half, const DequantConsts& k, h2& r0, h2& r1)
+{
+    if constexpr (FP6) {
+        const s2 two = {2, 2};
+        const uint32_t lo = half == 0 ? (q4 >> 2) : (q4 << 2);
+        const uint32_t hi = half == 0 ? q2 : (q2 << 2);
+        const uint32_t p = (hi & k.top2) | (lo & ~k.top2);
+        const uint32_t p8 = p << 8;
+        r0 = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p) >> two) & k.exp_man);
+        r1 = as_h2(__builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, p8) >> two) & k.exp_man);
+    } else {
+        const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+        const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
+        const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+        const uint32_t q = half == 0 ? q4 : (q4 >> 8);
+        r0 = as_h2((q & k.lo) | k.ex) - bias_lo;
+        r1 = __builtin_elementwise_fma(as_h2((q & k.hi) | k.ex), mul_hi, bias_hi);
+    }
+}
+
+struct MbCtx {
+    uint32_t abuf[4][4];
+    uint32_t addr_cur[4], addr_next[4];
+};
+
+// One step of the MB loop, fully static in BLK: block by block the 16 rows of A are multiplied into
+// the step's eight weight fragments.  Activations travel through a ring of four register buffers,
+// fetched from LDS two blocks ahead of their use (the latency hides behind 16 MFMAs); the s_waitcnt
+// immediates follow from the fixed issue order: [A(0), A(1)] from the previous step, the next step's
+// weight words (kExtra reads), then A(2), A(3), ...  After every MFMA `hook(block, t)` runs: the caller
+// uses it to dequantise the next step's fragments a few VALU instructions at a time.
+template <int MB, int kExtra, int BLK = 0>
+struct MbBlocks {
+    template <int phase, typename Hook>
+    static __device__ __forceinline__ void run(MbCtx& cx, const h8 (&frag)[8], f4 (&acc)[MB][8], Hook&& hook)
+    {
+        if constexpr (BLK < MB) {
+            constexpr int nb = BLK + 2;
+            uint32_t (&dst)[4] = cx.abuf[(phase + nb) & 3];
+            if constexpr (nb < MB)
+                lds_read_a4<nb * 1024>(dst, cx.addr_cur);
+            else
+                lds_read_a4<(nb - MB) * 1024>(dst, cx.addr_next);
+            // block 0 needs A(0): A(1), the extra reads and A(2) may be outstanding; from block 1 on the
+            // extra reads must be complete as well
+            constexpr int allow = BLK == 0 ? (8 + kExtra < 15 ? 8 + kExtra : 15) : 8;
+            __builtin_amdgcn_s_waitcnt(lgkmcnt_only(allow));
+            uint32_t (&src)[4] = cx.abuf[(phase + BLK) & 3];
+            asm volatile("" : "+v"(src[0]), "+v"(src[1]), "+v"(src[2]), "+v"(src[3]));
+            const h8 av = __builtin_bit_cast(h8, u4{src[0], src[1], src[2], src[3]});
+            mfma_acc<true>(acc[BLK][0], frag[0], av); hook(Int<BLK>{}, Int<0>{});
+            mfma_acc<false>(acc[BLK][1], frag[1], av); hook(Int<BLK>{}, Int<1>{});
+            mfma_acc<false>(acc[BLK][2], frag[2], av); hook(Int<BLK>{}, Int<2>{});
+            mfma_acc<false>(acc[BLK][3], frag[3], av); hook(Int<BLK>{}, Int<3>{});
+            mfma_acc<false>(acc[BLK][4], frag[4], av); hook(Int<BLK>{}, Int<4>{});
+            mfma_acc<false>(acc[BLK][5], frag[5], av); hook(Int<BLK>{}, Int<5>{});
+            mfma_acc<false>(acc[BLK][6], frag[6], av); hook(Int<BLK>{}, Int<6>{});
+            mfma_acc<false>(acc[BLK][7], frag[7], av); hook(Int<BLK>{}, Int<7>{});
+            MbBlocks<MB, kExtra, BLK + 1>::template run<phase>(cx, frag, acc, hook);
+        }
+    }
+};
+
+template <bool FP6, bool G128, int DEPTH, int MB>
+__device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
+                                               int step_begin, int step_end, f4 (&acc)[MB][8])
+{
+    static_assert(DEPTH >= 3, "needs two steps of look-ahead");
+    static_assert(MB == 2 || MB == 4, "the A register ring assumes MB | 4; 128 accumulator VGPRs at most");
+    constexpr bool kGroup = G128 && !FP6;
+    static_assert(!FP6 || DEPTH == 3, "the 2-bit plane alternates between two register sets");
+    constexpr int kAOff = 2048;
+    constexpr int kSlot = kAOff + MB * 1024;
+    constexpr int kOps = 2 + MB + (FP6 ? 2 : 0);          // vector-memory loads per step
+    constexpr int kUnroll = kGroup ? 4 : 2;
+    constexpr int kW = 2;                                 // LDS reads of one step's weight words
+    static_assert(kOps * (DEPTH - 2) <= 63, "vmcnt is a 6-bit counter");
+    const int lane = threadIdx.x & 63;
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+
+    DequantConsts kc;
+    kc.lo = vgpr_const(0x000f000fu);
+    kc.hi = vgpr_const(0x00f000f0u);
+    kc.ex = vgpr_const(0x64006400u);
+    kc.top2 = vgpr_const(0xc0c0c0c0u);
+    kc.exp_man = vgpr_const(0x9f009f00u);
+
+    // ---- fetch side: uniform 64-bit bases on the scalar unit, per-lane 32-bit offsets that never change.
+    // The offsets carry the compensation for the immediates (see dma16_m0): the second k-block of the
+    // words sits 1 KiB further in LDS and one row further in memory; the A blocks get theirs on the
+    // scalar base, so that the lane offsets stay non-negative.  The FP6 2-bit plane (8 bytes per lane and
+    // k-block, already in owner order in memory) skips LDS: it is loaded into registers two steps ahead,
+    // alternating between two register sets, which keeps an FP6 slot as small as an INT4 one.
+    const PlaneGeometry geo = plane_geometry(p, ti);
+    const size_t row4 = geo.row4, row2 = geo.row2;
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;      // whose granule of the k-block this lane needs
+    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
+    const uint32_t v4b = v4 + (uint32_t)row4 - 1024;
+    const unsigned char* base4 = uniform_ptr(reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                                             geo.tile4 + (size_t)(2 * step_begin) * row4);
+    const uint32_t v2 = (uint32_t)owner * 8, v2b = v2 + (uint32_t)row2;
+    const unsigned char* base2 = uniform_ptr(reinterpret_cast<const unsigned char*>(p.b_fp6_2) +
+                                             geo.tile2 + (size_t)(2 * step_begin) * row2);
+    u2 tq[2][2];                                          // [register set][k-block]
+    const int a_m = lane >> 2;
+    const int tile_row0 = ti.mtile * 16 * MB;
+    uint32_t va[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        int row = tile_row0 + 16 * mb + a_m;
+        row = row < p.m ? row : p.m - 1;
+        va[mb] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3)) + 4096 -
+                 (kAOff + 1024 * mb) % 4096;
+    }
+    const unsigned char* base_a = uniform_ptr(reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
+                                              (size_t)(ti.a_step0 + step_begin) * 64 - 4096);
+    const unsigned char* base_gs =
+        uniform_ptr(reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN));
+    const uint32_t vgs = 4 * lane;
+    constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;
+    unsigned char* gs_ring = ring + DEPTH * kSlot;
+    const uint32_t ring_lds = uniform32(lds_addr(ring));
+    const uint32_t gs_lds = uniform32(lds_addr(gs_ring));
+
+    int issued = step_begin;
+    const int last = step_end - 1;
+    auto issue = [&](int slot, int set) {
+        const uint32_t dst = ring_lds + slot * kSlot;
+        set_m0(dst);
+        dma16_m0<0, true>(base4, v4);
+        dma16_m0<1024, true>(base4, v4b);
+        dma_a_blocks<MB, kAOff>(dst, base_a, va);
+        if (FP6) {
+            asm volatile("global_load_dwordx2 %0, %2, %4 nt\n\tglobal_load_dwordx2 %1, %3, %4 nt"
+                         : "=&v"(tq[set][0]), "=&v"(tq[set][1]) : "v"(v2), "v"(v2b), "s"(base2) : "memory");
+        }
+        if (kGroup && (issued & 3) == 0) {
+            set_m0(gs_lds + ((issued >> 2) & kScaleMask) * 256);
+            dma4_m0(base_gs + (size_t)(issued >> 2) * (size_t)uniform32(p.n4) * 2, vgs);
+        }
+        if (issued < last) {
+            issued++;
+            base4 += 2 * row4;
+            base2 += 2 * row2;
+            base_a += 64;
+        }
+    };
+
+    // ---- read side
+    const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
+    uint32_t rda[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * c + (d ^ ((c >> 2) & 3))) * 16 + 4 * i;
+    const uint32_t rdgs = gs_lds + (64 * sigma + l) * 2;    // weight side: column (j, half) at +32j +16half
+
+    uint32_t gs_next[8];
+    h2 gs_cur[8];
+    MbCtx cx;
+    WeightRegs w;
+    auto fetch_w = [&](int slot) {
+        const uint32_t so = slot * kSlot;
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
+                     : "=&v"(w.q0), "=&v"(w.q1) : "v"(rd4 + so) : "memory");
+    };
+    auto fetch_scales = [&](int group) {
+        const uint32_t ga = rdgs + (group & kScaleMask) * 256;
+        asm volatile(
+            "ds_read_u16 %0, %8\n\tds_read_u16 %1, %8 offset:16\n\tds_read_u16 %2, %8 offset:32\n\t"
+            "ds_read_u16 %3, %8 offset:48\n\tds_read_u16 %4, %8 offset:64\n\tds_read_u16 %5, %8 offset:80\n\t"
+            "ds_read_u16 %6, %8 offset:96\n\tds_read_u16 %7, %8 offset:112"
+            : "=&v"(gs_next[0]), "=&v"(gs_next[1]), "=&v"(gs_next[2]), "=&v"(gs_next[3]), "=&v"(gs_next[4]),
+              "=&v"(gs_next[5]), "=&v"(gs_next[6]), "=&v"(gs_next[7])
+            : "v"(ga) : "memory");
+    };
+    auto settle_scales = [&]() {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            asm volatile("" : "+v"(gs_next[t]));
+            gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
+        }
+    };
+    // A quarter of one j group (a "chunk": 4..8 VALU instructions): chunk = 4j + 2*half + word.  The
+    // word is tied to this point of the program first, the results after, so the instructions stay
+    // between the two MFMAs the chunk was placed between.
+    h2 part[2];
+    auto chunk = [&](int ck, int set, h8 (&frag)[8]) {
+        const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
+        uint32_t q4 = word ? w.q1[j] : w.q0[j];
+        uint32_t q2 = 0;
+        asm volatile("" : "+v"(q4));
+        if (word) w.q1[j] = q4; else w.q0[j] = q4;
+        if (FP6) {
+            uint32_t t = tq[set][word][j >> 1];
+            asm volatile("" : "+v"(t));
+            tq[set][word][j >> 1] = t;
+            q2 = t << (4 * (j & 1));
+        }
+        h2 r0, r1;
+        dequant_half<FP6>(q2, q4, half, kc, r0, r1);
+        if (kGroup) {
+            r0 = r0 * gs_cur[2 * j + half];
+            r1 = r1 * gs_cur[2 * j + half];
+        }
+        if (word == 0) {
+            part[0] = r0;
+            part[1] = r1;
+            asm volatile("" : "+v"(part[0]), "+v"(part[1]));
+        } else {
+            frag[2 * j + half] = join(part[0], part[1], r0, r1);
+            asm volatile("" : "+v"(frag[2 * j + half]));
+        }
+    };
+    auto slot_addrs = [&](uint32_t (&addr)[4], int slot) {
+        const uint32_t so = slot * kSlot;
+#pragma unroll
+        for (int d = 0; d < 4; d++) addr[d] = rda[d] + so;
+    };
+
+    int slot_in = 0;
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; d++) {
+        issue(slot_in, d & 1);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    }
+    h8 frag[2][8];
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+    slot_addrs(cx.addr_next, 0);
+    fetch_w(0);
+    lds_read_a4<0>(cx.abuf[0], cx.addr_next);
+    lds_read_a4<1024>(cx.abuf[1], cx.addr_next);
+    if (kGroup) fetch_scales(step_begin >> 2);
+    __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
+    if (kGroup) settle_scales();
+#pragma unroll
+    for (int ck = 0; ck < 16; ck++) chunk(ck, 0, frag[0]);
+    int slot_rd = 1;
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s += kUnroll) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            issue(slot_in, u & 1);                                    // step s+u+2 (FP6: DEPTH is 3)
+            slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+#pragma unroll
+            for (int d = 0; d < 4; d++) cx.addr_cur[d] = cx.addr_next[d];
+            slot_addrs(cx.addr_next, slot_rd);
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+            // step s+u+1 (and its group scales) has landed: read its words now, dequantise them
+            // between this step's MFMAs
+            fetch_w(slot_rd);
+            const bool next_group = kGroup && u == kUnroll - 1;       // step s+u+1 starts a 128-row group
+            if (next_group) fetch_scales((s + u + 1) >> 2);
+            slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
+            h8 (&cur)[8] = frag[u & 1];
+            h8 (&nxt)[8] = frag[(u + 1) & 1];
+            auto hook = [&](auto blk, auto t) {
+                constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
+                constexpr int avail = 8 * MB - 8;                     // chunks go after the MFMAs of blocks >= 1
+                if constexpr (mslot == 8) {
+                    if (next_group) settle_scales();
+                }
+                if constexpr (mslot >= 8) {
+                    constexpr int c0 = (mslot - 8) * 16 / avail, c1 = (mslot - 7) * 16 / avail;
+#pragma unroll
+                    for (int ck = c0; ck < c1; ck++) chunk(ck, (u + 1) & 1, nxt);
+                }
+            };
+            constexpr int kExtraMax = kW + (kGroup ? 8 : 0);
+            if ((u & 1) == 0)                                          // buffer of block 0: (u * MB) mod 4
+                MbBlocks<MB, kExtraMax>::template run<0>(cx, cur, acc, hook);
+            else
+                MbBlocks<MB, kExtraMax>::template run<(MB & 3)>(cx, cur, acc, hook);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    // MFMA results -> VALU reads: the wait states, then every accumulator is passed through an (empty)
+    // asm so that no read of it can be scheduled above them.
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            asm volatile("" : "+v"(acc[mb][t]));
+        }
+    if (FP6) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int t = 0; t < 8; t++) acc[mb][t] *= 4096.0f;
+    }
+}
+
+// Epilogue of the MB kernel: block by block, the four k slices are summed through LDS (wave wk finishes
+// rows wk, wk+4, ... of the block, lane L owns columns 2L, 2L+1); then C is written, or the rows are
+// published and the last-arriving workgroup of the (tile, row tile) gathers all parts in part order.
+// `smem`, `flag` and `valid` belong to the WK waves that share a tile and a row tile (the whole workgroup in
+// gemm_mb_kernel, one of WM groups in gemm_wm_kernel); a group without rows goes through the barriers
+// without touching memory.
+template <int MB, int WK = kWaves>
+__device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, f4 (&acc)[MB][8],
+                                             bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
+                                             bool valid = true, int first_fp6 = WK)
+{
+    constexpr int RMAX = 16 / WK, PCHUNK = 32 / RMAX;                // parts whose loads are in flight together
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const int lane = threadIdx.x & 63;
+    const bool leader = lane == 0 && wk == 0;
+    const int c = lane & 15, q = lane >> 4;
+    const int row0 = ti.mtile * 16 * MB;
+    const int nrows = !valid ? 0 : (p.m - row0 < 16 * MB ? p.m - row0 : 16 * MB);
+    float s0 = 1.0f, s1 = 1.0f;
+    if (per_column_scale) {
+        const uint16_t* sp = ti.fp6 ? p.s_fp6 : p.s_int4;
+        const int nr = ti.tcol * kTileN + 2 * lane;
+        const h2 sv = *reinterpret_cast<const h2*>(sp + (nr & ~31) + scale_slot(nr & 31));
+        s0 = (float)sv[0];
+        s1 = (float)sv[1];
+    }
+    float x0 = 1.0f, x1 = 1.0f;                                      // row mix: FP6 column scales of slices >= first_fp6
+    if (first_fp6 < WK) {
+        const int nr = ti.tcol * kTileN + 2 * lane;
+        const h2 sv = *reinterpret_cast<const h2*>(p.s_fp6 + (nr & ~31) + scale_slot(nr & 31));
+        x0 = (float)sv[0];
+        x1 = (float)sv[1];
+    }
+    uint16_t* c_out = p.C + (size_t)row0 * p.n + ti.col0 + 2 * lane;
+    auto store_row = [&](int row, float v0, float v1) {
+        if (p.fused) {
+            store_fused(p, (size_t)(row0 + row), ti.col0 + 2 * lane, v0 * s0, v1 * s1);
+            return;
+        }
+        h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
+        *reinterpret_cast<h2*>(c_out + (size_t)row * p.n) = o;
+    };
+    constexpr size_t kSlotU64 = (size_t)MB * 16 * kTileN / 2;
+    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) +
+                                (size_t)(ti.mtile * p.tiles + ti.tile) * ks * kSlotU64 + lane;
+    unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
+
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        __syncthreads();
+        float* mine = reinterpret_cast<float*>(smem + wk * wave_lds) + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[mb][t];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            const int m = wk + r * WK, row = 16 * mb + m;
+            if (row < nrows) {
+                float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                for (int j = 0; j < WK; j++) {
+                    const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + j * wave_lds) +
+                                                              m * kRedStride + 2 * lane);
+                    v0 += j >= first_fp6 ? v[0] * x0 : v[0];
+                    v1 += j >= first_fp6 ? v[1] * x1 : v[1];
+                }
+                if (ks == 1) {
+                    store_row(row, v0, v1);
+                } else {
+                    const f2 v = {v0, v1};
+                    __hip_atomic_store(my + (size_t)row * (kTileN / 2), __builtin_bit_cast(unsigned long long, v),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+    }
+    if (ks == 1) return;
+
+    FP6M_MARK(p, 3);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
+    if (leader) {
+        int last = 0;
+        if (valid) last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ks - 1;
+        *flag = last;
+    }
+    __syncthreads();
+    if (!*flag) return;
+    FP6M_MARK(p, 5);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll 1
+    for (int mb = 0; mb < MB; mb++) {
+        float v0[RMAX], v1[RMAX];
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            v0[r] = 0.f;
+            v1[r] = 0.f;
+        }
+        for (int pp = 0; pp < ks; pp += PCHUNK) {
+            unsigned long long t[PCHUNK][RMAX];
+#pragma unroll
+            for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+                for (int r = 0; r < RMAX; r++) {
+                    const int row = 16 * mb + wk + r * WK;
+                    t[u][r] = 0;
+                    if (row < nrows && pp + u < ks)
+                        t[u][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + (size_t)row * (kTileN / 2),
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+            for (int u = 0; u < PCHUNK; u++)
+#pragma unroll
+                for (int r = 0; r < RMAX; r++) {
+                    const f2 v = __builtin_bit_cast(f2, t[u][r]);
+                    v0[r] += v[0];
+                    v1[r] += v[1];
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            const int row = 16 * mb + wk + r * WK;
+            if (row < nrows) store_row(row, v0[r], v1[r]);
+        }
+    }
+    // the counter is next touched by a later launch on the stream: the reset needs no ordering here
+    if (leader) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr int mb_wave_lds(int mb, int d4, int d6)
+{
+    return max3(d4 * (2048 + mb * 1024) + scale_slab_bytes(d4), d6 * (2048 + mb * 1024), 16 * kRedStride * 4);
+}
+
+// WK = k slices (waves) per workgroup: four, or eight (one workgroup per CU, two waves per SIMD) for grids that
+// would otherwise leave every SIMD a single wave.
+template <bool G128, int MB, int D4, int D6, int WK>
+__global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
+{
+    constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
+    static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];
+
+    FP6M_MARK(p, 0);
+    TileInfo ti = locate_tile(p);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int step_begin, step_end;
+    wave_k_range<G128, WK>(p, ti.part, wave, step_begin, step_end);
+    if (p.k4) row_mix_slice(p, ti.part * WK + wave, p.ksplit * WK, ti, step_begin, step_end);
+
+    f4 acc[MB][8];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
+    unsigned char* ring = smem + wave * kWaveLds;
+    if (step_begin < step_end) {
+        if (ti.fp6)
+            stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+        else
+            stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
+    }
+    FP6M_MARK(p, 2);
+    wg_finish_mb<MB, WK>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+                         reinterpret_cast<int*>(smem + WK * kWaveLds), true, p.k4 ? p.slices4 - ti.part * WK : WK);
+    FP6M_MARK(p, 7);
+}
+
+}  // namespace fp6m

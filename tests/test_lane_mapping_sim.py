@@ -1,6 +1,6 @@
 """
 Lane-level simulation, on the CPU, of how the gfx950 kernel routes packed words to MFMA operands
-(fp6-marlin_amd/csrc/fp6m_gemm.hip): linear 16-byte loads -> swizzled wave-private LDS slab -> permuted
+(fp6-marlin_amd/csrc/gemm_m16.h): linear 16-byte loads -> swizzled wave-private LDS slab -> permuted
 reads -> in-register dequant -> v_mfma_f32_16x16x32_f16 with the weights as the 16-row operand.
 
 The MFMA is modelled from its documented operand layout: lane L supplies row/column L % 16 and the
