@@ -445,6 +445,13 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
 
 extern "C" {
 
+int fp6m_init_gather(int dev)
+{
+    fp6m::DeviceScratch* d = nullptr;
+    if (int rc = fp6m::ensure_scratch(dev, &d)) return rc;
+    return fp6m::ensure_gather_buffer(dev, d);
+}
+
 int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
              void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
              int quant_cols, int group_size)

@@ -32,6 +32,7 @@ lib.fp6m_pack_mixed_device.restype = _int
 lib.fp6m_pack_mixed_device.argtypes = [_vp, _int, _int, _int, _int, _int, _vp, _vp, _vp, _int, _vp]
 lib.fp6m_workspace_elems.argtypes = [_int, _int]
 lib.fp6m_init.argtypes = [_int]
+lib.fp6m_init_gather.argtypes = [_int]
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
 lib.fp6m_mul_fused.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _vp, _vp,
                                _vp, _vp, _int]
@@ -45,7 +46,7 @@ lib.fp6m_int4_quantize.argtypes = [_vp, _sz, _sz, _int, _vp, _vp, _vp]
 lib.fp6m_int4_pack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_permute_scales.argtypes = [_vp, _vp, _sz]
 lib.fp6m_unpack_to_fp16.argtypes = [_vp, _vp, _vp, _sz, _sz, _int, _int]
-for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_repack_gfx950, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
+for _f in (lib.fp6m_init, lib.fp6m_init_gather, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_repack_gfx950, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
            lib.fp6m_int4_quantize, lib.fp6m_int4_pack, lib.fp6m_permute_scales, lib.fp6m_unpack_to_fp16):
     _f.restype = _int
 
@@ -184,8 +185,10 @@ def workspace_elems(n, max_par=16):
     return int(lib.fp6m_workspace_elems(n, max_par))
 
 
-def init(device=0):
-    code = lib.fp6m_init(int(device))
+def init(device=0, gather=False):
+    """Allocate the per-device scratch now (and, with `gather`, the buffer that `a_cols` gathers pass through)
+    instead of on first use: call it before HIP-graph capture or any other region that must not allocate."""
+    code = lib.fp6m_init_gather(int(device)) if gather else lib.fp6m_init(int(device))
     if code != OK:
         raise RuntimeError(f"fp6m_init: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
 

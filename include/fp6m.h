@@ -138,6 +138,9 @@ size_t fp6m_workspace_elems(int prob_n, int max_par);
  * must not allocate).  No counterpart in the reference (which reduces through C in fp16).
  */
 int fp6m_init(int dev);
+/* The same for the 64 MiB buffer that gathered activations pass through (a_cols of fp6m_mul_fused / fp6m_mul_rows):
+ * allocated by the first gathering call on a device, or eagerly here.  No counterpart in the reference. */
+int fp6m_init_gather(int dev);
 
 /*
  * FP16 -> FP6 (e3m2) row quantiser.  Replaces

@@ -164,3 +164,50 @@ def test_fused_argument_errors():
     fp6_marlin.mul_fused(A, B, C, s, ws)                               # nothing to fuse: plain GEMM
     torch.cuda.synchronize()
     assert float(C.abs().sum()) == 0
+
+
+def test_graph_replays_of_fused_and_row_mix_calls(oracle):
+    """`mul`, `mul_fused` (gather + scatter + bias + residual) and `mul_rows` captured in one HIP graph: every
+    replay, with eager work and synchronisation in between, reproduces the eager results bit for bit."""
+    import fp6_marlin
+    m, k, n, qc, gs, qr = 16, 1024, 512, 256, 128, 256
+    ref, B, s = packed(oracle, k, n, qc, gs, seed=21)
+    w = np.random.default_rng(22).normal(0, 0.02, (k, n)).astype(np.float16)
+    _, br, sr = oracle.gen_row_mix_weight(w, qr)
+    Br, Sr = torch.from_numpy(br).to(dev()), torch.from_numpy(sr).to(dev())
+    g = torch.Generator().manual_seed(23)
+    A = torch.randn((m, k), generator=g).half().to(dev())
+    a_cols = torch.randperm(k, generator=g).to(torch.int32).to(dev())
+    c_cols = torch.randperm(n, generator=g).to(torch.int32).to(dev())
+    bias = torch.randn(n, generator=g).half().to(dev())
+    res = torch.randn((m, n), generator=g).half().to(dev())
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+    outs = [torch.empty((m, n), dtype=torch.half, device=dev()) for _ in range(3)]
+    fp6_marlin.init(0, gather=True)                                     # nothing may allocate during capture
+
+    def work():
+        fp6_marlin.mul(A, B, outs[0], s, ws, qc, -1, -1, -1, 16, gs)
+        fp6_marlin.mul_fused(A, B, outs[1], s, ws, qc, gs, a_cols=a_cols, c_cols=c_cols, bias=bias, residual=res)
+        fp6_marlin.mul_rows(A, Br, outs[2], Sr, ws, qr, a_cols=a_cols)
+
+    work()
+    torch.cuda.synchronize()
+    eager = [o.clone() for o in outs]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        work()                                                          # warm-up on the capture stream
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        work()
+    for rep in range(4):
+        for o in outs:
+            o.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, e in zip(outs, eager):
+            assert torch.equal(o, e), rep
+        assert int(ws.abs().sum()) == 0
+        fp6_marlin.mul(A, B, outs[0], s, ws, qc, -1, -1, -1, 16, gs)     # eager work between replays
+        torch.cuda.synchronize()
