@@ -21,6 +21,8 @@ What each function follows (paths relative to the reference checkout):
 ``gen_int4_weight``    ``test.py:85-121``
 ``gen_mixed_weight``   ``test.py:123-152`` (the wire format of ``B`` and ``s``)
 ``matmul_ref``         ``test.py:165-167`` (dequantise-then-matmul), fp32 here
+``gen_row_mix_weight`` no counterpart: ``gen_int4_weight`` on the first rows,
+                       ``gen_fp6_weight`` on the last ones (same columns)
 =====================  ======================================================
 
 Pinning of the ctypes-bound functions is described at the top of
@@ -32,6 +34,11 @@ and the PTX ``mma.m16n8k16`` fragment maps).  ``int4_quantize`` with
 per-channel only, ``fp6_marlin_cuda_kernel.cu:447-448``): it is the same
 formula applied per 128-row group, and is **parity unpinned** against the
 reference by construction; it is checked against its closed form only.
+``gen_row_mix_weight`` is likewise **parity unpinned** against the reference
+(which mixes along columns only, ``fp6_marlin_cuda_kernel.cu:308-337``): it
+concatenates the outputs of two pinned generators, and
+``tests/test_oracle_pins.py`` checks that its packed words decode, with the
+kernel's decode rules, to the check weight it returns.
 """
 import ctypes
 import os

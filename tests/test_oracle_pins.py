@@ -228,3 +228,32 @@ def test_mixed_wire_format(oracle):
     assert b_all4.size == k // 16 * 2 * n
     _, b_all6, _ = oracle.gen_mixed_weight(w[:, :256].copy(), 256)
     assert b_all6.size == k * 3 // 32 * 2 * 256
+
+
+def test_row_mix_wire_format(oracle):
+    """The row-mixed operands (no reference counterpart): the INT4 words of the first rows and the FP6 planes of the
+    last rows decode, with the kernel's decode rules, to the check weight the function returns; sizes and scale
+    layout are those the GEMM entry documents."""
+    rng = np.random.default_rng(8)
+    k, n, qr = 384, 256, 128
+    k4 = k - qr
+    w = rng.normal(0, 0.02, (k, n)).astype(np.float16)
+    ref, b, s = oracle.gen_row_mix_weight(w, qr)
+    words4 = k4 * n // 8
+    assert b.dtype == np.int32 and b.size == words4 + qr * n * 3 // 16
+    assert s.size == (k4 // 128) * n + n and ref.shape == (k, n)
+    i4 = kr.decode_int4(b[:words4], k4, n)                               # nibble - 8
+    s4 = s[: (k4 // 128) * n].reshape(k4 // 128, n)                      # natural column order, one row per group
+    assert np.array_equal((i4 * np.repeat(s4, 128, axis=0)).astype(np.float16), ref[:k4])
+    f6 = kr.decode_fp6(b[words4:], qr, n)
+    s6 = s[(k4 // 128) * n:]
+    s6_nat = np.array([s6[32 * (c // 32) + kr.scale_slot(c % 32)] for c in range(n)], dtype=np.float16)
+    assert np.array_equal((f6 * s6_nat[None, :]).astype(np.float16), ref[k4:])
+    # the shipped packer builds the same buffers from the same two routines (FP6 part in the harness layout)
+    import torch
+    import fp6_marlin
+    wt = torch.from_numpy(w)
+    b4, s4p, r4 = fp6_marlin.pack_mixed_weight(wt[:k4].contiguous(), -1, 128)
+    b6, s6p, r6 = fp6_marlin.pack_mixed_weight(wt[k4:].contiguous(), n, -1, harness_layout=True)
+    assert np.array_equal(torch.cat([b4, b6]).numpy(), b) and np.array_equal(torch.cat([s4p, s6p]).numpy(), s)
+    assert np.array_equal(torch.cat([r4, r6], 0).numpy(), ref)
