@@ -121,6 +121,22 @@ int pack_temp(int dev, void** ptr)
     return FP6M_OK;
 }
 
+inline SliceRule make_rule(int units, int nslices)
+{
+    SliceRule r;
+    r.q = units / nslices;
+    r.first_long = nslices - units % nslices;
+    return r;
+}
+
+inline FastDiv make_div(long long d, long long max_n)
+{
+    FastDiv f;
+    f.d = (uint32_t)d;
+    f.magic = d > 1 && d < 65536 && max_n < 65536 ? (uint32_t)((0x100000000ULL + (unsigned long long)d - 1) / (unsigned long long)d) : 0;
+    return f;
+}
+
 // m <= 16 configurations: rows of A per ring slot, WN x WK waves, ring depths of INT4 / FP6 tiles.
 //   0: rows <= 4,  one tile x four k slices per workgroup, four ring slots (three for FP6 tiles)
 //   1: rows <= 16, same shape, 1 KiB of A per slot
@@ -366,6 +382,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (ks < 1) ks = 1;
             while (ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > kScratchBytes) ks--;
             a.ksplit = (int)ks;
+            a.rule[0] = a.rule[1] = make_rule(units, a.ksplit * wk);
+            a.div[0] = a.div[1] = make_div(a.ksplit, (long long)(a.groups6 + a.groups4) * a.ksplit);
             dim3 grid((unsigned)((a.groups6 + a.groups4) * a.ksplit), (unsigned)groups_m);
             if (getenv("FP6M_VERBOSE"))
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: shared fragments, %d tile(s) x %d k slice(s), row tiles %d ks=%d grid=%ux%u\n",
@@ -402,8 +420,16 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (row_mix) {
                 a.ks6 = 0;                                            // no FP6 column region: groups6 is 0
                 a.slices4 = deal_slices(a.ks4 * cfg.wk);
+                a.rule[0] = make_rule(k4 / 128, a.slices4);
+                a.rule[1] = make_rule(fu.quant_rows / 64, a.ks4 * cfg.wk - a.slices4);
+            } else {
+                a.rule[0] = make_rule(units, a.ks4 * cfg.wk);
+                a.rule[1] = make_rule(units, (a.ks6 > 0 ? a.ks6 : 1) * cfg.wk);
             }
-            dim3 grid((unsigned)(a.groups6 * a.ks6 + a.groups4 * a.ks4), 1);
+            const long long wgs = (long long)a.groups6 * a.ks6 + (long long)a.groups4 * a.ks4;
+            a.div[0] = make_div(a.groups4, wgs);
+            a.div[1] = make_div(a.groups6, wgs);
+            dim3 grid((unsigned)wgs, 1);
             if (getenv("FP6M_VERBOSE"))
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u\n", a.m, prob_n,
                         prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x);
@@ -427,7 +453,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
             int wk = base * ks <= scratch->cus && units / 16 >= ks ? 8 : kWaves;
             if (const char* e = getenv("FP6M_WK")) wk = atoi(e) == 8 ? 8 : kWaves;   // tuning/testing override
-            if (row_mix) a.slices4 = deal_slices(a.ksplit * wk);
+            if (row_mix) {
+                a.slices4 = deal_slices(a.ksplit * wk);
+                a.rule[0] = make_rule(k4 / 128, a.slices4);
+                a.rule[1] = make_rule(fu.quant_rows / 64, a.ksplit * wk - a.slices4);
+            } else {
+                a.rule[0] = a.rule[1] = make_rule(units, a.ksplit * wk);
+            }
+            a.div[0] = a.div[1] = make_div(a.ksplit, (long long)a.tiles * a.ksplit);
             dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
             if (getenv("FP6M_VERBOSE"))
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d k slices %d grid=%ux%u\n", a.m, prob_n, prob_k,

@@ -22,6 +22,29 @@ constexpr int kRedStride = kTileN + 4;                       // floats per row o
 constexpr size_t kScratchBytes = size_t(64) << 20;           // per-device partial-sum scratch
 constexpr size_t kPackTempBytes = size_t(1) << 20;           // + the packer's flag and per-column maxima
 
+// Slice i of a tile's k range, in units (two k steps; four with group scales): the first `first_long` slices hold q
+// units, the others q + 1, so that inside a workgroup the longer slices come last (the lock-step kernel lets every
+// wave run the longest slice's step count from its own begin, which must stay inside k).
+struct SliceRule {
+    int q, first_long;
+};
+__host__ __device__ inline int slice_begin(const SliceRule& r, int i)
+{
+    const int extra = i - r.first_long;
+    return i * r.q + (extra > 0 ? extra : 0);
+}
+
+// n / d for n, d < 65536 as the high half of n * ceil(2^32 / d) (exact in that range: the error term n * e / 2^32 stays
+// below 1 / d); magic 0 stands for a plain division (d = 1, or operands out of range).
+struct FastDiv {
+    uint32_t d, magic;
+};
+__device__ __forceinline__ int fast_div(const FastDiv& f, int n)
+{
+    if (f.magic) return (int)__umulhi((uint32_t)n, f.magic);
+    return f.d == 1 ? n : n / (int)f.d;
+}
+
 struct GemmArgs {
     const uint16_t* A;
     const uint32_t* b_int4;   // INT4 words
@@ -43,6 +66,10 @@ struct GemmArgs {
     // row mix (fp6m_mul_rows): rows [0, k4) of every column are INT4 with group scales, rows [k4, k) FP6.  The
     // k slices of a tile (parts x waves) are numbered INT4 first: slices [0, slices4) cover the INT4 rows.
     int k4, slices4;          // 0 = column mix
+    // Division-free bookkeeping, prepared by the host (a 64-bit division costs a wave hundreds of scalar
+    // instructions before its first load):
+    SliceRule rule[2];        // k slices of a tile: [0] INT4 tiles / INT4 rows (all tiles for m > 16), [1] FP6
+    FastDiv div[2];           // m <= 16: by groups4 / groups6;  m > 16: [0] by ksplit
     // weight planes in the gfx950 order (fp6m_repack_gfx950): [tile][k-block][MFMA lane] instead of the reference's
     // [k-block][64-column group][fragment owner]
     int native;
@@ -122,19 +149,17 @@ struct TileInfo {
     int a_step0;             // k step of A that step 0 of the wave's weight segment multiplies (row mix: k4 / 32)
 };
 
-// Row mix: slice `sl` of the `nsl` slices of a tile -> its segment (ti.fp6, ti.a_step0) and its steps there.
-__device__ __forceinline__ void row_mix_slice(const GemmArgs& p, int sl, int nsl, TileInfo& ti, int& begin, int& end)
+// Row mix: slice `sl` of a tile's slices -> its segment (ti.fp6, ti.a_step0) and its steps there.
+__device__ __forceinline__ void row_mix_slice(const GemmArgs& p, int sl, TileInfo& ti, int& begin, int& end)
 {
     ti.fp6 = sl >= p.slices4;
     if (!ti.fp6) {
-        const int units = p.k4 / 128;
-        begin = (int)((long long)units * sl / p.slices4) * 4;
-        end = (int)((long long)units * (sl + 1) / p.slices4) * 4;
+        begin = slice_begin(p.rule[0], sl) * 4;
+        end = slice_begin(p.rule[0], sl + 1) * 4;
         ti.a_step0 = 0;
     } else {
-        const int units = (p.k - p.k4) / 64, s6 = sl - p.slices4, n6 = nsl - p.slices4;
-        begin = (int)((long long)units * s6 / n6) * 2;
-        end = (int)((long long)units * (s6 + 1) / n6) * 2;
+        begin = slice_begin(p.rule[1], sl - p.slices4) * 2;
+        end = slice_begin(p.rule[1], sl - p.slices4 + 1) * 2;
         ti.a_step0 = p.k4 / 32;
     }
 }
@@ -168,7 +193,7 @@ __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 {
     TileInfo t;
     const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    t.tile = logical / p.ksplit;
+    t.tile = fast_div(p.div[0], logical);
     t.part = logical - t.tile * p.ksplit;
     t.mtile = blockIdx.y;
     t.fp6 = t.tile < p.tiles6;
@@ -185,11 +210,9 @@ template <bool G128, int WK = kWaves>
 __device__ __forceinline__ void wave_k_range(const GemmArgs& p, int part, int wave, int& begin, int& end)
 {
     constexpr int unit_steps = G128 ? 4 : 2;
-    const int units = p.k / (32 * unit_steps);
-    const int nwaves = p.ksplit * WK;
     const int wv = part * WK + wave;
-    begin = (int)((long long)units * wv / nwaves) * unit_steps;
-    end = (int)((long long)units * (wv + 1) / nwaves) * unit_steps;
+    begin = slice_begin(p.rule[0], wv) * unit_steps;
+    end = slice_begin(p.rule[0], wv + 1) * unit_steps;
 }
 
 // ------------------------------------------------------------------------------------------------ loads, waits, dequantisers

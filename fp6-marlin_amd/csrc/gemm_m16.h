@@ -363,7 +363,7 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     const int local = ti.fp6 ? logical : logical - wgs6;
     const int groups = ti.fp6 ? p.groups6 : p.groups4;
     const int ks = ti.fp6 ? p.ks6 : p.ks4;
-    ti.part = local / groups;                                            // part-major: neighbours share k, adjoin in n
+    ti.part = fast_div(p.div[ti.fp6 ? 1 : 0], local);                    // part-major: neighbours share k, adjoin in n
     const int group = local - ti.part * groups;
     ti.tcol = group * WN + wn;
     ti.region_n = ti.fp6 ? p.qc : p.n4;
@@ -373,13 +373,12 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     ti.col0 = (ti.fp6 ? p.n4 : 0) + ti.tcol * kTileN;
 
     constexpr int unit_steps = G128 ? 4 : 2;
-    const int units = p.k / (32 * unit_steps);
-    const int kp = ti.part * WK + wk, kparts = ks * WK;
-    int step_begin = (int)((long long)units * kp / kparts) * unit_steps;
-    int step_end = (int)((long long)units * (kp + 1) / kparts) * unit_steps;
+    const int kp = ti.part * WK + wk;
+    int step_begin = slice_begin(p.rule[ti.fp6 ? 1 : 0], kp) * unit_steps;
+    int step_end = slice_begin(p.rule[ti.fp6 ? 1 : 0], kp + 1) * unit_steps;
     ti.a_step0 = 0;
     const bool region6 = ti.fp6;                                         // the workgroup's column region
-    if (p.k4) row_mix_slice(p, kp, kparts, ti, step_begin, step_end);    // per wave: INT4 or FP6 rows of the tile
+    if (p.k4) row_mix_slice(p, kp, ti, step_begin, step_end);            // per wave: INT4 or FP6 rows of the tile
 
     f4 acc[1][8];
 #pragma unroll

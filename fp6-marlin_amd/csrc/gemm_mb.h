@@ -490,7 +490,7 @@ __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int step_begin, step_end;
     wave_k_range<G128, WK>(p, ti.part, wave, step_begin, step_end);
-    if (p.k4) row_mix_slice(p, ti.part * WK + wave, p.ksplit * WK, ti, step_begin, step_end);
+    if (p.k4) row_mix_slice(p, ti.part * WK + wave, ti, step_begin, step_end);
 
     f4 acc[MB][8];
 #pragma unroll

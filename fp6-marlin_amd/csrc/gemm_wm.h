@@ -311,7 +311,7 @@ __global__ __launch_bounds__(512, 2) void gemm_wm_kernel(const GemmArgs p)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave % WM, wn = WN == 2 ? wave / WM : 0, wk = WN == 2 ? 0 : wave / WM;
     const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    const int group = logical / p.ksplit;                            // WN adjacent tiles of one region
+    const int group = fast_div(p.div[0], logical);                   // WN adjacent tiles of one region
     TileInfo ti;
     ti.part = logical - group * p.ksplit;
     ti.fp6 = group < p.groups6;
@@ -329,22 +329,15 @@ __global__ __launch_bounds__(512, 2) void gemm_wm_kernel(const GemmArgs p)
     ti.col0 = (ti.fp6 ? p.n4 : 0) + tcol * kTileN;
     ti.a_step0 = 0;
 
-    // k slices: part-major, then wk; every wave of the workgroup runs the longest slice's step count
+    // k slices: part-major, then wk; every wave of the workgroup runs the longest slice's step count.  Longer
+    // slices come last (SliceRule), so begin + longest stays inside k for every slice that has work; a slice
+    // without work keeps step with the others on steps [0, longest).
     constexpr int unit_steps = G128 ? 4 : 2;
-    const int units = p.k / (32 * unit_steps);
-    const int nslices = p.ksplit * WK;
-    int step_begin = 0, step_end = 0, longest = 0;
-#pragma unroll
-    for (int q = 0; q < WK; q++) {
-        const int sl = ti.part * WK + q;
-        const int b = (int)((long long)units * sl / nslices) * unit_steps;
-        const int e = (int)((long long)units * (sl + 1) / nslices) * unit_steps;
-        if (q == wk) {
-            step_begin = b;
-            step_end = e;
-        }
-        longest = e - b > longest ? e - b : longest;
-    }
+    const int sl = ti.part * WK + wk;
+    int step_begin = slice_begin(p.rule[0], sl) * unit_steps;
+    int step_end = slice_begin(p.rule[0], sl + 1) * unit_steps;
+    const int longest = (p.rule[0].q + (ti.part * WK + WK - 1 >= p.rule[0].first_long ? 1 : 0)) * unit_steps;
+    if (step_begin == step_end) step_begin = step_end = 0;
 
     f4 acc[MB][8];
 #pragma unroll
