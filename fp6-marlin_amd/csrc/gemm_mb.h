@@ -347,12 +347,18 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
 // `smem`, `flag` and `valid` belong to the WK waves that share a tile and a row tile (the whole workgroup in
 // gemm_mb_kernel, one of WM groups in gemm_wm_kernel); a group without rows goes through the barriers
 // without touching memory.
-template <int MB, int WK = kWaves>
+template <int MB, int WK = kWaves, int BPR = 1>
 __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, f4 (&acc)[MB][8],
                                              bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
                                              bool valid = true, int first_fp6 = WK)
 {
-    constexpr int RMAX = 16 / WK, PCHUNK = 32 / RMAX;                // parts whose loads are in flight together
+    // BPR: 16-row blocks per round of the reduction through LDS (a wave's region holds BPR * 16 rows of kRedStride
+    // floats).  The rounds are bound by LDS bandwidth (every wave writes and reads its whole accumulator once) plus two
+    // barriers each, so fewer rounds help; the gather below keeps the loads of up to 32 rows in flight per lane.
+    static_assert(MB % BPR == 0, "whole rounds");
+    constexpr int RMAX = 16 / WK;                                    // rows of a block one wave finishes
+    constexpr int MBC = MB < (32 / RMAX > 0 ? 32 / RMAX : 1) ? MB : (32 / RMAX > 0 ? 32 / RMAX : 1);   // blocks per gather round
+    constexpr int PCH = 32 / (MBC * RMAX) > 0 ? 32 / (MBC * RMAX) : 1;                                 // parts per gather round
     typedef float f2 __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x & 63;
     const bool leader = lane == 0 && wk == 0;
@@ -389,33 +395,55 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
 
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
+    for (int mb0 = 0; mb0 < MB; mb0 += BPR) {
         __syncthreads();
+        if (mb0 == 0) FP6M_MARK(p, 1);                               // every wave of the group has left its loop
         float* mine = reinterpret_cast<float*>(smem + wk * wave_lds) + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
 #pragma unroll
-        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[mb][t];
+        for (int b = 0; b < BPR; b++)
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                *reinterpret_cast<f4*>(mine + b * 16 * kRedStride + 16 * (t >> 1) + 8 * (t & 1)) = acc[mb0 + b][t];
         __syncthreads();
+        // all LDS reads of the round first (rows beyond m are read too: the slab is there), one wait, then the sums
+        f2 tv[BPR][RMAX][WK];
 #pragma unroll
-        for (int r = 0; r < RMAX; r++) {
-            const int m = wk + r * WK, row = 16 * mb + m;
-            if (row < nrows) {
+        for (int b = 0; b < BPR; b++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++)
+#pragma unroll
+                for (int j = 0; j < WK; j++)
+                    tv[b][r][j] = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + j * wave_lds) +
+                                                               (b * 16 + wk + r * WK) * kRedStride + 2 * lane);
+#pragma unroll
+        for (int b = 0; b < BPR; b++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                const int row = 16 * (mb0 + b) + wk + r * WK;
                 float v0 = 0.f, v1 = 0.f;
+                if (first_fp6 >= WK) {                               // (uniform) the usual case: plain sums
 #pragma unroll
-                for (int j = 0; j < WK; j++) {
-                    const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + j * wave_lds) +
-                                                              m * kRedStride + 2 * lane);
-                    v0 += j >= first_fp6 ? v[0] * x0 : v[0];
-                    v1 += j >= first_fp6 ? v[1] * x1 : v[1];
-                }
-                if (ks == 1) {
-                    store_row(row, v0, v1);
+                    for (int j = 0; j < WK; j++) {
+                        v0 += tv[b][r][j][0];
+                        v1 += tv[b][r][j][1];
+                    }
                 } else {
-                    const f2 v = {v0, v1};
-                    __hip_atomic_store(my + (size_t)row * (kTileN / 2), __builtin_bit_cast(unsigned long long, v),
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int j = 0; j < WK; j++) {
+                        v0 += j >= first_fp6 ? tv[b][r][j][0] * x0 : tv[b][r][j][0];
+                        v1 += j >= first_fp6 ? tv[b][r][j][1] * x1 : tv[b][r][j][1];
+                    }
+                }
+                if (row < nrows) {
+                    if (ks == 1) {
+                        store_row(row, v0, v1);
+                    } else {
+                        const f2 v = {v0, v1};
+                        __hip_atomic_store(my + (size_t)row * (kTileN / 2), __builtin_bit_cast(unsigned long long, v),
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
             }
-        }
     }
     if (ks == 1) return;
 
@@ -432,40 +460,49 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     if (!*flag) return;
     FP6M_MARK(p, 5);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // The last arrival sums all parts in part order: MBC blocks at a time, PCH parts' loads in flight together.
 #pragma unroll 1
-    for (int mb = 0; mb < MB; mb++) {
-        float v0[RMAX], v1[RMAX];
+    for (int mb0 = 0; mb0 < MB; mb0 += MBC) {
+        float v0[MBC][RMAX], v1[MBC][RMAX];
 #pragma unroll
-        for (int r = 0; r < RMAX; r++) {
-            v0[r] = 0.f;
-            v1[r] = 0.f;
+        for (int b = 0; b < MBC; b++)
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                v0[b][r] = 0.f;
+                v1[b][r] = 0.f;
+            }
+        for (int pp = 0; pp < ks; pp += PCH) {
+            unsigned long long t[PCH][MBC][RMAX];
+#pragma unroll
+            for (int u = 0; u < PCH; u++)
+#pragma unroll
+                for (int b = 0; b < MBC; b++)
+#pragma unroll
+                    for (int r = 0; r < RMAX; r++) {
+                        const int row = 16 * (mb0 + b) + wk + r * WK;
+                        t[u][b][r] = 0;
+                        if (row < nrows && pp + u < ks)
+                            t[u][b][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + (size_t)row * (kTileN / 2),
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+            for (int u = 0; u < PCH; u++)
+#pragma unroll
+                for (int b = 0; b < MBC; b++)
+#pragma unroll
+                    for (int r = 0; r < RMAX; r++) {
+                        const f2 v = __builtin_bit_cast(f2, t[u][b][r]);
+                        v0[b][r] += v[0];
+                        v1[b][r] += v[1];
+                    }
         }
-        for (int pp = 0; pp < ks; pp += PCHUNK) {
-            unsigned long long t[PCHUNK][RMAX];
 #pragma unroll
-            for (int u = 0; u < PCHUNK; u++)
+        for (int b = 0; b < MBC; b++)
 #pragma unroll
-                for (int r = 0; r < RMAX; r++) {
-                    const int row = 16 * mb + wk + r * WK;
-                    t[u][r] = 0;
-                    if (row < nrows && pp + u < ks)
-                        t[u][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + (size_t)row * (kTileN / 2),
-                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-#pragma unroll
-            for (int u = 0; u < PCHUNK; u++)
-#pragma unroll
-                for (int r = 0; r < RMAX; r++) {
-                    const f2 v = __builtin_bit_cast(f2, t[u][r]);
-                    v0[r] += v[0];
-                    v1[r] += v[1];
-                }
-        }
-#pragma unroll
-        for (int r = 0; r < RMAX; r++) {
-            const int row = 16 * mb + wk + r * WK;
-            if (row < nrows) store_row(row, v0[r], v1[r]);
-        }
+            for (int r = 0; r < RMAX; r++) {
+                const int row = 16 * (mb0 + b) + wk + r * WK;
+                if (row < nrows) store_row(row, v0[b][r], v1[b][r]);
+            }
     }
     // the counter is next touched by a later launch on the stream: the reset needs no ordering here
     if (leader) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -505,7 +542,8 @@ __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const
             stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
     }
     FP6M_MARK(p, 2);
-    wg_finish_mb<MB, WK>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+    constexpr int BPR = kWaveLds >= 2 * 16 * kRedStride * 4 ? 2 : 1;  // the drained rings hold two blocks per wave
+    wg_finish_mb<MB, WK, BPR>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
                          reinterpret_cast<int*>(smem + WK * kWaveLds), true, p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
 }
