@@ -291,6 +291,11 @@ def fused_bench(args):
     probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
     a_cols = torch.randperm(k, generator=gen).to(torch.int32).cuda()
     c_cols = torch.randperm(n, generator=gen).to(torch.int32).cuda()
+    # the map a Layer with chosen FP6 output features uses: the other features in order, then the chosen ones
+    picked = torch.randperm(n, generator=gen)[:qc if qc else 256].sort().values
+    keep = torch.ones(n, dtype=torch.bool)
+    keep[picked] = False
+    c_layer = torch.cat([torch.nonzero(keep).reshape(-1), picked]).to(torch.int32).cuda()
     inv = torch.argsort(c_cols.long())
     bias = torch.randn(n, generator=gen).half().cuda()
     res = torch.randn((m, n), generator=gen).half().cuda()
@@ -313,7 +318,8 @@ def fused_bench(args):
         torch.index_select(p.C, 1, inv, out=out)
         out.add_(bias).add_(res)
 
-    variants = {"mul": plain, "fused_scatter": fused(c_cols=c_cols), "fused_gather": fused(a_cols=a_cols),
+    variants = {"mul": plain, "fused_scatter": fused(c_cols=c_cols), "fused_scatter_layer_map": fused(c_cols=c_layer),
+                "fused_gather": fused(a_cols=a_cols),
                 "fused_bias_residual": fused(bias=bias, residual=res),
                 "fused_all": fused(a_cols=a_cols, c_cols=c_cols, bias=bias, residual=res), "torch_kernels_around_mul": around}
     row = {"fused": f"m={m} {k}x{n} qc={qc} gs={gs}"}

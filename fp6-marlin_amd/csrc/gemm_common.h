@@ -113,29 +113,44 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int total)
     return x * q + (x < r ? x : r) + (b >> 3);
 }
 
-// Epilogue of fp6m_mul_fused for two adjacent packed columns of one row: C[row, c_cols[col]] =
+// Epilogue of fp6m_mul_fused for the two adjacent packed columns a lane owns: C[row, c_cols[col]] =
 // fp16(v + bias[c_cols[col]] + residual[row, c_cols[col]]), everything added in fp32 and rounded once.
+// The lane's destination columns and bias are looked up once (FusedCols), the rows then only add and store.
 // Map entries are clamped to the row so that a bad map cannot write outside C.
-__device__ __forceinline__ void store_fused(const GemmArgs& p, size_t row, int col, float v0, float v1)
+struct FusedCols {
+    int c0, c1;
+    float b0, b1;
+};
+__device__ __forceinline__ FusedCols fused_cols(const GemmArgs& p, int col)
 {
-    int c0 = col, c1 = col + 1;
+    FusedCols f;
+    f.c0 = col;
+    f.c1 = col + 1;
+    f.b0 = f.b1 = 0.f;
+    if (!p.fused) return f;
     if (p.c_cols) {
-        c0 = p.c_cols[col];
-        c1 = p.c_cols[col + 1];
-        c0 = c0 < 0 ? 0 : (c0 >= p.n ? p.n - 1 : c0);
-        c1 = c1 < 0 ? 0 : (c1 >= p.n ? p.n - 1 : c1);
+        f.c0 = p.c_cols[col];
+        f.c1 = p.c_cols[col + 1];
+        f.c0 = f.c0 < 0 ? 0 : (f.c0 >= p.n ? p.n - 1 : f.c0);
+        f.c1 = f.c1 < 0 ? 0 : (f.c1 >= p.n ? p.n - 1 : f.c1);
     }
     if (p.bias) {
-        v0 += (float)__builtin_bit_cast(_Float16, p.bias[c0]);
-        v1 += (float)__builtin_bit_cast(_Float16, p.bias[c1]);
+        f.b0 = (float)__builtin_bit_cast(_Float16, p.bias[f.c0]);
+        f.b1 = (float)__builtin_bit_cast(_Float16, p.bias[f.c1]);
     }
+    return f;
+}
+__device__ __forceinline__ void store_fused(const GemmArgs& p, const FusedCols& f, size_t row, float v0, float v1)
+{
+    v0 += f.b0;
+    v1 += f.b1;
     const size_t r = row * (size_t)p.n;
     if (p.residual) {
-        v0 += (float)__builtin_bit_cast(_Float16, p.residual[r + c0]);
-        v1 += (float)__builtin_bit_cast(_Float16, p.residual[r + c1]);
+        v0 += (float)__builtin_bit_cast(_Float16, p.residual[r + f.c0]);
+        v1 += (float)__builtin_bit_cast(_Float16, p.residual[r + f.c1]);
     }
-    p.C[r + c0] = __builtin_bit_cast(uint16_t, (_Float16)v0);
-    p.C[r + c1] = __builtin_bit_cast(uint16_t, (_Float16)v1);
+    p.C[r + f.c0] = __builtin_bit_cast(uint16_t, (_Float16)v0);
+    p.C[r + f.c1] = __builtin_bit_cast(uint16_t, (_Float16)v1);
 }
 
 // ------------------------------------------------------------------------------------------------ tile bookkeeping

@@ -254,9 +254,10 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
         x1 = (float)sv[1];
     }
     uint16_t* c_out = p.C + ti.col0 + 2 * lane;
+    const FusedCols fcols = fused_cols(p, tile_valid ? ti.col0 + 2 * lane : 0);
     auto store_row = [&](int m, float v0, float v1) {
         if (p.fused) {
-            store_fused(p, (size_t)m, ti.col0 + 2 * lane, v0 * s0, v1 * s1);
+            store_fused(p, fcols, (size_t)m, v0 * s0, v1 * s1);
             return;
         }
         h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};

@@ -381,9 +381,10 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
         x1 = (float)sv[1];
     }
     uint16_t* c_out = p.C + (size_t)row0 * p.n + ti.col0 + 2 * lane;
+    const FusedCols fcols = fused_cols(p, ti.col0 + 2 * lane);
     auto store_row = [&](int row, float v0, float v1) {
         if (p.fused) {
-            store_fused(p, (size_t)(row0 + row), ti.col0 + 2 * lane, v0 * s0, v1 * s1);
+            store_fused(p, fcols, (size_t)(row0 + row), v0 * s0, v1 * s1);
             return;
         }
         h2 o = {(_Float16)(v0 * s0), (_Float16)(v1 * s1)};
