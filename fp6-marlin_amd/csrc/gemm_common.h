@@ -113,6 +113,19 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int total)
     return x * q + (x < r ? x : r) + (b >> 3);
 }
 
+// Kernel arguments are fetched with scalar loads that the compiler otherwise issues where each field is first used:
+// three or four dependent round trips (0.2-0.4 us each on a cold kernarg buffer) before a wave's first weight load.
+// Naming the fields in one asm statement at the top makes them one batch behind a single wait.
+__device__ __forceinline__ void preload_args(const GemmArgs& p)
+{
+    asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
+                        "s"(p.scratch), "s"(p.counters));
+    asm volatile("" : : "s"(p.m), "s"(p.n), "s"(p.k), "s"(p.n4), "s"(p.qc), "s"(p.tiles6), "s"(p.tiles), "s"(p.ksplit),
+                        "s"(p.ks6), "s"(p.ks4), "s"(p.groups6), "s"(p.groups4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
+    asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
+                        "s"(p.div[0].d), "s"(p.div[0].magic), "s"(p.div[1].d), "s"(p.div[1].magic), "s"(p.fused));
+}
+
 // Epilogue of fp6m_mul_fused for the two adjacent packed columns a lane owns: C[row, c_cols[col]] =
 // fp16(v + bias[c_cols[col]] + residual[row, c_cols[col]]), everything added in fp32 and rounded once.
 // The lane's destination columns and bias are looked up once (FusedCols), the rows then only add and store.

@@ -265,19 +265,31 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
     };
 
     // Sum of the WK slices of my rows.
+    // All LDS reads first (rows beyond m and waves without a tile read whatever the slab holds; it is never stored),
+    // one wait, then the sums in slice order.
+    f2 tv[RMAX][WK];
+#pragma unroll
+    for (int r = 0; r < RMAX; r++)
+#pragma unroll
+        for (int j = 0; j < WK; j++)
+            tv[r][j] = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + (j * WN + wn) * wave_lds) +
+                                                    ((wk + r * WK) & 15) * kRedStride + 2 * lane);
     float v0[RMAX], v1[RMAX];
 #pragma unroll
     for (int r = 0; r < RMAX; r++) {
         v0[r] = 0.f;
         v1[r] = 0.f;
-        const int m = wk + r * WK;
-        if (tile_valid && m < nrows) {
+        if (first_fp6 >= WK) {                                           // (uniform) the usual case: plain sums
 #pragma unroll
             for (int j = 0; j < WK; j++) {
-                const f2 v = *reinterpret_cast<const f2*>(reinterpret_cast<const float*>(smem + (j * WN + wn) * wave_lds) +
-                                                          m * kRedStride + 2 * lane);
-                v0[r] += j >= first_fp6 ? v[0] * x0 : v[0];
-                v1[r] += j >= first_fp6 ? v[1] * x1 : v[1];
+                v0[r] += tv[r][j][0];
+                v1[r] += tv[r][j][1];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < WK; j++) {
+                v0[r] += j >= first_fp6 ? tv[r][j][0] * x0 : tv[r][j][0];
+                v1[r] += j >= first_fp6 ? tv[r][j][1] * x1 : tv[r][j][1];
             }
         }
     }
@@ -354,6 +366,7 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);
     __shared__ __attribute__((aligned(16))) unsigned char smem[NW * kWaveLds + 16];
 
+    preload_args(p);
     FP6M_MARK(p, 0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
     const int wn = wave % WN, wk = wave / WN;
@@ -364,7 +377,11 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
     const int local = ti.fp6 ? logical : logical - wgs6;
     const int groups = ti.fp6 ? p.groups6 : p.groups4;
     const int ks = ti.fp6 ? p.ks6 : p.ks4;
-    ti.part = fast_div(p.div[ti.fp6 ? 1 : 0], local);                    // part-major: neighbours share k, adjoin in n
+    // (both entries are read at fixed kernarg offsets and selected by value: an index computed here would turn
+    // into a second, dependent scalar load, which measured 0.4 us before the first weight load)
+    const FastDiv gdiv = {ti.fp6 ? p.div[1].d : p.div[0].d, ti.fp6 ? p.div[1].magic : p.div[0].magic};
+    const SliceRule srule = {ti.fp6 ? p.rule[1].q : p.rule[0].q, ti.fp6 ? p.rule[1].first_long : p.rule[0].first_long};
+    ti.part = fast_div(gdiv, local);                                     // part-major: neighbours share k, adjoin in n
     const int group = local - ti.part * groups;
     ti.tcol = group * WN + wn;
     ti.region_n = ti.fp6 ? p.qc : p.n4;
@@ -375,8 +392,8 @@ __global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArg
 
     constexpr int unit_steps = G128 ? 4 : 2;
     const int kp = ti.part * WK + wk;
-    int step_begin = slice_begin(p.rule[ti.fp6 ? 1 : 0], kp) * unit_steps;
-    int step_end = slice_begin(p.rule[ti.fp6 ? 1 : 0], kp + 1) * unit_steps;
+    int step_begin = slice_begin(srule, kp) * unit_steps;
+    int step_end = slice_begin(srule, kp + 1) * unit_steps;
     ti.a_step0 = 0;
     const bool region6 = ti.fp6;                                         // the workgroup's column region
     if (p.k4) row_mix_slice(p, kp, ti, step_begin, step_end);            // per wave: INT4 or FP6 rows of the tile

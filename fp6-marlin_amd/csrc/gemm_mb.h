@@ -523,6 +523,7 @@ __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const
     static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];
 
+    preload_args(p);
     FP6M_MARK(p, 0);
     TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);

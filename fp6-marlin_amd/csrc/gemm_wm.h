@@ -308,6 +308,7 @@ __global__ __launch_bounds__(512, 2) void gemm_wm_kernel(const GemmArgs p)
     constexpr int MB = 4, WM = kWmRows, WK = 2 / WN;
     __shared__ __attribute__((aligned(16))) unsigned char smem[wm_lds<WN>()];
 
+    preload_args(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave % WM, wn = WN == 2 ? wave / WM : 0, wk = WN == 2 ? 0 : wave / WM;
     const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
