@@ -408,13 +408,41 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (ks > ks_steps) ks = ks_steps;
             if (ks > ks_k) ks = ks_k;
             if (ks > traffic_cap) ks = traffic_cap;
+            if (ks < 1) ks = 1;
+            auto ks6_of = [&](long long c) { return 2 * c <= ks_k ? 2 * c : (c > ks_k ? c : ks_k); };
+            // Second opinion from a small cost model (per-workgroup timelines on MI355X): a wave takes about 0.40 us per
+            // k step when its workgroup has the CU to itself, 0.56 us when two share it, 0.72 us when every CU hosts
+            // two, more beyond; the kernel lasts as long as the longest slice on the busiest CU, plus 2.5 us and
+            // 0.15 us per partner when tiles are split across workgroups.  Grids of exactly one or two workgroups per
+            // CU with equal slices beat the one-and-a-half rule by 4-10 % where the shape allows them; the rule's
+            // choice is kept unless the model sees 8 % or more.
+            {
+                const int unit_steps = g128 ? 4 : 2;
+                auto model_us = [&](long long c) -> double {
+                    const long long c6 = a.groups6 ? ks6_of(c) : 0;
+                    const double load = (double)(a.groups4 * c + a.groups6 * c6) / scratch->cus;
+                    if (load > 3.0) return 1e9;
+                    const double t = load <= 1.0 ? 0.40 : (load <= 1.9 ? 0.56 : (load <= 2.0 ? 0.72 : 1.10));
+                    auto longest = [&](long long slices) { return (double)((units + slices - 1) / slices) * unit_steps; };
+                    double steps = a.groups4 ? longest(c * cfg.wk) : 0.0;
+                    if (a.groups6 && 1.5 * longest(c6 * cfg.wk) > steps) steps = 1.5 * longest(c6 * cfg.wk);
+                    const long long partners = c > c6 ? c : c6;
+                    return steps * t + (partners > 1 ? 2.5 + 0.15 * partners : 0.0);
+                };
+                long long cmax = ks_steps < ks_k ? ks_steps : ks_k;
+                if (cmax > traffic_cap) cmax = traffic_cap;
+                long long best = ks;
+                for (long long c = 1; c <= cmax; c++)
+                    if (model_us(c) < model_us(best)) best = c;
+                if (model_us(best) < 0.92 * model_us(ks)) ks = best;
+            }
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
             const size_t slot_bytes = (size_t)cfg.wn * 16 * kTileN * sizeof(float);
             while (ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > kScratchBytes) ks--;
             a.ks4 = (int)ks;
-            a.ks6 = (int)(2 * ks <= ks_k ? 2 * ks : (ks > ks_k ? ks : ks_k));
+            a.ks6 = (int)ks6_of(ks);
             if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
             a.ksplit = a.ks4;
             if (row_mix) {
