@@ -162,6 +162,13 @@ inline M16Config m16_config(int m)
 
 inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
+    if (cfg.wk == 8) {
+        if (cfg.id == 0)
+            launch_m16<4, 1, 8, 4, 3>(a, g128, grid, stream);
+        else
+            launch_m16<16, 1, 8, 4, 3>(a, g128, grid, stream);
+        return;
+    }
     if (cfg.id == 0)
         launch_m16<4, 1, 4, 4, 3>(a, g128, grid, stream);
     else
@@ -394,55 +401,77 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // FP6 steps cost about twice an INT4 step, so the FP6 region is split twice as finely.  The
             // split is bounded so that every wave keeps at least one k unit, partial-sum traffic stays
             // well below the weight stream and the partial tiles fit the scratch.
-            const M16Config cfg = m16_config(a.m);
+            M16Config cfg = m16_config(a.m);
             a.groups6 = (a.tiles6 + cfg.wn - 1) / cfg.wn;
             a.groups4 = (a.tiles - a.tiles6 + cfg.wn - 1) / cfg.wn;
             const long long groups = a.groups6 + a.groups4;
-            const long long ks_k = units / cfg.wk > 0 ? units / cfg.wk : 1;   // at least one k unit per wave
-            // Measured on MI355X: the kernel is fastest with about one and a half workgroups per CU
-            // (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle), as long as every
-            // wave keeps at least four k steps.
+            const int unit_steps = g128 ? 4 : 2;
+            // Bounds of the split for a workgroup of wk waves: at least one k unit and four k steps per wave, and the
+            // partial-sum traffic well below the weight stream.
+            auto ks_units = [&](int wk) { return units / wk > 0 ? (long long)(units / wk) : 1LL; };
+            auto ks_limit = [&](int wk) {
+                long long c = prob_k / 32 / (4 * wk) > 0 ? prob_k / 32 / (4 * wk) : 1;
+                if (c > ks_units(wk)) c = ks_units(wk);
+                if (c > traffic_cap) c = traffic_cap;
+                return c;
+            };
+            auto ks6_of = [&](long long c, int wk) { return 2 * c <= ks_units(wk) ? 2 * c : (c > ks_units(wk) ? c : ks_units(wk)); };
+            // Measured on MI355X: with four waves per workgroup the kernel is fastest with about one and a half
+            // workgroups per CU (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle).
             const long long target_wgs = (long long)scratch->cus * 3 / 2;
             long long ks = (target_wgs + groups / 2) / groups;
-            const long long ks_steps = prob_k / 32 / (4 * cfg.wk) > 0 ? prob_k / 32 / (4 * cfg.wk) : 1;
-            if (ks > ks_steps) ks = ks_steps;
-            if (ks > ks_k) ks = ks_k;
-            if (ks > traffic_cap) ks = traffic_cap;
+            if (ks > ks_limit(cfg.wk)) ks = ks_limit(cfg.wk);
             if (ks < 1) ks = 1;
-            auto ks6_of = [&](long long c) { return 2 * c <= ks_k ? 2 * c : (c > ks_k ? c : ks_k); };
             // Second opinion from a small cost model (per-workgroup timelines on MI355X): a wave takes about 0.40 us per
-            // k step when its workgroup has the CU to itself, 0.56 us when two share it, 0.72 us when every CU hosts
-            // two, more beyond; the kernel lasts as long as the longest slice on the busiest CU, plus 2.5 us and
-            // 0.15 us per partner when tiles are split across workgroups.  Grids of exactly one or two workgroups per
-            // CU with equal slices beat the one-and-a-half rule by 4-10 % where the shape allows them; the rule's
-            // choice is kept unless the model sees 8 % or more.
+            // k step when its four-wave workgroup has the CU to itself, 0.56 us when the CU hosts eight waves (two such
+            // workgroups, or one of eight waves), 0.72 us when every CU does, 1.1 us beyond; the kernel lasts as long as
+            // the longest slice on the busiest CU, plus 2.5 us and 0.15 us per partner when tiles are split across
+            // workgroups.  Grids of exactly one or two workgroups per CU with equal slices, and eight-wave workgroups
+            // that need no split at all, beat the rule by 4-15 % where the shape allows them; the rule's choice is kept
+            // unless the model sees 8 % or more.
             {
-                const int unit_steps = g128 ? 4 : 2;
-                auto model_us = [&](long long c) -> double {
-                    const long long c6 = a.groups6 ? ks6_of(c) : 0;
+                auto model_us = [&](int wk, long long c) -> double {
+                    const long long c6 = a.groups6 ? ks6_of(c, wk) : 0;
                     const double load = (double)(a.groups4 * c + a.groups6 * c6) / scratch->cus;
-                    if (load > 3.0) return 1e9;
-                    const double t = load <= 1.0 ? 0.40 : (load <= 1.9 ? 0.56 : (load <= 2.0 ? 0.72 : 1.10));
+                    double t;
+                    if (wk == 4) {
+                        if (load > 3.0) return 1e9;
+                        t = load <= 1.0 ? 0.40 : (load <= 1.9 ? 0.56 : (load <= 2.0 ? 0.72 : 1.10));
+                    } else {
+                        // eight waves per workgroup paid off only with one workgroup on (nearly) every CU: measured
+                        // slower both when CUs hosted two of them and when a quarter or more of the CUs stayed idle
+                        if (load > 1.0 || load < 0.75) return 1e9;
+                        t = 0.56;
+                    }
                     auto longest = [&](long long slices) { return (double)((units + slices - 1) / slices) * unit_steps; };
-                    double steps = a.groups4 ? longest(c * cfg.wk) : 0.0;
-                    if (a.groups6 && 1.5 * longest(c6 * cfg.wk) > steps) steps = 1.5 * longest(c6 * cfg.wk);
+                    double steps = a.groups4 ? longest(c * wk) : 0.0;
+                    if (a.groups6 && 1.5 * longest(c6 * wk) > steps) steps = 1.5 * longest(c6 * wk);
                     const long long partners = c > c6 ? c : c6;
                     return steps * t + (partners > 1 ? 2.5 + 0.15 * partners : 0.0);
                 };
-                long long cmax = ks_steps < ks_k ? ks_steps : ks_k;
-                if (cmax > traffic_cap) cmax = traffic_cap;
+                int best_wk = cfg.wk;
                 long long best = ks;
-                for (long long c = 1; c <= cmax; c++)
-                    if (model_us(c) < model_us(best)) best = c;
-                if (model_us(best) < 0.92 * model_us(ks)) ks = best;
+                for (int wk = 4; wk <= 8; wk += 4)
+                    for (long long c = 1; c <= ks_limit(wk); c++)
+                        if (model_us(wk, c) < model_us(best_wk, best)) {
+                            best_wk = wk;
+                            best = c;
+                        }
+                if (model_us(best_wk, best) < 0.92 * model_us(cfg.wk, ks)) {
+                    cfg.wk = best_wk;
+                    ks = best;
+                }
             }
+            if (const char* e = getenv("FP6M_WK16")) cfg.wk = atoi(e) == 8 ? 8 : 4;   // tuning/testing override
+            const long long ks_k = ks_units(cfg.wk);
+            if (ks > ks_k) ks = ks_k;
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
             const size_t slot_bytes = (size_t)cfg.wn * 16 * kTileN * sizeof(float);
             while (ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > kScratchBytes) ks--;
             a.ks4 = (int)ks;
-            a.ks6 = (int)ks6_of(ks);
+            a.ks6 = (int)ks6_of(ks, cfg.wk);
             if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
             a.ksplit = a.ks4;
             if (row_mix) {

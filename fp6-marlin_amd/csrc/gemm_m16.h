@@ -360,7 +360,7 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
 
 template <bool G128, int AROWS, int WN, int WK, int D4, int D6>
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
-__global__ __launch_bounds__(64 * WN * WK, 3) void gemm_m16_kernel(const GemmArgs p)
+__global__ __launch_bounds__(64 * WN * WK, WK == 8 ? 2 : 3) void gemm_m16_kernel(const GemmArgs p)
 {
     constexpr int NW = WN * WK;
     constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);

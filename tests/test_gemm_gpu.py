@@ -175,6 +175,18 @@ def test_eight_k_slices_per_workgroup(oracle):
     run(oracle, 40, 512, 8192, qc=256, gs=128)
 
 
+def test_decode_kernel_with_eight_waves_per_workgroup(oracle):
+    """The m <= 16 kernel with eight k slices per workgroup (picked for grids of about one workgroup per CU, e.g.
+    8192 x 10240 at m = 1), forced on small and ragged problems, with and without a k split across workgroups."""
+    e = {"FP6M_WK16": 8}
+    for m in (1, 3, 4, 5, 16):
+        run(oracle, m, 512, 1024, qc=256, gs=128, env=e)
+        run(oracle, m, 768, 512, qc=128, env=e)
+        run(oracle, m, 256, 64, 64, 256, qc=-1, env=e)                  # one k unit: seven idle waves
+        run(oracle, m, 512, 2048, qc=256, ksplit=3, env=e)
+    run(oracle, 1, 10240, 8192, qc=256, gs=128)                         # the dispatcher's own choice of it
+
+
 def test_max_par_chunks_m(oracle):
     """m-tiles beyond max_par go to further launches (fp6_marlin_cuda_kernel.cu:917-948)."""
     run(oracle, 300, 512, 512, qc=256, max_par=2)
