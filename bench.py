@@ -194,7 +194,7 @@ def headline(args):
                    "m": m, "quant_cols": qc, "group_size": gs, "weight_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "fp6m::gemm_m16_kernel<true, 4, 1, 4, 4, 3>", "us_per_launch": round(per_launch * 1e6, 3),
+                     "kernel": "fp6m::gemm_m16_kernel<true, 4, 1, WK, 4, 3> (WK = 4 or 8 waves per workgroup, chosen per shape)", "us_per_launch": round(per_launch * 1e6, 3),
                      "bytes_per_launch": step_bytes // launches_per_step},
         "cpu_baseline": cpu_baseline(torch),
         "fp16_hipblaslt": {"ms_per_step": round(wall16 / args.steps * 1e3, 5),

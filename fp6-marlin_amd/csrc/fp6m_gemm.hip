@@ -440,14 +440,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     } else {
                         // eight waves per workgroup paid off only with one workgroup on (nearly) every CU: measured
                         // slower both when CUs hosted two of them and when a quarter or more of the CUs stayed idle
-                        if (load > 1.0 || load < 0.75) return 1e9;
+                        // (without a k split of the INT4 tiles there is no tail to lose, so fewer busy CUs still pay)
+                        if (load > 1.0 || load < (c == 1 ? 0.5 : 0.75)) return 1e9;
                         t = 0.56;
                     }
                     auto longest = [&](long long slices) { return (double)((units + slices - 1) / slices) * unit_steps; };
-                    double steps = a.groups4 ? longest(c * wk) : 0.0;
-                    if (a.groups6 && 1.5 * longest(c6 * wk) > steps) steps = 1.5 * longest(c6 * wk);
-                    const long long partners = c > c6 ? c : c6;
-                    return steps * t + (partners > 1 ? 2.5 + 0.15 * partners : 0.0);
+                    auto tail = [](long long partners) { return partners > 1 ? 2.5 + 0.15 * partners : 0.0; };
+                    const double int4_us = a.groups4 ? longest(c * wk) * t + tail(c) : 0.0;
+                    const double fp6_us = a.groups6 ? 1.5 * longest(c6 * wk) * t + tail(c6) : 0.0;   // an FP6 step moves 1.5x the bytes
+                    return int4_us > fp6_us ? int4_us : fp6_us;
                 };
                 int best_wk = cfg.wk;
                 long long best = ks;
