@@ -111,8 +111,8 @@ class Layer(nn.Module):
       ``s``          float16 1-D: INT4 scales (per column in the reference's permuted order, or
                      [infeatures/128, outfeatures-quant_cols] in natural column order when
                      ``groupsize=128``) followed by the FP6 per-column scales (permuted order)
-      ``meta``       int32 [6]: format version, infeatures, outfeatures, quant_cols, groupsize, word order
-                     (0 reference, 1 gfx950); a checkpoint whose ``meta`` differs from the layer's is refused
+      ``meta``       int32 [7]: format version, infeatures, outfeatures, quant_cols, groupsize, word order
+                     (0 reference, 1 gfx950), quant_rows; a checkpoint whose ``meta`` differs is refused
       ``workspace``  int32 zeros, outfeatures // 128 * 16 (not saved)
 
     Which output features are kept in FP6: by default the *last* ``quant_cols`` ones (what the reference's
@@ -120,12 +120,16 @@ class Layer(nn.Module):
     of ``quant_cols`` output features) ``pack`` moves those columns to the tail itself and ``forward`` writes
     every result column back to its own place inside the GEMM (``mul_fused``), so callers see W's own order.
     ``layout="gfx950"`` stores the packed words as per-tile sequential streams (``repack_gfx950``).
+
+    ``quant_rows`` instead keeps *input* features in FP6 (``mul_rows``: every column's last ``quant_rows`` rows FP6, the
+    rows before them INT4 with group-128 scales); ``fp6_in_channels`` names which ones, and ``forward`` gathers the
+    activations accordingly inside the call.
     """
 
     FORMAT_VERSION = 1
 
     def __init__(self, infeatures, outfeatures, groupsize=-1, quant_cols=-1, fp6_channels=None, bias=False,
-                 layout="reference"):
+                 layout="reference", quant_rows=0, fp6_in_channels=None):
         super().__init__()
         if groupsize not in (-1, 128):
             raise ValueError("Only groupsize -1 and 128 are supported.")
@@ -134,14 +138,37 @@ class Layer(nn.Module):
         qc = 0 if quant_cols in (-1, 0) else quant_cols
         if infeatures % 128 or outfeatures % 128 or qc % 128 or qc > outfeatures:
             raise ValueError("infeatures, outfeatures and quant_cols must be multiples of 128")
+        qr = int(quant_rows)
+        if qr:
+            if qc or groupsize != 128 or fp6_channels is not None:
+                raise ValueError("quant_rows (FP6 on input features) needs groupsize=128 and no quant_cols / fp6_channels")
+            if qr < 0 or qr >= infeatures or qr % 128:
+                raise ValueError("quant_rows must be a positive multiple of 128 below infeatures")
+        elif fp6_in_channels is not None:
+            raise ValueError("fp6_in_channels needs quant_rows")
         self.k, self.n, self.groupsize, self.quant_cols, self.layout = infeatures, outfeatures, groupsize, quant_cols, layout
+        self.quant_rows = qr
         n4 = outfeatures - qc
-        words = infeatures * n4 // 8 + infeatures * qc * 3 // 16
-        nscale = (n4 if groupsize == -1 else infeatures // 128 * n4) + qc
+        if qr:
+            words = (infeatures - qr) * outfeatures // 8 + qr * outfeatures * 3 // 16
+            nscale = (infeatures - qr) // 128 * outfeatures + outfeatures
+        else:
+            words = infeatures * n4 // 8 + infeatures * qc * 3 // 16
+            nscale = (n4 if groupsize == -1 else infeatures // 128 * n4) + qc
         self.register_buffer("B", torch.empty(words, dtype=torch.int32))
         self.register_buffer("s", torch.empty(nscale, dtype=torch.float16))
         self.register_buffer("meta", torch.tensor([self.FORMAT_VERSION, infeatures, outfeatures, qc, groupsize,
-                                                   int(layout == "gfx950")], dtype=torch.int32))
+                                                   int(layout == "gfx950"), qr], dtype=torch.int32))
+        if fp6_in_channels is not None:
+            picked = torch.as_tensor(fp6_in_channels, dtype=torch.int64).reshape(-1)
+            if picked.numel() != qr or picked.unique().numel() != qr or picked.min() < 0 or picked.max() >= infeatures:
+                raise ValueError("fp6_in_channels must name quant_rows distinct input features")
+            keep = torch.ones(infeatures, dtype=torch.bool)
+            keep[picked] = False
+            # packed row kk multiplies input feature a_cols[kk]: the others in order, then the chosen ones
+            self.register_buffer("a_cols", torch.cat([torch.nonzero(keep).reshape(-1), picked]).to(torch.int32))
+        else:
+            self.a_cols = None
         self.register_buffer("workspace", torch.zeros(outfeatures // 128 * 16, dtype=torch.int32), persistent=False)
         if fp6_channels is not None:
             picked = torch.as_tensor(fp6_channels, dtype=torch.int64).reshape(-1)
@@ -162,7 +189,7 @@ class Layer(nn.Module):
         meta = state_dict.get(prefix + "meta")
         if meta is not None and not torch.equal(meta.cpu().to(torch.int32), self.meta.cpu()):
             raise RuntimeError(f"{prefix}: checkpoint format {meta.tolist()} does not match this layer {self.meta.tolist()} "
-                               "(version, infeatures, outfeatures, quant_cols, groupsize, word order)")
+                               "(version, infeatures, outfeatures, quant_cols, groupsize, word order, quant_rows)")
         super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def pack(self, linear):
@@ -176,9 +203,18 @@ class Layer(nn.Module):
             raise ValueError("weight shape does not match the layer")
         if self.c_cols is not None:
             w = w[:, self.c_cols.long().to(w.device)].contiguous()
-        B, s, w_ref = pack_mixed_weight(w, self.quant_cols, self.groupsize, harness_layout=False)
+        if self.quant_rows:
+            if self.a_cols is not None:
+                w = w[self.a_cols.long().to(w.device)].contiguous()
+            B, s, w_ref = pack_row_mix_weight(w, self.quant_rows)
+            if self.a_cols is not None:                            # the check weight in W's own row order
+                own = torch.empty_like(w_ref)
+                own[self.a_cols.long().to(w_ref.device)] = w_ref
+                w_ref = own
+        else:
+            B, s, w_ref = pack_mixed_weight(w, self.quant_cols, self.groupsize, harness_layout=False)
         if self.layout == "gfx950":
-            B = cabi.repack_gfx950(B, self.k, self.n, self.quant_cols)
+            B = cabi.repack_gfx950(B, self.k, self.n, self.quant_cols, self.quant_rows)
         self.B.copy_(B)
         self.s.copy_(s)
         if self.bias is not None and isinstance(linear, nn.Module) and getattr(linear, "bias", None) is not None:
@@ -193,10 +229,13 @@ class Layer(nn.Module):
         """y = x @ W (+ bias) (+ residual, float16 of y's shape), as one GEMM call."""
         x2 = x.reshape(-1, x.shape[-1]).to(torch.float16).contiguous()
         out = torch.empty((x2.shape[0], self.n), dtype=torch.float16, device=x2.device)
-        if self.c_cols is None and self.bias is None and residual is None and self.layout == "reference":
+        res = None if residual is None else residual.reshape(-1, self.n).to(torch.float16).contiguous()
+        if self.quant_rows:
+            cabi.mul_rows(x2, self.B, out, self.s, self.workspace, self.quant_rows, a_cols=self.a_cols, bias=self.bias,
+                          residual=res, layout=self.layout)
+        elif self.c_cols is None and self.bias is None and residual is None and self.layout == "reference":
             cabi.mul(x2, self.B, out, self.s, self.workspace, self.quant_cols, -1, -1, -1, 16, self.groupsize)
         else:
-            res = None if residual is None else residual.reshape(-1, self.n).to(torch.float16).contiguous()
             cabi.mul_fused(x2, self.B, out, self.s, self.workspace, self.quant_cols, self.groupsize, c_cols=self.c_cols,
                            bias=self.bias, residual=res, layout=self.layout)
         return out.reshape(x.shape[:-1] + (self.n,))

@@ -170,3 +170,33 @@ def test_row_mix_packer_and_errors(oracle):
         fp6_marlin.mul_rows(A.to(dev()), Bd, C, sd, ws, 192)                      # 768 - 192 is no multiple of 128
     with pytest.raises(ValueError):
         fp6_marlin.pack_row_mix_weight(w, 100)
+
+
+def test_layer_with_fp6_input_features(oracle):
+    """`Layer(quant_rows=..., fp6_in_channels=...)`: chosen input features in FP6, gathered inside the call; the check
+    weight comes back in the linear layer's own order; both word orders agree bit for bit; checkpoints carry the mix."""
+    import fp6_marlin
+    torch.manual_seed(4)
+    k, n, qr = 768, 512, 256
+    lin = torch.nn.Linear(k, n, bias=True).half()
+    picked = torch.randperm(k)[:qr]
+    x = torch.randn((5, k), dtype=torch.half)
+    outs = []
+    for layout in ("reference", "gfx950"):
+        layer = fp6_marlin.Layer(k, n, groupsize=128, quant_rows=qr, fp6_in_channels=picked, bias=True, layout=layout)
+        w_ref = layer.pack(lin)
+        err = (w_ref.float() - lin.weight.data.t().float()).abs().mean(1) / lin.weight.data.t().float().abs().mean(1)
+        assert err.max() < 0.3                                         # row order restored (a wrong order gives ~1.4)
+        layer = layer.to(dev())
+        y = layer(x.to(dev())).cpu()
+        y_ref = x.float() @ w_ref.float() + lin.bias.data.float()
+        assert oracle.rel_err(y.numpy(), y_ref.numpy()) <= TOL
+        outs.append(y)
+        clone = fp6_marlin.Layer(k, n, groupsize=128, quant_rows=qr, fp6_in_channels=picked, bias=True, layout=layout)
+        clone.load_state_dict(layer.state_dict())
+        assert torch.equal(clone.to(dev())(x.to(dev())).cpu(), y)
+        with pytest.raises(RuntimeError, match="does not match"):
+            fp6_marlin.Layer(k, n, groupsize=128, quant_cols=256, bias=True, layout=layout).load_state_dict(layer.state_dict(), strict=False)
+    assert torch.equal(outs[0], outs[1])
+    with pytest.raises(ValueError):
+        fp6_marlin.Layer(k, n, groupsize=-1, quant_rows=qr)
