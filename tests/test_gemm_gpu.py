@@ -321,3 +321,33 @@ def test_layer_with_chosen_fp6_channels_bias_residual_and_checkpoint(oracle):
         with pytest.raises(RuntimeError, match="does not match"):
             other.load_state_dict(layer.state_dict())
     assert torch.equal(outs[0], outs[1])
+
+
+def test_dispatcher_choices_over_many_shapes(oracle):
+    """The dispatcher picks waves per workgroup and the k split per shape (rule + cost model): a sweep over decode
+    shapes with random packed words against the pinned unpacker, so that every combination it can choose is exercised
+    with real sizes (eight-wave workgroups without a k split, exact one- and two-per-CU grids, long k)."""
+    import fp6_marlin
+    g = torch.Generator().manual_seed(5)
+    gs = 128
+    for k, n, qc in [(1024, 2048, 256), (4096, 10240, 256), (4096, 17920, 256), (4096, 28672, 0), (4096, 32768, 256),
+                     (5120, 5120, 256), (6656, 6656, 128), (6656, 17920, 256), (11008, 2048, 256), (13824, 5120, 512),
+                     (8192, 28672, 256), (2048, 57344, 256)]:
+        n4 = n - qc
+        B = torch.randint(-2 ** 31, 2 ** 31 - 1, (k * n4 // 8 + k * qc * 3 // 16,), generator=g, dtype=torch.int64).to(torch.int32)
+        s = (torch.rand((k // gs) * n4 + qc, generator=g) * 0.01 + 0.001).half()
+        w = fp6_marlin.unpack_to_fp16(B, s, k, n, qc if qc else -1, gs).to(dev())
+        Bd, sd = B.to(dev()), s.to(dev())
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+        for m in (1, 4, 16):
+            print(f"case dispatch m={m} k={k} n={n} qc={qc}", flush=True)
+            a = torch.randn((m, k), generator=g).half().to(dev())
+            C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+            fp6_marlin.mul(a, Bd, C, sd, ws, qc if qc else -1, -1, -1, -1, 16, gs)
+            torch.cuda.synchronize()
+            ref = a.float() @ w.float()
+            err = ((C.float() - ref).abs().mean() / ref.abs().mean()).item()
+            assert err <= TOL, (m, k, n, qc, err)
+            assert int(ws.abs().sum().item()) == 0
+        del w, Bd, sd
+        torch.cuda.empty_cache()
