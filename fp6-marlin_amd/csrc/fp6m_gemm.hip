@@ -9,12 +9,14 @@
 //    fragment owner's k-pair index becomes the high lane bits, dequantises in registers and feeds
 //    v_mfma_f32_16x16x32_f16 with the *weights as the 16-row operand* (C^T = W^T A^T), so a single
 //    MFMA covers 16 columns x 32 k for up to 16 rows of A.  No workgroup barrier in the main loop.
-//  * A workgroup is four such waves splitting k; they are summed through LDS.  `ksplit` workgroups may
+//  * A workgroup is four (or eight) such waves splitting k; they are summed through LDS.  `ksplit` workgroups may
 //    share a tile; each writes its fp32 partial tile to a per-device scratch, and the workgroup that
 //    arrives last (one atomic counter per tile in `workspace`) sums the partials in a fixed order,
 //    applies the scales and writes fp16 C.  Nobody spins, so there is nothing to deadlock on, and the
 //    counters are zero again when the launch drains.
 //  * INT4 and FP6 tiles are entries of one tile list handled by the same launch.
+//  * The dispatcher picks the kernel by m, and for m <= 16 the waves per workgroup and the k split per shape
+//    (a rule plus a small cost model fitted to per-workgroup timelines on MI355X).
 //
 // gemm_common.h  argument block, tile bookkeeping, load / wait / dequantisation helpers
 // gemm_m16.h     gemm_m16_kernel (m <= 16)
