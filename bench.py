@@ -2,7 +2,7 @@
 """Benchmark of the mixed INT4/FP6 weight-only GEMM on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]          one JSON line (the driver's contract)
-    python bench.py --sweep gpurun_out/sweep.json                per-shape table for all BASELINE configs
+    python bench.py --sweep sweep.json                           per-shape table for all BASELINE configs
     python bench.py --shape 128,8192,8192                        one shape (m,k,n[,quant_cols,group_size])
 
 Workload of the JSON line: decode (M=1) through Llama-2-7B layer shapes (K x N) 4096x12288, 4096x4096,
