@@ -7,13 +7,31 @@ namespace fp6m {
 // ------------------------------------------------------------------------------------------------ m <= 16: LDS-ring kernel
 //
 // Every wave keeps a private ring of DEPTH slots in LDS.  A slot is one k step (32 rows of k) of its
-// tile: the packed words (2 x 1 KiB 4-bit/INT4, + 2 x 512 B FP6 2-bit) and the 16 x 32 fp16 activation
-// block (1 KiB).  Slots are filled by direct-to-LDS global loads (no VGPR staging): lane L's data lands
-// at slot + 16 L, so the *global* granule each lane fetches is permuted (inside aligned 64-byte quads,
-// which keeps the loads coalesced) to obtain a layout that the permuted reads hit without bank
-// conflicts.  The loads of step s + DEPTH - 1 are issued before step s is consumed; `s_waitcnt vmcnt`
-// with a constant count is the only synchronisation in the loop.  LDS reads are inline asm so that
-// the compiler does not serialise them behind every outstanding direct-to-LDS load.
+// tile's packed words (2 x 1 KiB 4-bit/INT4, + 2 x 512 B FP6 2-bit).  Slots are filled by direct-to-LDS
+// global loads (no VGPR staging): lane L's data lands at slot + 16 L, so the *global* granule each lane
+// fetches is permuted (inside aligned 64-byte quads, which keeps the loads coalesced) to obtain a layout
+// that the permuted reads hit without bank conflicts.  The loads of step s + DEPTH - 1 are issued before
+// step s is consumed; `s_waitcnt vmcnt` with a constant count is the only synchronisation in the loop.
+// LDS reads are inline asm so that the compiler does not serialise them behind every outstanding
+// direct-to-LDS load.
+// The activations are fetched two steps at a time (a whole 128-byte line of every row per load) into a
+// ring of their own behind the word slots: what limits a workgroup's rate is its requests in flight, and
+// 64 bytes per row and step doubled the requests the activations cost (at m = 16 two fifths of all
+// requests; one fetch per pair of steps took 6-10 % off those launches).
+
+// Ring slots of A (one slot = a pair of steps): the pair being read, the pairs of the depth - 1 steps fetched
+// ahead, and the one the next fetch fills.  A slot holds 128 bytes of each of its rows.
+constexpr int pair_slots(int depth) { return (depth + 2) / 2; }
+constexpr int pair_bytes(int arows) { return arows * 128; }
+constexpr int a_ring_bytes(int depth, int arows) { return pair_slots(depth) * pair_bytes(arows); }
+// Loads of n consecutive steps, the first with parity `first` within its pair: the words of each, and
+// `a_ops` loads of A in front of every pair.
+constexpr int newer_step_ops(int word_ops, int a_ops, int first, int n)
+{
+    int ops = word_ops * n;
+    for (int t = 0; t < n; t++) ops += ((first + t) & 1) == 0 ? a_ops : 0;
+    return ops;
+}
 
 struct StepRegs {
     u4 q0, q1;          // 4-bit plane / INT4 words of the two k-blocks
@@ -21,16 +39,18 @@ struct StepRegs {
     uint32_t a[4];      // activations in MFMA operand order
 };
 
-// AROWS = rows of A a slot holds (4 or 16): 64 bytes per row and step.
+// AROWS = rows of A the ring holds (4 or 16).
 template <bool FP6, bool G128, int DEPTH, int AROWS>
 __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                             int step_begin, int step_end, f4 (&acc)[1][8])
 {
     static_assert(DEPTH >= 3, "needs two steps of look-ahead");
     constexpr bool kGroup = G128 && !FP6;                 // group scales apply to INT4 tiles only
-    constexpr int kAOff = FP6 ? 3072 : 2048;
-    constexpr int kSlot = kAOff + AROWS * 64;
-    constexpr int kOps = FP6 ? 4 : 3;                     // direct-to-LDS loads per step
+    constexpr int kPairSlots = pair_slots(DEPTH);         // step pairs of A alive at once
+    constexpr int kPair = pair_bytes(AROWS);
+    constexpr int kSlot = FP6 ? 3072 : 2048;              // a step's packed words
+    constexpr int kWordOps = FP6 ? 3 : 2;                 // direct-to-LDS loads of the packed words per step
+    constexpr int kAOps = AROWS == 16 ? 2 : 1;            // ... and of A per pair of steps
     constexpr int kReads = FP6 ? 8 : 6;                   // LDS reads per step
     constexpr int kUnroll = kGroup ? 4 : 2;               // steps per loop trip (step counts are multiples of it)
     const int lane = threadIdx.x & 63;
@@ -54,33 +74,60 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
     const unsigned char* base2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2) + geo.tile2 +
                                  (size_t)(2 * step_begin) * row2;
-    const int a_m = lane >> 2;
-    const bool a_active = a_m < AROWS && ti.mtile * 16 + a_m < p.m;
-    const uint32_t va = (uint32_t)(a_active ? a_m : 0) * (uint32_t)p.k * 2 + 16 * ((lane & 3) ^ ((a_m >> 2) & 3));
+    // A: load o brings rows 8o .. 8o+7 (AROWS = 4: the lower half of the wave brings rows 0 .. 3), eight lanes
+    // per row.  LDS position lane = 8 * row + chunk' holds the row's 16-byte chunk 4h + d (step parity h,
+    // quarter d) at chunk' = 4h + (d ^ (row >> 1 & 3)).  Rows past m re-read row m-1, so the lanes that take
+    // part never depend on m and neither does the count of loads in flight.
+    const bool a_lane = AROWS == 16 || lane < 32;
+    uint32_t vap[kAOps];
+#pragma unroll
+    for (int o = 0; o < kAOps; o++) {
+        const int prow = (lane >> 3) & (AROWS - 1) & 7, pch = lane & 7;
+        int row = ti.mtile * 16 + 8 * o + prow;
+        row = row < p.m ? row : p.m - 1;
+        vap[o] = (uint32_t)(row - ti.mtile * 16) * (uint32_t)p.k * 2 + 16 * ((pch & 4) | ((pch & 3) ^ ((prow >> 1) & 3)));
+    }
     const unsigned char* base_a = reinterpret_cast<const unsigned char*>(p.A + (size_t)ti.mtile * 16 * p.k) +
                                   (size_t)(ti.a_step0 + step_begin) * 64;
+    unsigned char* a_ring = ring + DEPTH * kSlot;
+    const int last_pair = (step_end - step_begin) / 2 - 1;
+    int pairs_issued = 0, pair_in = 0;
     const unsigned char* base_gs = reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN);
     const uint32_t vgs = 4 * lane;
     constexpr int kScaleMask = DEPTH <= 5 ? 1 : 3;        // 256-byte slabs of group scales: 2 suffice up to depth 5
-    unsigned char* gs_ring = ring + DEPTH * kSlot;
+    unsigned char* gs_ring = a_ring + kPairSlots * kPair;
 
     int issued = step_begin;                              // next step to fetch (clamped at the last one)
     const int last = step_end - 1;
-    auto issue = [&](int slot) {
+    // `even`: the step fetched is the first of its pair (counted from step_begin; a compile-time fact at every call)
+    auto issue = [&](int slot, bool even) {
         unsigned char* dst = ring + slot * kSlot;
+        if (even) {
+            unsigned char* adst = a_ring + pair_in * kPair;
+            if (a_lane) dma16(base_a + vap[0], adst);
+            if (kAOps == 2) dma16(base_a + vap[kAOps - 1], adst + 1024);
+            pair_in = pair_in + 1 == kPairSlots ? 0 : pair_in + 1;
+            if (pairs_issued < last_pair) {               // (fetches past the end repeat the last pair)
+                pairs_issued++;
+                base_a += 128;
+            }
+        }
         dma16_stream(base4 + v4, dst);
         dma16_stream(base4 + row4 + v4, dst + 1024);
         if (FP6) dma16_stream(base2 + v2, dst + 2048);
-        if (a_active) dma16(base_a + va, dst + kAOff);
         if (kGroup && (issued & 3) == 0)
             dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & kScaleMask) * 256);
         if (issued < last) {                              // uniform: pointers move on the scalar unit
             issued++;
             base4 += 2 * row4;
             base2 += 2 * row2;
-            base_a += 64;
         }
     };
+    // Loads that may stay in flight while the oldest fetched step must have landed: those of the DEPTH - 2 newer
+    // steps, the first of which is the second of its pair (kWaitOdd) or the first (kWaitEven).  The occasional
+    // load of group scales only makes the wait stricter.
+    constexpr int kWaitOdd = newer_step_ops(kWordOps, kAOps, 1, DEPTH - 2);
+    constexpr int kWaitEven = newer_step_ops(kWordOps, kAOps, 0, DEPTH - 2);
 
     // ---- read side (lane = MFMA identity)
     const int owner = p.native ? lane : 32 * sigma + 4 * l + i;   // whose granule of the k-block this lane needs
@@ -91,12 +138,13 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     const int ar = c & (AROWS - 1);                       // rows beyond AROWS re-read a valid row; their sums are never stored
     uint32_t rda[4];
 #pragma unroll
-    for (int d = 0; d < 4; d++) rda[d] = ring_lds + kAOff + (4 * ar + (d ^ ((ar >> 2) & 3))) * 16 + 4 * i;
+    for (int d = 0; d < 4; d++)
+        rda[d] = lds_addr(a_ring) + (ar >> 3) * 1024 + (8 * (ar & 7) + (d ^ ((ar >> 1) & 3))) * 16 + 4 * i;
     const int q = i;                                      // result side: quarter of the column slots
     const uint32_t rdgs = lds_addr(gs_ring) + (64 * (q >> 1) + 4 * (q & 1)) * 2;
 
     // kReads LDS reads of one step, not waited for.
-    auto fetch = [&](StepRegs& r, int slot) {
+    auto fetch = [&](StepRegs& r, int slot, int pair_slot, bool odd) {
         const uint32_t so = slot * kSlot;
         if (FP6) {
             asm volatile(
@@ -107,9 +155,16 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
             asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
                          : "=&v"(r.q0), "=&v"(r.q1) : "v"(rd4 + so) : "memory");
         }
-        asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7"
-                     : "=&v"(r.a[0]), "=&v"(r.a[1]), "=&v"(r.a[2]), "=&v"(r.a[3])
-                     : "v"(rda[0] + so), "v"(rda[1] + so), "v"(rda[2] + so), "v"(rda[3] + so) : "memory");
+        const uint32_t ao = pair_slot * kPair;
+        if (odd)                                // the second step of a pair: the other half of every row's line
+            asm volatile("ds_read_b32 %0, %4 offset:64\n\tds_read_b32 %1, %5 offset:64\n\t"
+                         "ds_read_b32 %2, %6 offset:64\n\tds_read_b32 %3, %7 offset:64"
+                         : "=&v"(r.a[0]), "=&v"(r.a[1]), "=&v"(r.a[2]), "=&v"(r.a[3])
+                         : "v"(rda[0] + ao), "v"(rda[1] + ao), "v"(rda[2] + ao), "v"(rda[3] + ao) : "memory");
+        else
+            asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7"
+                         : "=&v"(r.a[0]), "=&v"(r.a[1]), "=&v"(r.a[2]), "=&v"(r.a[3])
+                         : "v"(rda[0] + ao), "v"(rda[1] + ao), "v"(rda[2] + ao), "v"(rda[3] + ao) : "memory");
     };
     // After the counter wait, the registers of `r` hold their data: make every later use depend on it.
     auto settle = [&](StepRegs& r) {
@@ -139,25 +194,30 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     // Pipeline: while step s is being computed, the LDS reads of step s+1 are in flight and the
     // direct-to-LDS loads of steps s+2 .. s+DEPTH-1 are outstanding.
     int slot_in = 0;
-#pragma unroll 1
+#pragma unroll
     for (int d = 0; d < DEPTH - 1; d++) {
-        issue(slot_in);
+        issue(slot_in, (d & 1) == 0);
         slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
     }
     StepRegs regs[2];
-    __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));         // step 0 has landed; step 1 is the oldest newer one
     FP6M_MARK(p, 1);
-    fetch(regs[0], 0);
+    fetch(regs[0], 0, 0, false);
     int slot_rd = 1;                                      // slot of the step whose LDS reads come next
+    int pair_rd = 0;                                      // A ring slot of the pair that step belongs to
     f4 grp[8];
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            issue(slot_in);
+            issue(slot_in, ((u + DEPTH - 1) & 1) == 0);
             slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));   // step s+u+1 has landed
-            fetch(regs[(u + 1) & 1], slot_rd);
+            if (u & 1)                                                    // step s+u+1 has landed
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));
+            else
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven));
+            if (u & 1) pair_rd = pair_rd + 1 == kPairSlots ? 0 : pair_rd + 1;   // step s+u+1 opens a pair
+            fetch(regs[(u + 1) & 1], slot_rd, pair_rd, (u & 1) == 0);
             slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
             __builtin_amdgcn_s_waitcnt(lgkmcnt_only(kReads));             // reads of step s+u (older) are done
             settle(regs[u & 1]);
@@ -203,7 +263,8 @@ constexpr int scale_slab_bytes(int depth) { return depth <= 5 ? 512 : 1024; }
 constexpr int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
 constexpr int wave_lds_bytes(int d4, int d6, int arows)
 {
-    return max3(d4 * (2048 + arows * 64) + scale_slab_bytes(d4), d6 * (3072 + arows * 64), 16 * kRedStride * 4);
+    return max3(d4 * 2048 + a_ring_bytes(d4, arows) + scale_slab_bytes(d4), d6 * 3072 + a_ring_bytes(d6, arows),
+                16 * kRedStride * 4);
 }
 
 // The m <= 16 kernel.
@@ -360,7 +421,7 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
 
 template <bool G128, int AROWS, int WN, int WK, int D4, int D6>
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
-__global__ __launch_bounds__(64 * WN * WK, WK == 8 ? 2 : 3) void gemm_m16_kernel(const GemmArgs p)
+__global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void gemm_m16_kernel(const GemmArgs p)
 {
     constexpr int NW = WN * WK;
     constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);
