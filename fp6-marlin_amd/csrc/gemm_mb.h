@@ -70,6 +70,12 @@ __device__ __forceinline__ void dequant_half(uint32_t q2, uint32_t q4, int half,
     }
 }
 
+// A pair slot (two k steps of A): per 16-row block two loads of 8 rows x 128 bytes; the second lands 64 bytes
+// further than it would back to back, so that rows 8 .. 15 use the other half of the banks and a read of one
+// step's half-lines by all 16 rows is conflict-free.
+constexpr int kPairHalf = 1024 + 64;                      // from a block's first load to its second
+constexpr int kPairBlock = 2 * kPairHalf;                 // from block to block
+
 struct MbCtx {
     uint32_t abuf[4][4];
     uint32_t addr_cur[4], addr_next[4];
@@ -81,18 +87,33 @@ struct MbCtx {
 // immediates follow from the fixed issue order: [A(0), A(1)] from the previous step, the next step's
 // weight words (kExtra reads), then A(2), A(3), ...  After every MFMA `hook(block, t)` runs: the caller
 // uses it to dequantise the next step's fragments a few VALU instructions at a time.
+// PAIRH < 0: a slot holds one step, blocks 1 KiB apart; addr_cur / addr_next are this step's and the next
+// step's slot.  PAIRH = 0 / 1: a slot holds a pair of steps (blocks 2 KiB apart, the second step's half of
+// every row 64 bytes on) and this is the pair's first / second step; addr_cur / addr_next are this pair's and
+// the next pair's slot.
 template <int MB, int kExtra, int BLK = 0>
 struct MbBlocks {
-    template <int phase, typename Hook>
+    // VMW >= 0 (second step of a pair): the next pair may still be in flight when the step starts; before its first
+    // read, wait until at most VMW vector-memory loads (the ones issued after it) are outstanding.
+    template <int phase, int PAIRH = -1, int VMW = -1, typename Hook>
     static __device__ __forceinline__ void run(MbCtx& cx, const h8 (&frag)[8], f4 (&acc)[MB][8], Hook&& hook)
     {
         if constexpr (BLK < MB) {
             constexpr int nb = BLK + 2;
             uint32_t (&dst)[4] = cx.abuf[(phase + nb) & 3];
-            if constexpr (nb < MB)
-                lds_read_a4<nb * 1024>(dst, cx.addr_cur);
-            else
-                lds_read_a4<(nb - MB) * 1024>(dst, cx.addr_next);
+            if constexpr (PAIRH < 0) {
+                if constexpr (nb < MB)
+                    lds_read_a4<nb * 1024>(dst, cx.addr_cur);
+                else
+                    lds_read_a4<(nb - MB) * 1024>(dst, cx.addr_next);
+            } else if constexpr (nb < MB) {
+                lds_read_a4<nb * kPairBlock + PAIRH * 64>(dst, cx.addr_cur);
+            } else if constexpr (PAIRH == 0) {
+                lds_read_a4<(nb - MB) * kPairBlock + 64>(dst, cx.addr_cur);
+            } else {
+                if constexpr (nb == MB && VMW >= 0) __builtin_amdgcn_s_waitcnt(vmcnt_only(VMW));
+                lds_read_a4<(nb - MB) * kPairBlock>(dst, cx.addr_next);
+            }
             // block 0 needs A(0): A(1), the extra reads and A(2) may be outstanding; from block 1 on the
             // extra reads must be complete as well
             constexpr int allow = BLK == 0 ? (8 + kExtra < 15 ? 8 + kExtra : 15) : 8;
@@ -108,7 +129,7 @@ struct MbBlocks {
             mfma_acc<false>(acc[BLK][5], frag[5], av); hook(Int<BLK>{}, Int<5>{});
             mfma_acc<false>(acc[BLK][6], frag[6], av); hook(Int<BLK>{}, Int<6>{});
             mfma_acc<false>(acc[BLK][7], frag[7], av); hook(Int<BLK>{}, Int<7>{});
-            MbBlocks<MB, kExtra, BLK + 1>::template run<phase>(cx, frag, acc, hook);
+            MbBlocks<MB, kExtra, BLK + 1>::template run<phase, PAIRH, VMW>(cx, frag, acc, hook);
         }
     }
 };
@@ -316,11 +337,18 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
                     for (int ck = c0; ck < c1; ck++) chunk(ck, (u + 1) & 1, nxt);
                 }
             };
-            constexpr int kExtraMax = kW + (kGroup ? 8 : 0);
-            if ((u & 1) == 0)                                          // buffer of block 0: (u * MB) mod 4
-                MbBlocks<MB, kExtraMax>::template run<0>(cx, cur, acc, hook);
-            else
-                MbBlocks<MB, kExtraMax>::template run<(MB & 3)>(cx, cur, acc, hook);
+            // (the LDS reads issued between A(1) and A(2): the words, and the group scales where a group starts)
+            if ((u & 1) == 0) {                                        // buffer of block 0: (u * MB) mod 4
+                if (next_group)
+                    MbBlocks<MB, kW + 8>::template run<0>(cx, cur, acc, hook);
+                else
+                    MbBlocks<MB, kW>::template run<0>(cx, cur, acc, hook);
+            } else {
+                if (next_group)
+                    MbBlocks<MB, kW + 8>::template run<(MB & 3)>(cx, cur, acc, hook);
+                else
+                    MbBlocks<MB, kW>::template run<(MB & 3)>(cx, cur, acc, hook);
+            }
         }
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
@@ -333,6 +361,257 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
         for (int t = 0; t < 8; t++) {
             asm volatile("" : "+v"(acc[mb][t]));
         }
+    if (FP6) {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int t = 0; t < 8; t++) acc[mb][t] *= 4096.0f;
+    }
+}
+
+// The MB = 4 variant of stream_tile_mb: activations fetched a pair of k steps at a time, packed words through
+// registers.
+//
+// What bounds a workgroup's rate is its requests in flight, and A dominated them: 64 half-lines per step and
+// wave against 16 lines of words (fetching only half of the distinct lines measured 10-15 % faster at
+// m = 64 .. 256).  Here one load brings 8 rows x 128 bytes -- whole lines, two steps of k -- into a ring of two
+// pair slots (MB x 2 KiB each).  That is 4 KiB more LDS per wave than three one-step slots, which eight waves
+// per CU only have if the words stay out of LDS: each lane loads its own two 16-byte granules of a step (the
+// k-block row is contiguous, so the wave still reads whole lines) into one of two register sets, two steps
+// ahead of the MFMAs and one ahead of the dequantisation, exactly the look-ahead the three-slot ring gave.
+// A pair's first step issues the words two steps on, then the next pair of A; its second step only words.  Either
+// step starts once the words of the following step have landed, which leaves that next pair and the newest words in
+// flight; the second step waits for the pair in its middle, right before it reads the next step's first A block.
+// A load of group scales goes out in front of the words of some first steps and is counted there.
+constexpr int pair_load_imm(int q) { return ((q / 2) % 2) * kPairBlock + (q % 2) * kPairHalf; }
+static_assert(pair_load_imm(3) < 4096, "immediate of a direct-to-LDS load");
+template <int MB, int I = 0>
+__device__ __forceinline__ void dma_a_pair(uint32_t slot_lds, const void* sbase_a, const uint32_t (&voff)[2 * MB])
+{
+    if constexpr (I < 2 * MB) {
+        // four loads (two blocks) per value of M0: the immediate reaches 4 KiB
+        if constexpr (I % 4 == 0) set_m0(slot_lds + (I / 2) * kPairBlock);
+        dma16_m0<pair_load_imm(I), false>(sbase_a, voff[I]);
+        dma_a_pair<MB, I + 1>(slot_lds, sbase_a, voff);
+    }
+}
+constexpr int mbp_wave_lds(int mb) { return max3(2 * mb * kPairBlock + 512, 2 * 16 * kRedStride * 4, 0); }
+
+template <bool FP6, bool G128, int MB>
+__device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
+                                                int step_begin, int step_end, f4 (&acc)[MB][8])
+{
+    static_assert(MB == 4, "the A register ring runs with phase 0 in every step");
+    constexpr bool kGroup = G128 && !FP6;
+    constexpr int kPair = MB * kPairBlock;                // one pair slot
+    constexpr int kWOps = FP6 ? 4 : 2;                    // register loads per step
+    constexpr int kAOps = 2 * MB;                         // direct-to-LDS loads per pair
+    constexpr int kUnroll = kGroup ? 4 : 2;
+    static_assert(kAOps + kWOps + 1 <= 63, "vmcnt is a 6-bit counter");
+    const int lane = threadIdx.x & 63;
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+
+    DequantConsts kc;
+    kc.lo = vgpr_const(0x000f000fu);
+    kc.hi = vgpr_const(0x00f000f0u);
+    kc.ex = vgpr_const(0x64006400u);
+    kc.top2 = vgpr_const(0xc0c0c0c0u);
+    kc.exp_man = vgpr_const(0x9f009f00u);
+
+    // ---- fetch side
+    const PlaneGeometry geo = plane_geometry(p, ti);
+    const size_t row4 = geo.row4, row2 = geo.row2;
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;      // whose granule of the k-block this lane needs
+    const uint32_t v4 = (uint32_t)owner * 16, v4b = v4 + (uint32_t)row4;
+    const unsigned char* base4 = uniform_ptr(reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4) +
+                                             geo.tile4 + (size_t)(2 * step_begin) * row4);
+    const uint32_t v2 = (uint32_t)owner * 8, v2b = v2 + (uint32_t)row2;
+    const unsigned char* base2 = uniform_ptr(reinterpret_cast<const unsigned char*>(p.b_fp6_2) +
+                                             geo.tile2 + (size_t)(2 * step_begin) * row2);
+    u4 wq[2][2];                                          // [register set][k-block]
+    u2 tq[2][2];
+    // A: load 2b + o brings rows 8o .. 8o+7 of block b, eight lanes per row; LDS position lane = 8 * row + chunk'
+    // holds the row's 16-byte chunk 4h + d (step parity h, quarter d) at chunk' = 4h + (d ^ (row >> 1 & 3)).
+    const int tile_row0 = ti.mtile * 16 * MB;
+    const int prow = lane >> 3, pch = lane & 7;
+    uint32_t va[2 * MB];
+#pragma unroll
+    for (int q = 0; q < 2 * MB; q++) {
+        int row = tile_row0 + 8 * q + prow;
+        row = row < p.m ? row : p.m - 1;
+        va[q] = (uint32_t)(row - tile_row0) * (uint32_t)p.k * 2 + 16 * ((pch & 4) | ((pch & 3) ^ ((prow >> 1) & 3))) +
+                4096 - pair_load_imm(q);
+    }
+    const unsigned char* base_a = uniform_ptr(reinterpret_cast<const unsigned char*>(p.A + (size_t)tile_row0 * p.k) +
+                                              (size_t)(ti.a_step0 + step_begin) * 64 - 4096);
+    const unsigned char* base_gs =
+        uniform_ptr(reinterpret_cast<const unsigned char*>(p.s_int4 + (size_t)ti.tcol * kTileN));
+    const uint32_t vgs = 4 * lane;
+    const uint32_t ring_lds = uniform32(lds_addr(ring));
+    const uint32_t gs_lds = ring_lds + 2 * kPair;
+
+    int issued = step_begin;
+    const int last = step_end - 1;
+    int pairs_issued = 0, a_slot = 0;
+    const int last_pair = (step_end - step_begin) / 2 - 1;
+    auto issue_a = [&]() {
+        dma_a_pair<MB>(ring_lds + a_slot * kPair, base_a, va);
+        a_slot ^= 1;
+        if (pairs_issued < last_pair) {                   // (fetches past the end repeat the last pair)
+            pairs_issued++;
+            base_a += 128;
+        }
+    };
+    // returns whether a load of group scales went out in front of the words
+    auto issue_w = [&](int set) {
+        const bool scales = kGroup && (issued & 3) == 0;
+        if (scales) {
+            set_m0(gs_lds + ((issued >> 2) & 1) * 256);
+            dma4_m0(base_gs + (size_t)(issued >> 2) * (size_t)uniform32(p.n4) * 2, vgs);
+        }
+        asm volatile("global_load_dwordx4 %0, %2, %4 nt\n\tglobal_load_dwordx4 %1, %3, %4 nt"
+                     : "=&v"(wq[set][0]), "=&v"(wq[set][1]) : "v"(v4), "v"(v4b), "s"(base4) : "memory");
+        if (FP6) {
+            asm volatile("global_load_dwordx2 %0, %2, %4 nt\n\tglobal_load_dwordx2 %1, %3, %4 nt"
+                         : "=&v"(tq[set][0]), "=&v"(tq[set][1]) : "v"(v2), "v"(v2b), "s"(base2) : "memory");
+        }
+        if (issued < last) {
+            issued++;
+            base4 += 2 * row4;
+            base2 += 2 * row2;
+        }
+        return scales;
+    };
+
+    // ---- read side
+    const uint32_t rdgs = gs_lds + (64 * sigma + l) * 2;    // weight side: column (j, half) at +32j +16half
+    uint32_t gs_next[8];
+    h2 gs_cur[8];
+    MbCtx cx;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        cx.addr_cur[d] = ring_lds + (c >> 3) * kPairHalf + (8 * (c & 7) + (d ^ ((c >> 1) & 3))) * 16 + 4 * i;
+        cx.addr_next[d] = 0;
+    }
+    uint32_t to_next = kPair;                             // from this pair's slot to the other one (uniform)
+    auto fetch_scales = [&](int group) {
+        const uint32_t ga = rdgs + (group & 1) * 256;
+        asm volatile(
+            "ds_read_u16 %0, %8\n\tds_read_u16 %1, %8 offset:16\n\tds_read_u16 %2, %8 offset:32\n\t"
+            "ds_read_u16 %3, %8 offset:48\n\tds_read_u16 %4, %8 offset:64\n\tds_read_u16 %5, %8 offset:80\n\t"
+            "ds_read_u16 %6, %8 offset:96\n\tds_read_u16 %7, %8 offset:112"
+            : "=&v"(gs_next[0]), "=&v"(gs_next[1]), "=&v"(gs_next[2]), "=&v"(gs_next[3]), "=&v"(gs_next[4]),
+              "=&v"(gs_next[5]), "=&v"(gs_next[6]), "=&v"(gs_next[7])
+            : "v"(ga) : "memory");
+    };
+    auto settle_scales = [&]() {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            asm volatile("" : "+v"(gs_next[t]));
+            gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
+        }
+    };
+    // A quarter of one j group (4..8 VALU instructions): chunk = 4j + 2*half + word; see stream_tile_mb.
+    h2 part[2];
+    auto chunk = [&](int ck, int set, h8 (&frag)[8]) {
+        const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
+        uint32_t q4 = wq[set][word][j];
+        uint32_t q2 = 0;
+        asm volatile("" : "+v"(q4));
+        wq[set][word][j] = q4;
+        if (FP6) {
+            uint32_t t = tq[set][word][j >> 1];
+            asm volatile("" : "+v"(t));
+            tq[set][word][j >> 1] = t;
+            q2 = t << (4 * (j & 1));
+        }
+        h2 r0, r1;
+        dequant_half<FP6>(q2, q4, half, kc, r0, r1);
+        if (kGroup) {
+            r0 = r0 * gs_cur[2 * j + half];
+            r1 = r1 * gs_cur[2 * j + half];
+        }
+        if (word == 0) {
+            part[0] = r0;
+            part[1] = r1;
+            asm volatile("" : "+v"(part[0]), "+v"(part[1]));
+        } else {
+            frag[2 * j + half] = join(part[0], part[1], r0, r1);
+            asm volatile("" : "+v"(frag[2 * j + half]));
+        }
+    };
+
+    issue_a();                                            // pair 0
+    issue_w(0);                                           // steps 0 and 1
+    issue_w(1);                                           // (an odd step: never with group scales)
+    h8 frag[2][8];
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWOps));        // all but the words of step 1
+    lds_read_a4<0>(cx.abuf[0], cx.addr_cur);
+    lds_read_a4<kPairBlock>(cx.abuf[1], cx.addr_cur);
+    if (kGroup) fetch_scales(step_begin >> 2);
+    __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
+    if (kGroup) settle_scales();
+#pragma unroll
+    for (int ck = 0; ck < 16; ck++) chunk(ck, 0, frag[0]);
+#pragma unroll 1
+    for (int s = step_begin; s < step_end; s += kUnroll) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+            const bool scales = issue_w(u & 1);                       // step s+u+2 (its set was drained a step ago)
+            if ((u & 1) == 0) issue_a();                              // the pair after this one
+            // the words of step s+u+1 have landed, and any group scales issued before them (its A did so half a
+            // step earlier); group scales only ever go out in a pair's first step
+            if ((u & 1) == 0 && scales)
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(kAOps + kWOps + 1));
+            else
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(kAOps + kWOps));
+            const bool next_group = kGroup && u == kUnroll - 1;       // step s+u+1 starts a 128-row group
+            if (next_group) fetch_scales((s + u + 1) >> 2);
+            h8 (&cur)[8] = frag[u & 1];
+            h8 (&nxt)[8] = frag[(u + 1) & 1];
+            auto hook = [&](auto blk, auto t) {
+                constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
+                constexpr int avail = 8 * MB - 8;                     // chunks go after the MFMAs of blocks >= 1
+                if constexpr (mslot == 8) {
+                    if (next_group) settle_scales();
+                }
+                if constexpr (mslot >= 8) {
+                    constexpr int c0 = (mslot - 8) * 16 / avail, c1 = (mslot - 7) * 16 / avail;
+#pragma unroll
+                    for (int ck = c0; ck < c1; ck++) chunk(ck, (u + 1) & 1, nxt);
+                }
+            };
+            if ((u & 1) == 0) {
+                MbBlocks<MB, 0>::template run<0, 0>(cx, cur, acc, hook);
+            } else {
+#pragma unroll
+                for (int d = 0; d < 4; d++) cx.addr_next[d] = cx.addr_cur[d] + to_next;
+                if (next_group)                                        // (the reads of the group scales sit between A(1) and A(2))
+                    MbBlocks<MB, 8>::template run<0, 1, kWOps>(cx, cur, acc, hook);
+                else
+                    MbBlocks<MB, 0>::template run<0, 1, kWOps>(cx, cur, acc, hook);
+#pragma unroll
+                for (int d = 0; d < 4; d++) cx.addr_cur[d] = cx.addr_next[d];   // on to the next pair's slot
+                to_next = 0u - to_next;
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    // MFMA results -> VALU reads: the wait states, then every accumulator is passed through an (empty)
+    // asm so that no read of it can be scheduled above them.
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            asm volatile("" : "+v"(acc[mb][t]));
+        }
+    // loads into the word registers may still have been in flight up to the wait above
+#pragma unroll
+    for (int set = 0; set < 2; set++) {
+        asm volatile("" : "+v"(wq[set][0]), "+v"(wq[set][1]));
+        if (FP6) asm volatile("" : "+v"(tq[set][0]), "+v"(tq[set][1]));
+    }
     if (FP6) {
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
@@ -516,10 +795,14 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 
 // WK = k slices (waves) per workgroup: four, or eight (one workgroup per CU, two waves per SIMD) for grids that
 // would otherwise leave every SIMD a single wave.
-template <bool G128, int MB, int D4, int D6, int WK>
+// PAIR: the INT4 tiles fetch A by pairs of steps and their words through registers (stream_tile_mbp).
+template <bool G128, int MB, int D4, int D6, int WK, bool PAIR>
 __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
 {
-    constexpr int kWaveLds = mb_wave_lds(MB, D4, D6);
+    // (FP6 tiles keep the ring: with the 2-bit plane's registers on top, the paired loop no longer fits 256 VGPRs.)
+    constexpr bool kPaired = PAIR;
+    static_assert(!PAIR || MB == 4, "stream_tile_mbp is written for four blocks");
+    constexpr int kWaveLds = kPaired ? max3(mbp_wave_lds(MB), mb_wave_lds(MB, 0, D6), 0) : mb_wave_lds(MB, D4, D6);
     static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];
 
@@ -538,10 +821,17 @@ __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const
         for (int t = 0; t < 8; t++) acc[mb][t] = f4{0.f, 0.f, 0.f, 0.f};
     unsigned char* ring = smem + wave * kWaveLds;
     if (step_begin < step_end) {
-        if (ti.fp6)
-            stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
-        else
-            stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
+        if constexpr (kPaired) {
+            if (ti.fp6)
+                stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+            else
+                stream_tile_mbp<false, G128, MB>(p, ti, ring, step_begin, step_end, acc);
+        } else {
+            if (ti.fp6)
+                stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+            else
+                stream_tile_mb<false, G128, D4, MB>(p, ti, ring, step_begin, step_end, acc);
+        }
     }
     FP6M_MARK(p, 2);
     constexpr int BPR = kWaveLds >= 2 * 16 * kRedStride * 4 ? 2 : 1;  // the drained rings hold two blocks per wave

@@ -175,6 +175,24 @@ def test_eight_k_slices_per_workgroup(oracle):
     run(oracle, 40, 512, 8192, qc=256, gs=128)
 
 
+def test_paired_activation_fetch_of_the_four_block_kernel(oracle):
+    """The m > 32 kernel with the activations fetched a pair of k steps at a time and the INT4 words through
+    registers (picked from 65 rows on), forced on and off: ragged row counts (row groups of eight that are partly
+    or wholly past m), one k unit per slice, group scales or not, FP6-only and INT4-only problems, eight or four
+    slices per workgroup, several launches."""
+    for pair in (1, 0):
+        for wk in (8, 4):
+            e = {"FP6M_PAIR": pair, "FP6M_WK": wk}
+            for m in (33, 41, 64, 65, 100, 128, 199):
+                run(oracle, m, 512, 1024, qc=256, gs=128, env=e)
+            run(oracle, 48, 768, 512, qc=128, env=e)
+            run(oracle, 70, 256, 64, qc=-1, env=e)                      # one k unit: idle slices
+            run(oracle, 130, 512, 2048, qc=256, ksplit=3, env=e)
+            run(oracle, 77, 512, 512, qc=512, ksplit=2, env=e)          # all FP6: every tile on the ring path
+            run(oracle, 300, 256, 1024, qc=-1, gs=128, max_par=2, env=e)   # three launches, the last of 44 rows
+    run(oracle, 256, 2048, 2048, qc=256, gs=128)                        # the dispatcher's own choice of it
+
+
 def test_decode_kernel_with_eight_waves_per_workgroup(oracle):
     """The m <= 16 kernel with eight k slices per workgroup (picked for grids of about one workgroup per CU, e.g.
     8192 x 10240 at m = 1), forced on small and ragged problems, with and without a k split across workgroups."""
