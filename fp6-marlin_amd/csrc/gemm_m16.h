@@ -115,17 +115,21 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
         dma16_stream(base4 + v4, dst);
         dma16_stream(base4 + row4 + v4, dst + 1024);
         if (FP6) dma16_stream(base2 + v2, dst + 2048);
-        if (kGroup && (issued & 3) == 0)
+        const bool scales = kGroup && (issued & 3) == 0;  // (never again once `issued` stops at the last, odd step)
+        if (scales)
             dma4(base_gs + (size_t)(issued >> 2) * p.n4 * 2 + vgs, gs_ring + ((issued >> 2) & kScaleMask) * 256);
         if (issued < last) {                              // uniform: pointers move on the scalar unit
             issued++;
             base4 += 2 * row4;
             base2 += 2 * row2;
         }
+        return scales;
     };
     // Loads that may stay in flight while the oldest fetched step must have landed: those of the DEPTH - 2 newer
-    // steps, the first of which is the second of its pair (kWaitOdd) or the first (kWaitEven).  The occasional
-    // load of group scales only makes the wait stricter.
+    // steps, the first of which is the second of its pair (kWaitOdd) or the first (kWaitEven), plus the load of
+    // group scales that closes the fetch of every fourth step, for as long as that step is among the newer ones
+    // (left out of the count, it made two steps in four wait for a load issued only one step earlier).
+    static_assert(!kGroup || DEPTH == 4, "the steps whose waits count a load of group scales are written out for depth 4");
     constexpr int kWaitOdd = newer_step_ops(kWordOps, kAOps, 1, DEPTH - 2);
     constexpr int kWaitEven = newer_step_ops(kWordOps, kAOps, 0, DEPTH - 2);
 
@@ -205,17 +209,27 @@ __device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& t
     fetch(regs[0], 0, 0, false);
     int slot_rd = 1;                                      // slot of the step whose LDS reads come next
     int pair_rd = 0;                                      // A ring slot of the pair that step belongs to
+    bool scales_in_flight = false;
     f4 grp[8];
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            issue(slot_in, ((u + DEPTH - 1) & 1) == 0);
+            const bool scales = issue(slot_in, ((u + DEPTH - 1) & 1) == 0);
             slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
-            if (u & 1)                                                    // step s+u+1 has landed
-                __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));
-            else
-                __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven));
+            if (kGroup && u == 1) scales_in_flight = scales;              // the fetch of step s+4: a multiple of four
+            const bool one_more = kGroup && (u == 1 || u == 2) && scales_in_flight;
+            if (u & 1) {                                                  // step s+u+1 has landed
+                if (one_more)
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd + 1));
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));
+            } else {
+                if (one_more)
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven + 1));
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven));
+            }
             if (u & 1) pair_rd = pair_rd + 1 == kPairSlots ? 0 : pair_rd + 1;   // step s+u+1 opens a pair
             fetch(regs[(u + 1) & 1], slot_rd, pair_rd, (u & 1) == 0);
             slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;

@@ -147,7 +147,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     constexpr int kOps = 2 + MB + (FP6 ? 2 : 0);          // vector-memory loads per step
     constexpr int kUnroll = kGroup ? 4 : 2;
     constexpr int kW = 2;                                 // LDS reads of one step's weight words
-    static_assert(kOps * (DEPTH - 2) <= 63, "vmcnt is a 6-bit counter");
+    static_assert(kOps * (DEPTH - 2) + 1 <= 63, "vmcnt is a 6-bit counter");
     const int lane = threadIdx.x & 63;
     const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
 
@@ -207,7 +207,8 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
             asm volatile("global_load_dwordx2 %0, %2, %4 nt\n\tglobal_load_dwordx2 %1, %3, %4 nt"
                          : "=&v"(tq[set][0]), "=&v"(tq[set][1]) : "v"(v2), "v"(v2b), "s"(base2) : "memory");
         }
-        if (kGroup && (issued & 3) == 0) {
+        const bool scales = kGroup && (issued & 3) == 0;  // (never again once `issued` stops at the last, odd step)
+        if (scales) {
             set_m0(gs_lds + ((issued >> 2) & kScaleMask) * 256);
             dma4_m0(base_gs + (size_t)(issued >> 2) * (size_t)uniform32(p.n4) * 2, vgs);
         }
@@ -217,7 +218,12 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
             base2 += 2 * row2;
             base_a += 64;
         }
+        return scales;
     };
+    // The load of group scales closes the fetch of every fourth step and counts in the waits for as long as that
+    // step is among the DEPTH - 2 newest: the fetch goes out in sub-step kScaleU of the unrolled loop.
+    static_assert(!kGroup || DEPTH == 3 || DEPTH == 4, "sub-steps that count the load of group scales");
+    constexpr int kScaleU = (5 - DEPTH) & 3;
 
     // ---- read side
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
@@ -307,16 +313,21 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
 #pragma unroll
     for (int ck = 0; ck < 16; ck++) chunk(ck, 0, frag[0]);
     int slot_rd = 1;
+    bool scales_in_flight = false;
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            issue(slot_in, u & 1);                                    // step s+u+2 (FP6: DEPTH is 3)
+            const bool scales = issue(slot_in, u & 1);                // step s+u+2 (FP6: DEPTH is 3)
             slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
 #pragma unroll
             for (int d = 0; d < 4; d++) cx.addr_cur[d] = cx.addr_next[d];
             slot_addrs(cx.addr_next, slot_rd);
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
+            if (kGroup && u == kScaleU) scales_in_flight = scales;
+            if (kGroup && u >= kScaleU && u < kScaleU + DEPTH - 2 && scales_in_flight)
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2) + 1));
+            else
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(kOps * (DEPTH - 2)));
             // step s+u+1 (and its group scales) has landed: read its words now, dequantise them
             // between this step's MFMAs
             fetch_w(slot_rd);
