@@ -507,24 +507,38 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
-            while (ks > 1 && (size_t)base * ks * tile_bytes > kScratchBytes) ks--;
+            while (ks > 1 && (size_t)(a.tiles + a.tiles6) * mtiles * ks * tile_bytes > kScratchBytes) ks--;   // (FP6 tiles: 2 ks)
             a.ksplit = (int)ks;
             // A grid of at most one workgroup per CU would leave every SIMD a single wave: give the workgroup eight
             // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
             int wk = base * ks <= scratch->cus && units / 16 >= ks ? 8 : kWaves;
             if (const char* e = getenv("FP6M_WK")) wk = atoi(e) == 8 ? 8 : kWaves;   // tuning/testing override
+            // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
+            // FP6 tiles' workgroups set the length of the launch (8192 x 8192 at m = 128: 33 us against 29 us with INT4
+            // only).  Their k range is cut twice as finely where every slice still gets two units and the grid still
+            // fits the CUs in one go (5120 x 13824 at m = 128: 40 -> 31 us; a grid pushed into a second round loses far
+            // more than that).  A forced split applies to both kinds.
+            a.ks4 = (int)ks;
+            a.ks6 = (int)ks;
+            const long long resident = (long long)scratch->cus * (wk == 8 ? 1 : 2);
+            if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk &&
+                (base + (long long)a.tiles6 * mtiles) * ks <= resident)
+                a.ks6 = 2 * (int)ks;
             if (row_mix) {
                 a.slices4 = deal_slices(a.ksplit * wk);
                 a.rule[0] = make_rule(k4 / 128, a.slices4);
                 a.rule[1] = make_rule(fu.quant_rows / 64, a.ksplit * wk - a.slices4);
             } else {
-                a.rule[0] = a.rule[1] = make_rule(units, a.ksplit * wk);
+                a.rule[0] = make_rule(units, a.ks4 * wk);
+                a.rule[1] = make_rule(units, a.ks6 * wk);
             }
-            a.div[0] = a.div[1] = make_div(a.ksplit, (long long)a.tiles * a.ksplit);
-            dim3 grid((unsigned)(a.tiles * a.ksplit), (unsigned)mtiles);
+            const long long wgs = (long long)a.tiles6 * a.ks6 + (long long)(a.tiles - a.tiles6) * a.ks4;
+            a.div[0] = make_div(a.ks4, wgs);
+            a.div[1] = make_div(a.ks6, wgs);
+            dim3 grid((unsigned)wgs, (unsigned)mtiles);
             if (getenv("FP6M_VERBOSE"))
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks=%d k slices %d grid=%ux%u\n", a.m, prob_n, prob_k,
-                        mb, mtiles, a.ksplit, wk, grid.x, grid.y);
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks4=%d ks6=%d k slices %d grid=%ux%u\n", a.m, prob_n,
+                        prob_k, mb, mtiles, a.ks4, a.ks6, wk, grid.x, grid.y);
             // From two row tiles on, the requests A costs weigh more than the shorter look-ahead of the paired fetch
             // (measured: 64 rows 1-3 % slower with it, 128 rows 0-8 % faster, 256 and 512 rows 4-14 %).
             bool pair = a.m > 64;

@@ -69,7 +69,7 @@ struct GemmArgs {
     // Division-free bookkeeping, prepared by the host (a 64-bit division costs a wave hundreds of scalar
     // instructions before its first load):
     SliceRule rule[2];        // k slices of a tile: [0] INT4 tiles / INT4 rows (all tiles for m > 16), [1] FP6
-    FastDiv div[2];           // m <= 16: by groups4 / groups6;  m > 16: [0] by ksplit
+    FastDiv div[2];           // m <= 16: by groups4 / groups6;  m > 16: by ks4 / ks6 (the large-m kernel: [0] by ksplit)
     // weight planes in the gfx950 order (fp6m_repack_gfx950): [tile][k-block][MFMA lane] instead of the reference's
     // [k-block][64-column group][fragment owner]
     int native;
@@ -217,15 +217,21 @@ __device__ __forceinline__ PlaneGeometry plane_geometry(const GemmArgs& p, const
     return g;
 }
 
+// The m > 16 kernel's workgroup: blockIdx.x walks the FP6 tiles' (tile, k part) pairs first (ks6 parts each), then the
+// INT4 tiles' (ks4 parts each); blockIdx.y the row tiles.
 __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 {
     TileInfo t;
     const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    t.tile = fast_div(p.div[0], logical);
-    t.part = logical - t.tile * p.ksplit;
+    const int wgs6 = p.tiles6 * p.ks6;
+    t.fp6 = logical < wgs6;
+    const int local = t.fp6 ? logical : logical - wgs6;
+    // (both entries are read at fixed offsets and selected by value: an index would become a dependent scalar load)
+    const FastDiv kdiv = {t.fp6 ? p.div[1].d : p.div[0].d, t.fp6 ? p.div[1].magic : p.div[0].magic};
+    t.tcol = fast_div(kdiv, local);
+    t.part = local - t.tcol * (t.fp6 ? p.ks6 : p.ks4);
+    t.tile = t.fp6 ? t.tcol : p.tiles6 + t.tcol;
     t.mtile = blockIdx.y;
-    t.fp6 = t.tile < p.tiles6;
-    t.tcol = t.fp6 ? t.tile : t.tile - p.tiles6;
     t.region_n = t.fp6 ? p.qc : p.n4;
     t.col0 = (t.fp6 ? p.n4 : 0) + t.tcol * kTileN;
     t.a_step0 = 0;
@@ -235,12 +241,13 @@ __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 // k range of one wave in steps of 32 (two k-blocks).  Units of two steps (four with group scales) keep
 // every wave's step count even and group-aligned.
 template <bool G128, int WK = kWaves>
-__device__ __forceinline__ void wave_k_range(const GemmArgs& p, int part, int wave, int& begin, int& end)
+__device__ __forceinline__ void wave_k_range(const GemmArgs& p, bool fp6, int part, int wave, int& begin, int& end)
 {
     constexpr int unit_steps = G128 ? 4 : 2;
     const int wv = part * WK + wave;
-    begin = slice_begin(p.rule[0], wv) * unit_steps;
-    end = slice_begin(p.rule[0], wv + 1) * unit_steps;
+    const SliceRule rule = {fp6 ? p.rule[1].q : p.rule[0].q, fp6 ? p.rule[1].first_long : p.rule[0].first_long};
+    begin = slice_begin(rule, wv) * unit_steps;
+    end = slice_begin(rule, wv + 1) * unit_steps;
 }
 
 // ------------------------------------------------------------------------------------------------ loads, waits, dequantisers

@@ -638,7 +638,8 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
 // gemm_mb_kernel, one of WM groups in gemm_wm_kernel); a group without rows goes through the barriers
 // without touching memory.
 template <int MB, int WK = kWaves, int BPR = 1>
-__device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, f4 (&acc)[MB][8],
+__device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, int slot_base,
+                                             f4 (&acc)[MB][8],
                                              bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
                                              bool valid = true, int first_fp6 = WK)
 {
@@ -681,8 +682,7 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
         *reinterpret_cast<h2*>(c_out + (size_t)row * p.n) = o;
     };
     constexpr size_t kSlotU64 = (size_t)MB * 16 * kTileN / 2;
-    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) +
-                                (size_t)(ti.mtile * p.tiles + ti.tile) * ks * kSlotU64 + lane;
+    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) + (size_t)slot_base * kSlotU64 + lane;
     unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
 
 #pragma unroll
@@ -822,8 +822,12 @@ __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const
     TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int step_begin, step_end;
-    wave_k_range<G128, WK>(p, ti.part, wave, step_begin, step_end);
-    if (p.k4) row_mix_slice(p, ti.part * WK + wave, ti, step_begin, step_end);
+    wave_k_range<G128, WK>(p, ti.fp6, ti.part, wave, step_begin, step_end);
+    // partial-sum slots, row tile by row tile: the FP6 tiles' (tile, part), then the INT4 tiles'
+    const int ks = ti.fp6 ? p.ks6 : p.ks4;
+    const int wgs6 = p.tiles6 * p.ks6;
+    const int slot_base = ti.mtile * (wgs6 + (p.tiles - p.tiles6) * p.ks4) + (ti.fp6 ? ti.tcol * p.ks6 : wgs6 + ti.tcol * p.ks4);
+    if (p.k4) row_mix_slice(p, ti.part * WK + wave, ti, step_begin, step_end);   // (no FP6 column tiles in a row mix)
 
     f4 acc[MB][8];
 #pragma unroll
@@ -846,7 +850,7 @@ __global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const
     }
     FP6M_MARK(p, 2);
     constexpr int BPR = kWaveLds >= 2 * 16 * kRedStride * 4 ? 2 : 1;  // the drained rings hold two blocks per wave
-    wg_finish_mb<MB, WK, BPR>(p, ti, wave, p.ksplit, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+    wg_finish_mb<MB, WK, BPR>(p, ti, wave, ks, slot_base, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
                          reinterpret_cast<int*>(smem + WK * kWaveLds), true, p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
 }

@@ -351,8 +351,8 @@ __global__ __launch_bounds__(512, 2) void gemm_wm_kernel(const GemmArgs p)
     else
         stream_tile_wm<false, G128, WN>(p, ti, slice, wm, wn, step_begin, step_end, step_begin + longest, acc);
     const int grp = wn * WM + wm;                                    // the WK waves that share a tile and a row tile
-    wg_finish_mb<MB, WK>(p, ti, wk, p.ksplit, acc, ti.fp6 || !G128, smem + grp * WK * kWmRegion, kWmRegion,
-                         reinterpret_cast<int*>(smem + wm_lds<WN>() - 64) + grp, valid);
+    wg_finish_mb<MB, WK>(p, ti, wk, p.ksplit, (ti.mtile * p.tiles + ti.tile) * p.ksplit, acc, ti.fp6 || !G128,
+                         smem + grp * WK * kWmRegion, kWmRegion, reinterpret_cast<int*>(smem + wm_lds<WN>() - 64) + grp, valid);
 }
 
 }  // namespace fp6m

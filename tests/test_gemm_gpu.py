@@ -193,6 +193,19 @@ def test_paired_activation_fetch_of_the_four_block_kernel(oracle):
     run(oracle, 256, 2048, 2048, qc=256, gs=128)                        # the dispatcher's own choice of it
 
 
+def test_fp6_tiles_with_a_finer_k_split_than_int4_tiles(oracle):
+    """m > 16 in a grid that is resident at once: the FP6 tiles' k range is cut into twice as many parts as the INT4
+    tiles' (their own slice rule, divisor, partial-sum slots and counters); here 2 against 1 and 4 against 2, with
+    group scales and without, ragged rows, both loops of the four-block kernel and the two-block one."""
+    for pair in (1, 0):
+        e = {"FP6M_PAIR": pair}
+        run(oracle, 100, 512, 4096, qc=256, gs=128, sms=1, env=e)
+        run(oracle, 100, 512, 2048, qc=256, sms=1, env=e)
+        run(oracle, 70, 768, 8192, qc=384, gs=128, sms=2, env=e)
+    run(oracle, 24, 512, 4096, qc=256, gs=128, sms=1)
+    run(oracle, 130, 768, 4096, qc=256, sms=1, env={"FP6M_VERBOSE": 1})
+
+
 def test_decode_kernel_with_eight_waves_per_workgroup(oracle):
     """The m <= 16 kernel with eight k slices per workgroup (picked for grids of about one workgroup per CU, e.g.
     8192 x 10240 at m = 1), forced on small and ragged problems, with and without a k split across workgroups."""
