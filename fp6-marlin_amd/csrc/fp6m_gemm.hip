@@ -437,7 +437,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     const double load = (double)(a.groups4 * c + a.groups6 * c6) / scratch->cus;
                     double t;
                     if (wk == 4) {
-                        if (load > 3.0) return 1e9;
+                        if (load > (cfg.id == 1 ? 2.0 : 3.0)) return 1e9;   // what a CU's LDS holds at once (16 rows of A: two)
                         t = load <= 1.0 ? 0.40 : (load <= 1.9 ? 0.56 : (load <= 2.0 ? 0.72 : 1.10));
                     } else {
                         // eight waves per workgroup paid off only with one workgroup on (nearly) every CU: measured
