@@ -14,7 +14,10 @@
 //    arrives last (one atomic counter per tile in `workspace`) sums the partials in a fixed order,
 //    applies the scales and writes fp16 C.  Nobody spins, so there is nothing to deadlock on, and the
 //    counters are zero again when the launch drains.
-//  * INT4 and FP6 tiles are entries of one tile list handled by the same launch.
+//  * INT4 and FP6 tiles are entries of one tile list handled by the same launch; FP6 tiles, whose steps cost
+//    more, may have their k range cut into twice as many parts.
+//  * Activations are fetched a whole 128-byte line of every row at a time (two k steps): a wave's rate is set by
+//    its memory requests in flight, not by their bytes.
 //  * The dispatcher picks the kernel by m, and for m <= 16 the waves per workgroup and the k split per shape
 //    (a rule plus a small cost model fitted to per-workgroup timelines on MI355X).
 //

@@ -6,9 +6,11 @@ namespace fp6m {
 
 // ------------------------------------------------------------------------------------------------ 16 < m: ring kernel with MB row blocks
 //
-// Same ring and lane routing as the m <= 16 kernel, but a slot carries MB blocks of 16 rows of A (1 KiB
-// each) and every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per
-// 16*MB rows.  A workgroup is one tile x four k slices; blockIdx.y walks the row tiles.  Group scales are
+// Same lane routing and k-sliced workgroup as the m <= 16 kernel, but a wave multiplies MB blocks of 16 rows of A and
+// every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per 16*MB rows.  Two
+// loops: stream_tile_mb keeps the words and one step of A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (INT4
+// tiles of launches with more than 64 rows) fetches A a pair of steps at a time and the words through registers.
+// A workgroup is one tile x four or eight k slices; blockIdx.y walks the row tiles.  Group scales are
 // applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more
 // registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
 // the number of direct-to-LDS loads per step is constant) and never stored.
