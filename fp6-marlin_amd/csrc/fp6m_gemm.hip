@@ -420,7 +420,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if (c > traffic_cap) c = traffic_cap;
                 return c;
             };
-            auto ks6_of = [&](long long c, int wk) { return 2 * c <= ks_units(wk) ? 2 * c : (c > ks_units(wk) ? c : ks_units(wk)); };
+            // FP6 tiles are split twice as finely as INT4 tiles (their steps move 1.5x the bytes); with FP6 tiles only
+            // there is nothing to keep step with and the split is the one asked for
+            auto ks6_of = [&](long long c, int wk) {
+                if (a.groups4 == 0) return c < ks_units(wk) ? c : ks_units(wk);
+                return 2 * c <= ks_units(wk) ? 2 * c : (c > ks_units(wk) ? c : ks_units(wk));
+            };
             // Measured on MI355X: with four waves per workgroup the kernel is fastest with about one and a half
             // workgroups per CU (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle).
             const long long target_wgs = (long long)scratch->cus * 3 / 2;
