@@ -524,8 +524,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
             // FP6 tiles' workgroups set the length of the launch (8192 x 8192 at m = 128: 33 us against 29 us with INT4
             // only).  Their k range is cut twice as finely where every slice still gets two units and the grid still
-            // fits the CUs in one go (5120 x 13824 at m = 128: 40 -> 31 us; a grid whose last workgroups must wait for a free CU loses far
-            // more than that).  A forced split applies to both kinds.
+            // fits the CUs in one go (5120 x 13824 at m = 128: 40 -> 31 us; a grid whose last workgroups must wait for
+            // a free CU loses far more than that).  A forced split applies to both kinds.
             a.ks4 = (int)ks;
             a.ks6 = (int)ks;
             const long long resident = (long long)scratch->cus * (wk == 8 ? 1 : 2);
