@@ -47,7 +47,9 @@ def weight_bytes(k, n, qc, gs):
 
 
 class Problem:
-    """Device operands of one (m, k, n) GEMM with random packed words."""
+    """Device operands of one (m, k, n) GEMM with random packed words.  All problems share one workspace: the
+    benchmark's calls run back to back on one stream (the library keeps a partial-sum region per workspace)."""
+    shared_ws = None
 
     def __init__(self, torch, m, k, n, qc, gs, gen, fp16_ref=False):
         dev = torch.device("cuda:0")
@@ -59,7 +61,11 @@ class Problem:
         self.s = (torch.rand(ns, generator=gen) * 0.01 + 0.001).half().to(dev)
         self.A = torch.randn((m, k), generator=gen).half().to(dev)
         self.C = torch.zeros((m, n), dtype=torch.half, device=dev)
-        self.ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev)
+        if Problem.shared_ws is None:
+            import fp6_marlin
+            Problem.shared_ws = fp6_marlin.init_workspace(torch.zeros(65536, dtype=torch.int32, device=dev))
+        assert n // 128 * 16 <= Problem.shared_ws.numel()
+        self.ws = Problem.shared_ws
         self.W16 = (torch.randn((k, n), generator=gen) * 0.02).half().to(dev) if fp16_ref else None
         self.bytes = weight_bytes(k, n, qc, gs)
         self.flops = 2 * m * k * n

@@ -172,6 +172,7 @@ const char* fp6m_strerror(int code)
         case FP6M_ERR_ARG: return "invalid argument";
         case FP6M_ERR_HIP: return "HIP runtime error";
         case FP6M_ERR_NO_GPU_CODE: return "library built without gfx950 kernels";
+        case FP6M_ERR_SCRATCH: return "the problem's partial sums do not fit this entry point's scratch: use fp6m_mul";
         default: return "unknown fp6m error";
     }
 }

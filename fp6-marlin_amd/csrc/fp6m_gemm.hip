@@ -30,6 +30,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 
 #include "fp6m.h"
@@ -60,14 +61,37 @@ __global__ __launch_bounds__(256) void gather_a_kernel(const uint16_t* __restric
 
 thread_local int g_last_hip_error = 0;
 
-struct DeviceScratch {
-    float* ptr = nullptr;
-    int cus = 0;
-    uint16_t* gathered = nullptr;   // gathered activations of fp6m_mul_fused (kGatherBytes, on first use)
+// Overrides of the dispatcher's choices, for tests and tuning runs (fp6m_tuning_set).  The product path reads no
+// environment variables; FP6M_VERBOSE alone is looked up once, when the library is loaded.
+constexpr int kUnset = INT32_MIN;
+struct Tuning {
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset;
+    int verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
+};
+Tuning g_tuning;
+
+// Device memory the GEMM needs beyond its operands: fp32 partial tiles of column tiles whose k range is shared by
+// several workgroups, and the buffer that gathered activations pass through.  The reference keeps its partial sums
+// in C under the locks in the caller's `workspace`, so its rule is one call at a time per workspace, and two calls
+// with two workspaces may overlap.  Here the rule is the same because the scratch belongs to the workspace: every
+// workspace address that has been seen on a device owns a region, allocated on its first call (or by
+// fp6m_init_workspace) and kept until fp6m_release_workspace.  The table is bounded; when it is full the library
+// waits for the device and frees every region, which is safe because nothing is in flight then.
+struct Region {
+    const void* workspace = nullptr;
+    float* partials = nullptr;      // kScratchBytes of partial tiles
+    uint16_t* gathered = nullptr;   // kGatherBytes, allocated by the first gathering call with this workspace
 };
 constexpr size_t kGatherBytes = size_t(64) << 20;
 constexpr int kMaxDevices = 64;
-DeviceScratch g_scratch[kMaxDevices];
+constexpr int kMaxRegions = 128;    // per device
+struct DeviceState {
+    int cus = 0;
+    int nregions = 0;
+    void* pack_temp = nullptr;      // kPackTempBytes for the on-GPU packer's flag and column maxima
+    Region regions[kMaxRegions];
+};
+DeviceState g_devices[kMaxDevices];
 std::mutex g_scratch_mutex;
 
 int hip_fail(hipError_t e)
@@ -76,53 +100,103 @@ int hip_fail(hipError_t e)
     return FP6M_ERR_HIP;
 }
 
-int ensure_scratch(int dev, DeviceScratch** out)
+// Runs `fn` with `dev` as the calling thread's current device and puts the previous one back.
+template <typename F>
+hipError_t on_device(int dev, F&& fn)
+{
+    int prev = 0;
+    hipError_t e = hipGetDevice(&prev);
+    if (e != hipSuccess) return e;
+    if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) return e;
+    e = fn();
+    if (prev != dev) (void)hipSetDevice(prev);
+    return e;
+}
+
+// Compute units of the device (queried once; no allocation).  Callers hold g_scratch_mutex.
+int device_state(int dev, DeviceState** out)
 {
     if (dev < 0 || dev >= kMaxDevices) return FP6M_ERR_ARG;
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    DeviceScratch& d = g_scratch[dev];
-    if (!d.ptr) {
-        int prev = 0;
-        hipError_t e = hipGetDevice(&prev);
-        if (e != hipSuccess) return hip_fail(e);
-        if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) return hip_fail(e);
-        void* mem = nullptr;
-        e = hipMalloc(&mem, kScratchBytes + kPackTempBytes);          // partial tiles, then the packer's scratch
+    DeviceState& d = g_devices[dev];
+    if (!d.cus) {
         int cus = 0;
-        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        if (prev != dev) (void)hipSetDevice(prev);
+        const hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (e != hipSuccess) return hip_fail(e);
-        d.ptr = static_cast<float*>(mem);
         d.cus = cus > 0 ? cus : 256;
     }
     *out = &d;
     return FP6M_OK;
 }
 
-// The buffer the gathered activations of fp6m_mul_fused go through: allocated on the first call that gathers.
-int ensure_gather_buffer(int dev, DeviceScratch* d)
+// Frees every region of the device after waiting for it.  Callers hold g_scratch_mutex.
+hipError_t free_regions(int dev, DeviceState& d)
+{
+    return on_device(dev, [&] {
+        hipError_t e = hipDeviceSynchronize();
+        for (int i = 0; i < d.nregions && e == hipSuccess; i++) {
+            e = hipFree(d.regions[i].partials);
+            if (e == hipSuccess && d.regions[i].gathered) e = hipFree(d.regions[i].gathered);
+            d.regions[i] = Region{};
+        }
+        if (e == hipSuccess) d.nregions = 0;
+        return e;
+    });
+}
+
+// The region of `workspace` on `dev`; the first call for an address allocates it (zeroed: the reduction protocols
+// leave what they use zeroed and rely on finding it so).
+int workspace_region(int dev, const void* workspace, bool want_gather, DeviceState** dev_out, Region** out)
 {
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (d->gathered) return FP6M_OK;
-    int prev = 0;
-    hipError_t e = hipGetDevice(&prev);
-    if (e != hipSuccess) return hip_fail(e);
-    if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) return hip_fail(e);
-    void* mem = nullptr;
-    e = hipMalloc(&mem, kGatherBytes);
-    if (prev != dev) (void)hipSetDevice(prev);
-    if (e != hipSuccess) return hip_fail(e);
-    d->gathered = static_cast<uint16_t*>(mem);
+    DeviceState* d = nullptr;
+    if (int rc = device_state(dev, &d)) return rc;
+    Region* r = nullptr;
+    for (int i = 0; i < d->nregions; i++)
+        if (d->regions[i].workspace == workspace) r = &d->regions[i];
+    if (!r) {
+        if (d->nregions == kMaxRegions) {
+            const hipError_t e = free_regions(dev, *d);
+            if (e != hipSuccess) return hip_fail(e);
+        }
+        void* mem = nullptr;
+        const hipError_t e = on_device(dev, [&] {
+            hipError_t e2 = hipMalloc(&mem, kScratchBytes);
+            if (e2 == hipSuccess) e2 = hipMemset(mem, 0, kScratchBytes);
+            return e2;
+        });
+        if (e != hipSuccess) {
+            if (mem) (void)hipFree(mem);
+            return hip_fail(e);
+        }
+        r = &d->regions[d->nregions++];
+        r->workspace = workspace;
+        r->partials = static_cast<float*>(mem);
+        r->gathered = nullptr;
+    }
+    if (want_gather && !r->gathered) {
+        void* mem = nullptr;
+        const hipError_t e = on_device(dev, [&] { return hipMalloc(&mem, kGatherBytes); });
+        if (e != hipSuccess) return hip_fail(e);
+        r->gathered = static_cast<uint16_t*>(mem);
+    }
+    *dev_out = d;
+    *out = r;
     return FP6M_OK;
 }
 
-// Scratch of the on-GPU packer (fp6m_pack.hip): kPackTempBytes behind the partial-sum tiles.
+// Scratch of the on-GPU packer (fp6m_pack.hip): one buffer per device (a pack call waits for its kernels).
 int pack_temp(int dev, void** ptr)
 {
-    DeviceScratch* d = nullptr;
-    const int rc = ensure_scratch(dev, &d);
-    if (rc != FP6M_OK) return rc;
-    *ptr = reinterpret_cast<unsigned char*>(d->ptr) + kScratchBytes;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    DeviceState* d = nullptr;
+    if (int rc = device_state(dev, &d)) return rc;
+    if (!d->pack_temp) {
+        void* mem = nullptr;
+        const hipError_t e = on_device(dev, [&] { return hipMalloc(&mem, kPackTempBytes); });
+        if (e != hipSuccess) return hip_fail(e);
+        d->pack_temp = mem;
+    }
+    *ptr = d->pack_temp;
     return FP6M_OK;
 }
 
@@ -217,10 +291,66 @@ extern "C" {
 
 int fp6m_last_hip_error(void) { return fp6m::g_last_hip_error; }
 
+int fp6m_tuning_set(const char* knob, int value)
+{
+    using fp6m::g_tuning;
+    if (!knob) {                                                      // NULL: back to the dispatcher's own choices
+        const int verbose = g_tuning.verbose;
+        g_tuning = fp6m::Tuning{};
+        g_tuning.verbose = verbose;
+        return FP6M_OK;
+    }
+    const struct { const char* name; int* field; } knobs[] = {
+        {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"verbose", &g_tuning.verbose}};
+    for (const auto& k : knobs)
+        if (!strcmp(knob, k.name)) {
+            *k.field = value;
+            return FP6M_OK;
+        }
+    return FP6M_ERR_ARG;
+}
+
 int fp6m_init(int dev)
 {
-    fp6m::DeviceScratch* d = nullptr;
-    return fp6m::ensure_scratch(dev, &d);
+    std::lock_guard<std::mutex> lock(fp6m::g_scratch_mutex);
+    fp6m::DeviceState* d = nullptr;
+    return fp6m::device_state(dev, &d);
+}
+
+int fp6m_init_workspace(int dev, const void* workspace, int with_gather)
+{
+    if (!workspace) return FP6M_ERR_ARG;
+    fp6m::DeviceState* d = nullptr;
+    fp6m::Region* r = nullptr;
+    return fp6m::workspace_region(dev, workspace, with_gather != 0, &d, &r);
+}
+
+int fp6m_release_workspace(int dev, const void* workspace)
+{
+    using namespace fp6m;
+    if (dev < 0 || dev >= kMaxDevices) return FP6M_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    DeviceState& d = g_devices[dev];
+    if (!workspace) {                                                 // all regions of the device
+        const hipError_t e = free_regions(dev, d);
+        return e == hipSuccess ? FP6M_OK : hip_fail(e);
+    }
+    for (int i = 0; i < d.nregions; i++) {
+        if (d.regions[i].workspace != workspace) continue;
+        const Region r = d.regions[i];
+        const hipError_t e = on_device(dev, [&] {
+            hipError_t e2 = hipDeviceSynchronize();                   // nothing in flight may still use the region
+            if (e2 == hipSuccess) e2 = hipFree(r.partials);
+            if (e2 == hipSuccess && r.gathered) e2 = hipFree(r.gathered);
+            return e2;
+        });
+        if (e != hipSuccess) return hip_fail(e);
+        d.regions[i] = d.regions[--d.nregions];
+        d.regions[d.nregions] = Region{};
+        return FP6M_OK;
+    }
+    return FP6M_OK;                                                   // no region: nothing to release
 }
 
 }  // extern "C"
@@ -279,8 +409,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     const bool g128 = group_size == 128 && n4 > 0;
     if (g128 && prob_k % 128 && !row_mix) return FP6M_ERR_PROB_SHAPE;
 
-    DeviceScratch* scratch = nullptr;
-    if (int rc = ensure_scratch(dev, &scratch)) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DeviceState* device = nullptr;
+    Region* region = nullptr;
+    const size_t scratch_bytes = kScratchBytes;
+    if (int rc = workspace_region(dev, workspace, fu.a_cols != nullptr, &device, &region)) return rc;
+    const int cus = device->cus;
 
     GemmArgs a;
     a.b_int4 = static_cast<const uint32_t*>(B);
@@ -288,7 +422,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.b_fp6_4 = a.b_fp6_2 + (size_t)prob_k * qc / 16;
     a.s_int4 = static_cast<const uint16_t*>(s);
     a.s_fp6 = a.s_int4 + (g128 ? (size_t)(prob_k / 128) * n4 : (size_t)n4);
-    a.scratch = scratch->ptr;
+    a.scratch = region->partials;
     a.counters = static_cast<int*>(workspace);
     a.n = prob_n;
     a.k = prob_k;
@@ -320,17 +454,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     // workgroups per CU) beyond.  128-row blocks (accumulators in AGPRs, one wave per SIMD) measured 10-15 %
     // faster for m >= 512 but left the register allocator no slack, and were dropped.
     int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
-    if (const char* e = getenv("FP6M_MB")) {   // tuning/testing override
-        const int v = atoi(e);
-        if (prob_m > 16 && (v == 2 || v == 4)) mb = v;
-    }
+    const Tuning tune = g_tuning;              // tuning/testing overrides (all unset in production)
+    if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4)) mb = tune.mb;
     // Launches of 1024 rows on large weights: four 64-row tiles share the dequantised fragments of a tile
     // (gemm_wm_kernel).  Measured on MI355X it beats the private-fragment kernel by 13-20 % there and loses
     // below (m = 512: 102 vs 96 us on 8192 x 8192), where its 256-row workgroups leave CUs idle.
     const long long rows_per_launch = prob_m < 64LL * max_par ? prob_m : 64LL * max_par;
     const long long weights = (long long)prob_n * prob_k;
     bool shared_frags = rows_per_launch >= 1024 && weights >= (64LL << 20);
-    if (const char* e = getenv("FP6M_WM")) shared_frags = prob_m > 16 && atoi(e) != 0;   // tuning/testing override
+    if (tune.wm != kUnset) shared_frags = prob_m > 16 && tune.wm != 0;
     if (row_mix) shared_frags = false;                                // its waves run in lock step on one segment
     // Row mix: the kWaves * ks slices of a tile are dealt to the two segments in proportion to their cost (an FP6
     // step costs about two INT4 steps), at least one each.
@@ -347,11 +479,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
     const int units = g128 ? prob_k / 128 : prob_k / 64;
 
-    hipStream_t st = static_cast<hipStream_t>(stream);
     if (fu.a_cols) {
         const long long launch_rows = prob_m < (long long)rows_per_tile * max_par ? prob_m : (long long)rows_per_tile * max_par;
         if ((size_t)launch_rows * prob_k * sizeof(uint16_t) > kGatherBytes) return FP6M_ERR_ARG;
-        if (int rc = ensure_gather_buffer(dev, scratch)) return rc;
     }
     for (int mt0 = 0; mt0 < mtiles_total; mt0 += max_par) {
         const int mtiles = mtiles_total - mt0 < max_par ? mtiles_total - mt0 : max_par;
@@ -364,27 +494,26 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             dim3 ggrid((unsigned)((prob_k / 2 + 255) / 256), (unsigned)a.m);
             hipLaunchKernelGGL(gather_a_kernel, ggrid, dim3(256), 0, st,
                                static_cast<const uint16_t*>(A) + (size_t)rows0 * fu.lda, fu.lda, fu.a_cols,
-                               scratch->gathered, prob_k);
-            a.A = scratch->gathered;
+                               region->gathered, prob_k);
+            a.A = region->gathered;
         } else {
             a.A = static_cast<const uint16_t*>(A) + (size_t)rows0 * prob_k;
         }
 
         const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
         const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
-        long long env_ks = 0;
-        if (const char* e = getenv("FP6M_KSPLIT")) env_ks = atoi(e);   // tuning/testing override
+        const long long env_ks = tune.ksplit != kUnset ? tune.ksplit : 0;
         if (shared_frags) {
             // two tiles per workgroup also share the A slabs: pays once the weights are large enough that
             // halving the grid still fills the chip (measured: 8192 x 16384 and up)
             int wn = weights >= (128LL << 20) ? 2 : 1;
-            if (const char* e = getenv("FP6M_WN")) wn = atoi(e) == 2 ? 2 : 1;   // tuning/testing override
+            if (tune.wn != kUnset) wn = tune.wn == 2 ? 2 : 1;
             const int wk = 2 / wn;
             a.groups6 = (a.tiles6 + wn - 1) / wn;
             a.groups4 = (a.tiles - a.tiles6 + wn - 1) / wn;
             const int groups_m = (mtiles + fp6m::kWmRows - 1) / fp6m::kWmRows;
             const long long base = (long long)(a.groups6 + a.groups4) * groups_m;
-            long long ks = scratch->cus / base;
+            long long ks = cus / base;
             const long long ks_k = units / (wk * 2) > 0 ? units / (wk * 2) : 1;
             const long long cap = (long long)prob_k / (16LL * rows_per_tile) > 0 ? (long long)prob_k / (16LL * rows_per_tile) : 1;
             if (ks > ks_k) ks = ks_k;
@@ -392,12 +521,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
-            while (ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > kScratchBytes) ks--;
+            while (ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > scratch_bytes) ks--;
             a.ksplit = (int)ks;
             a.rule[0] = a.rule[1] = make_rule(units, a.ksplit * wk);
             a.div[0] = a.div[1] = make_div(a.ksplit, (long long)(a.groups6 + a.groups4) * a.ksplit);
             dim3 grid((unsigned)((a.groups6 + a.groups4) * a.ksplit), (unsigned)groups_m);
-            if (getenv("FP6M_VERBOSE"))
+            if (tune.verbose)
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: shared fragments, %d tile(s) x %d k slice(s), row tiles %d ks=%d grid=%ux%u\n",
                         a.m, prob_n, prob_k, wn, wk, mtiles, a.ksplit, grid.x, grid.y);
             fp6m::launch_wm(a, g128, wn, grid, st);
@@ -428,7 +557,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             };
             // Measured on MI355X: with four waves per workgroup the kernel is fastest with about one and a half
             // workgroups per CU (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle).
-            const long long target_wgs = (long long)scratch->cus * 3 / 2;
+            const long long target_wgs = (long long)cus * 3 / 2;
             long long ks = (target_wgs + groups / 2) / groups;
             if (ks > ks_limit(cfg.wk)) ks = ks_limit(cfg.wk);
             if (ks < 1) ks = 1;
@@ -442,7 +571,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             {
                 auto model_us = [&](int wk, long long c) -> double {
                     const long long c6 = a.groups6 ? ks6_of(c, wk) : 0;
-                    const double load = (double)(a.groups4 * c + a.groups6 * c6) / scratch->cus;
+                    const double load = (double)(a.groups4 * c + a.groups6 * c6) / cus;
                     double t;
                     if (wk == 4) {
                         if (load > (cfg.id == 1 ? 2.0 : 3.0)) return 1e9;   // what a CU's LDS holds at once (16 rows of A: two)
@@ -473,14 +602,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     ks = best;
                 }
             }
-            if (const char* e = getenv("FP6M_WK16")) cfg.wk = atoi(e) == 8 ? 8 : 4;   // tuning/testing override
+            if (tune.wk16 != kUnset) cfg.wk = tune.wk16 == 8 ? 8 : 4;
             const long long ks_k = ks_units(cfg.wk);
             if (ks > ks_k) ks = ks_k;
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
             const size_t slot_bytes = (size_t)cfg.wn * 16 * kTileN * sizeof(float);
-            while (ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > kScratchBytes) ks--;
+            while (ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > scratch_bytes) ks--;
             a.ks4 = (int)ks;
             a.ks6 = (int)ks6_of(ks, cfg.wk);
             if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
@@ -498,7 +627,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.div[0] = make_div(a.groups4, wgs);
             a.div[1] = make_div(a.groups6, wgs);
             dim3 grid((unsigned)wgs, 1);
-            if (getenv("FP6M_VERBOSE"))
+            if (tune.verbose)
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u\n", a.m, prob_n,
                         prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x);
             launch_m16_any(cfg, a, g128, grid, st);
@@ -507,7 +636,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // Split k only as far as needed to give every CU a workgroup; partial tiles are 16*MB rows
             // of fp32, so the split is also capped by their traffic relative to the weight stream.
             const long long base = (long long)a.tiles * mtiles;
-            long long ks = scratch->cus / base;
+            long long ks = cus / base;
             const long long ks_k = units / (kWaves * 2) > 0 ? units / (kWaves * 2) : 1;
             const long long cap = (long long)prob_k / (16LL * rows_per_tile) > 0 ? (long long)prob_k / (16LL * rows_per_tile) : 1;
             if (ks > ks_k) ks = ks_k;
@@ -515,12 +644,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
-            while (ks > 1 && (size_t)(a.tiles + a.tiles6) * mtiles * ks * tile_bytes > kScratchBytes) ks--;   // (FP6 tiles: 2 ks)
+            while (ks > 1 && (size_t)(a.tiles + a.tiles6) * mtiles * ks * tile_bytes > scratch_bytes) ks--;   // (FP6 tiles: 2 ks)
             a.ksplit = (int)ks;
             // A grid of at most one workgroup per CU would leave every SIMD a single wave: give the workgroup eight
             // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
-            int wk = base * ks <= scratch->cus && units / 16 >= ks ? 8 : kWaves;
-            if (const char* e = getenv("FP6M_WK")) wk = atoi(e) == 8 ? 8 : kWaves;   // tuning/testing override
+            int wk = base * ks <= cus && units / 16 >= ks ? 8 : kWaves;
+            if (tune.wk != kUnset) wk = tune.wk == 8 ? 8 : kWaves;
             // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
             // FP6 tiles' workgroups set the length of the launch (8192 x 8192 at m = 128: 33 us against 29 us with INT4
             // only).  Their k range is cut twice as finely where every slice still gets two units and the grid still
@@ -528,7 +657,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // a free CU loses far more than that).  A forced split applies to both kinds.
             a.ks4 = (int)ks;
             a.ks6 = (int)ks;
-            const long long resident = (long long)scratch->cus * (wk == 8 ? 1 : 2);
+            const long long resident = (long long)cus * (wk == 8 ? 1 : 2);
             if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk &&
                 (base + (long long)a.tiles6 * mtiles) * ks <= resident)
                 a.ks6 = 2 * (int)ks;
@@ -544,13 +673,13 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.div[0] = make_div(a.ks4, wgs);
             a.div[1] = make_div(a.ks6, wgs);
             dim3 grid((unsigned)wgs, (unsigned)mtiles);
-            if (getenv("FP6M_VERBOSE"))
+            if (tune.verbose)
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks4=%d ks6=%d k slices %d grid=%ux%u\n", a.m, prob_n,
                         prob_k, mb, mtiles, a.ks4, a.ks6, wk, grid.x, grid.y);
             // From two row tiles on, the requests A costs weigh more than the shorter look-ahead of the paired fetch
             // (measured: 64 rows 1-3 % slower with it, 128 rows 0-8 % faster, 256 and 512 rows 4-14 %).
             bool pair = a.m > 64;
-            if (const char* e = getenv("FP6M_PAIR")) pair = mb == 4 && atoi(e) != 0;   // tuning/testing override
+            if (tune.pair != kUnset) pair = mb == 4 && tune.pair != 0;
             if (mb == 2) launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
             else if (pair) launch_mb<4, 3, 3, true>(a, g128, wk, grid, st);
             else launch_mb<4, 3, 3, false>(a, g128, wk, grid, st);
@@ -564,13 +693,6 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
 }  // namespace fp6m
 
 extern "C" {
-
-int fp6m_init_gather(int dev)
-{
-    fp6m::DeviceScratch* d = nullptr;
-    if (int rc = fp6m::ensure_scratch(dev, &d)) return rc;
-    return fp6m::ensure_gather_buffer(dev, d);
-}
 
 int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
              void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,

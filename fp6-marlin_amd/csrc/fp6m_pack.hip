@@ -16,10 +16,26 @@
 namespace fp6m {
 
 int hip_fail(hipError_t e);            // fp6m_gemm.hip: records the HIP error, returns FP6M_ERR_HIP
-int pack_temp(int dev, void** ptr);    // fp6m_gemm.hip: 1 MiB of per-device scratch behind the partial-sum tiles
+int pack_temp(int dev, void** ptr);    // fp6m_gemm.hip: 1 MiB of per-device scratch (allocated on first use)
 constexpr size_t kPackTemp = size_t(1) << 20;
 
 namespace {
+
+// Makes `dev` the calling thread's current device for the lifetime of the object and puts the previous one back.
+struct DeviceGuard {
+    int prev = -1;
+    hipError_t err;
+    explicit DeviceGuard(int dev)
+    {
+        err = hipGetDevice(&prev);
+        if (err == hipSuccess && prev != dev) err = hipSetDevice(dev);
+        else if (err == hipSuccess) prev = -1;                          // nothing to restore
+    }
+    ~DeviceGuard()
+    {
+        if (prev >= 0) (void)hipSetDevice(prev);
+    }
+};
 
 __device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
@@ -236,7 +252,8 @@ extern "C" int fp6m_pack_mixed_device(const void* w, int k, int n, int quant_col
     if (group_size != -1 && (group_size <= 0 || k % group_size || group_size % 16)) return FP6M_ERR_SHAPE;
     if ((size_t)qc * sizeof(unsigned) + 64 > kPackTemp) return FP6M_ERR_SHAPE;
     const int n4 = n - qc, g = group_size == -1 ? k : group_size, per_column = group_size == -1;
-    hipError_t e = hipSetDevice(dev);
+    DeviceGuard guard(dev);                                              // the caller's current device is restored on return
+    hipError_t e = guard.err;
     if (e != hipSuccess) return hip_fail(e);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint16_t* wp = static_cast<const uint16_t*>(w);

@@ -19,8 +19,8 @@ typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 constexpr int kWaves = 4;
 constexpr int kTileN = 128;          // columns per tile
 constexpr int kRedStride = kTileN + 4;                       // floats per row of the reduction slab
-constexpr size_t kScratchBytes = size_t(64) << 20;           // per-device partial-sum scratch
-constexpr size_t kPackTempBytes = size_t(1) << 20;           // + the packer's flag and per-column maxima
+constexpr size_t kScratchBytes = size_t(16) << 20;           // partial-sum scratch of one workspace
+constexpr size_t kPackTempBytes = size_t(1) << 20;           // the packer's flag and per-column maxima
 
 // Slice i of a tile's k range, in units (two k steps; four with group scales): the first `first_long` slices hold q
 // units, the others q + 1, so that inside a workgroup the longer slices come last (the lock-step kernel lets every

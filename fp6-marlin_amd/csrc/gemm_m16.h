@@ -389,7 +389,11 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
                                __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");               // my stores have completed
+    // Every wave waits until its own partial-sum stores are acknowledged (they are agent-scope write-through stores:
+    // the acknowledgement means they are visible to every other CU), and only then joins the barrier in front of
+    // the counter increment.  A workgroup-scope fence alone would not wait for them, and neither does s_barrier.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");               // (keeps the compiler from moving accesses across)
     __syncthreads();
     FP6M_MARK(p, 4);
     if (threadIdx.x == 0) {

@@ -741,7 +741,11 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     if (ks == 1) return;
 
     FP6M_MARK(p, 3);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    // Every wave waits until its own partial-sum stores are acknowledged (agent-scope write-through stores: visible to
+    // every other CU from then on) before it joins the barrier in front of the counter increment; neither a
+    // workgroup-scope fence nor s_barrier waits for outstanding stores.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");           // (keeps the compiler from moving accesses across)
     __syncthreads();
     int* counter = p.counters + ti.mtile * p.tiles + ti.tile;
     if (leader) {

@@ -21,11 +21,11 @@ try:
 except ImportError as e:  # pragma: no cover
     raise ImportError("fp6_marlin/_fp6m_torch.so is missing or does not load: build it with "
                       "`python fp6-marlin_amd/build.py`; there is no fallback implementation") from e
-from .cabi import init, workspace_elems, pack_mixed_weight_device, mul_fused, mul_rows, check_column_map, repack_gfx950, repack_gfx950_host
-from .layer import Layer, pack_mixed_weight, pack_row_mix_weight, int4_quantize, int4_pack, permute_scales, unpack_to_fp16
+from .cabi import init, init_workspace, release_workspace, workspace_elems, pack_mixed_weight_device, mul_fused, mul_rows, check_column_map, repack_gfx950, repack_gfx950_host
+from .layer import Layer, shared_workspace, pack_mixed_weight, pack_row_mix_weight, int4_quantize, int4_pack, permute_scales, unpack_to_fp16
 
-__all__ = ["prepacking", "quantize", "dequantize", "mul", "Layer", "pack_mixed_weight", "pack_mixed_weight_device", "int4_quantize",
-           "int4_pack", "permute_scales", "unpack_to_fp16", "init", "workspace_elems", "mul_fused", "mul_rows", "pack_row_mix_weight", "check_column_map", "repack_gfx950",
+__all__ = ["shared_workspace", "prepacking", "quantize", "dequantize", "mul", "Layer", "pack_mixed_weight", "pack_mixed_weight_device", "int4_quantize",
+           "int4_pack", "permute_scales", "unpack_to_fp16", "init", "init_workspace", "release_workspace", "workspace_elems", "mul_fused", "mul_rows", "pack_row_mix_weight", "check_column_map", "repack_gfx950",
            "repack_gfx950_host"]
 
 

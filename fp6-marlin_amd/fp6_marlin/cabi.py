@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfp6m.so")
 
-OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_RANGE, ERR_SHAPE, ERR_ARG, ERR_HIP, ERR_NO_GPU_CODE = range(8)
+OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_RANGE, ERR_SHAPE, ERR_ARG, ERR_HIP, ERR_NO_GPU_CODE, ERR_SCRATCH = range(9)
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
@@ -32,7 +32,12 @@ lib.fp6m_pack_mixed_device.restype = _int
 lib.fp6m_pack_mixed_device.argtypes = [_vp, _int, _int, _int, _int, _int, _vp, _vp, _vp, _int, _vp]
 lib.fp6m_workspace_elems.argtypes = [_int, _int]
 lib.fp6m_init.argtypes = [_int]
-lib.fp6m_init_gather.argtypes = [_int]
+lib.fp6m_tuning_set.argtypes = [ctypes.c_char_p, _int]
+lib.fp6m_tuning_set.restype = _int
+lib.fp6m_init_workspace.argtypes = [_int, _vp, _int]
+lib.fp6m_init_workspace.restype = _int
+lib.fp6m_release_workspace.argtypes = [_int, _vp]
+lib.fp6m_release_workspace.restype = _int
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
 lib.fp6m_mul_fused.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _vp, _vp,
                                _vp, _vp, _int]
@@ -46,9 +51,28 @@ lib.fp6m_int4_quantize.argtypes = [_vp, _sz, _sz, _int, _vp, _vp, _vp]
 lib.fp6m_int4_pack.argtypes = [_vp, _vp, _sz, _sz]
 lib.fp6m_permute_scales.argtypes = [_vp, _vp, _sz]
 lib.fp6m_unpack_to_fp16.argtypes = [_vp, _vp, _vp, _sz, _sz, _int, _int]
-for _f in (lib.fp6m_init, lib.fp6m_init_gather, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_repack_gfx950, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
+for _f in (lib.fp6m_init, lib.fp6m_mul, lib.fp6m_mul_fused, lib.fp6m_mul_rows, lib.fp6m_repack_gfx950, lib.fp6m_fp6_quantize, lib.fp6m_fp6_prepack, lib.fp6m_fp6_dequant,
            lib.fp6m_int4_quantize, lib.fp6m_int4_pack, lib.fp6m_permute_scales, lib.fp6m_unpack_to_fp16):
     _f.restype = _int
+
+
+class tuning:
+    """Context manager around fp6m_tuning_set: `with tuning(ksplit=3, wk=8): ...` overrides the dispatcher's choices
+    inside the block (tests and tuning runs only; process-wide, not thread-safe)."""
+
+    def __init__(self, **knobs):
+        self.knobs = {k: v for k, v in knobs.items() if v is not None}
+
+    def __enter__(self):
+        for name, value in self.knobs.items():
+            if lib.fp6m_tuning_set(name.encode(), int(value)) != OK:
+                lib.fp6m_tuning_set(None, 0)
+                raise ValueError(f"unknown tuning knob {name!r}")
+        return self
+
+    def __exit__(self, *exc):
+        lib.fp6m_tuning_set(None, 0)
+        return False
 
 
 def strerror(code):
@@ -185,12 +209,32 @@ def workspace_elems(n, max_par=16):
     return int(lib.fp6m_workspace_elems(n, max_par))
 
 
-def init(device=0, gather=False):
-    """Allocate the per-device scratch now (and, with `gather`, the buffer that `a_cols` gathers pass through)
-    instead of on first use: call it before HIP-graph capture or any other region that must not allocate."""
-    code = lib.fp6m_init_gather(int(device)) if gather else lib.fp6m_init(int(device))
+def init(device=0):
+    """Look up the device's properties now rather than in the first GEMM call.  Allocates nothing."""
+    code = lib.fp6m_init(int(device))
     if code != OK:
         raise RuntimeError(f"fp6m_init: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+
+
+def init_workspace(workspace, gather=False):
+    """Allocate the partial-sum region that belongs to `workspace` (a CUDA tensor) now (and, with `gather`, the
+    buffer that `a_cols` gathers pass through) instead of on its first call: do it before HIP-graph capture or any
+    other section that must not allocate.  Returns the workspace."""
+    code = lib.fp6m_init_workspace(workspace.device.index, workspace.data_ptr(), int(bool(gather)))
+    if code != OK:
+        raise RuntimeError(f"fp6m_init_workspace: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
+    return workspace
+
+
+def release_workspace(workspace=None, device=0):
+    """Wait for the device and free the region of `workspace` (call before the tensor is freed), or every region of
+    `device` when no workspace is given."""
+    if workspace is not None:
+        code = lib.fp6m_release_workspace(workspace.device.index, workspace.data_ptr())
+    else:
+        code = lib.fp6m_release_workspace(int(device), None)
+    if code != OK:
+        raise RuntimeError(f"fp6m_release_workspace: {strerror(code)} (hip error {lib.fp6m_last_hip_error()})")
 
 
 def mul(A, B, C, s, workspace, quant_cols=-1, thread_k=-1, thread_n=-1, sms=-1, max_par=16, group_size=-1):

@@ -103,6 +103,26 @@ def pack_row_mix_weight(w, quant_rows):
     return torch.cat([b4, b6]).contiguous(), torch.cat([s4, s6]).contiguous(), torch.cat([r4, r6], dim=0).contiguous()
 
 
+_workspaces = {}
+
+
+def shared_workspace(device, elems):
+    """The zeroed int32 workspace that every ``Layer.forward`` on `device`'s current stream uses: calls on one stream
+    never overlap, so they can share one workspace (and with it one partial-sum region of the library); different
+    streams get different ones, which keeps the rule "one call at a time per workspace".  It grows when a wider
+    layer turns up (the old tensor's region is released first)."""
+    device = torch.device(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < elems:
+        if ws is not None:
+            cabi.release_workspace(ws)
+        ws = torch.zeros(max(int(elems), 8192), dtype=torch.int32, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
 class Layer(nn.Module):
     """Linear layer ``y = x @ W (+ bias)`` with W [infeatures, outfeatures] stored as mixed INT4 / FP6.
 
@@ -113,7 +133,9 @@ class Layer(nn.Module):
                      ``groupsize=128``) followed by the FP6 per-column scales (permuted order)
       ``meta``       int32 [7]: format version, infeatures, outfeatures, quant_cols, groupsize, word order
                      (0 reference, 1 gfx950), quant_rows; a checkpoint whose ``meta`` differs is refused
-      ``workspace``  int32 zeros, outfeatures // 128 * 16 (not saved)
+    The GEMM's ``workspace`` (zeroed int32, outfeatures // 128 * 16 elements at least) is not a buffer of the layer:
+    ``forward`` takes ``shared_workspace``'s tensor of the current (device, stream), because the library keeps a
+    16 MiB partial-sum region per workspace address and calls that cannot overlap should share one.
 
     Which output features are kept in FP6: by default the *last* ``quant_cols`` ones (what the reference's
     harness does after moving its chosen columns to the tail, test.py:123-152).  With ``fp6_channels`` (indices
@@ -169,7 +191,6 @@ class Layer(nn.Module):
             self.register_buffer("a_cols", torch.cat([torch.nonzero(keep).reshape(-1), picked]).to(torch.int32))
         else:
             self.a_cols = None
-        self.register_buffer("workspace", torch.zeros(outfeatures // 128 * 16, dtype=torch.int32), persistent=False)
         if fp6_channels is not None:
             picked = torch.as_tensor(fp6_channels, dtype=torch.int64).reshape(-1)
             if picked.numel() != qc or picked.unique().numel() != qc or (qc and (picked.min() < 0 or picked.max() >= outfeatures)):
@@ -230,12 +251,13 @@ class Layer(nn.Module):
         x2 = x.reshape(-1, x.shape[-1]).to(torch.float16).contiguous()
         out = torch.empty((x2.shape[0], self.n), dtype=torch.float16, device=x2.device)
         res = None if residual is None else residual.reshape(-1, self.n).to(torch.float16).contiguous()
+        workspace = shared_workspace(x2.device, self.n // 128 * 16)
         if self.quant_rows:
-            cabi.mul_rows(x2, self.B, out, self.s, self.workspace, self.quant_rows, a_cols=self.a_cols, bias=self.bias,
+            cabi.mul_rows(x2, self.B, out, self.s, workspace, self.quant_rows, a_cols=self.a_cols, bias=self.bias,
                           residual=res, layout=self.layout)
         elif self.c_cols is None and self.bias is None and residual is None and self.layout == "reference":
-            cabi.mul(x2, self.B, out, self.s, self.workspace, self.quant_cols, -1, -1, -1, 16, self.groupsize)
+            cabi.mul(x2, self.B, out, self.s, workspace, self.quant_cols, -1, -1, -1, 16, self.groupsize)
         else:
-            cabi.mul_fused(x2, self.B, out, self.s, self.workspace, self.quant_cols, self.groupsize, c_cols=self.c_cols,
+            cabi.mul_fused(x2, self.B, out, self.s, workspace, self.quant_cols, self.groupsize, c_cols=self.c_cols,
                            bias=self.bias, residual=res, layout=self.layout)
         return out.reshape(x.shape[:-1] + (self.n,))

@@ -36,6 +36,7 @@ extern "C" {
 #define FP6M_ERR_ARG         5 /* null pointer, unsupported group_size / quant_cols                  */
 #define FP6M_ERR_HIP         6 /* a HIP runtime call failed; fp6m_last_hip_error() has the code      */
 #define FP6M_ERR_NO_GPU_CODE 7 /* the library was built without its gfx950 kernels                   */
+#define FP6M_ERR_SCRATCH     8 /* partial sums do not fit the scratch of an entry point that cannot grow it */
 
 /* Human-readable text for a return code (static storage). */
 const char* fp6m_strerror(int code);
@@ -95,7 +96,7 @@ int fp6m_repack_gfx950(const int32_t* in, int32_t* out, size_t k, size_t n, int 
  * any bias / residual addition to separate kernels of the caller.
  *   A, lda    device fp16 [m, lda] row-major.  Without a_cols, lda must equal prob_k.
  *   a_cols    device int32 [prob_k] or NULL: row kk of the packed weight multiplies column a_cols[kk] of A
- *             (0 <= a_cols[kk] < lda).  The gathered rows pass through a 64 MiB per-device buffer that the first
+ *             (0 <= a_cols[kk] < lda).  The gathered rows pass through a 64 MiB buffer of the call's workspace that the first
  *             such call allocates; min(prob_m, 64 * max_par) * prob_k * 2 bytes must fit (else FP6M_ERR_ARG).
  *   c_cols    device int32 [prob_n] or NULL: packed column j (INT4 columns first, then the FP6 columns) is written
  *             to column c_cols[j] of C; must be a permutation of 0 .. prob_n-1.
@@ -129,18 +130,44 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
                   void* workspace, int dev, void* stream, int sms, int max_par, int quant_rows, const int32_t* a_cols,
                   const int32_t* c_cols, const void* bias, const void* residual, int flags);
 
+/*
+ * Testing / tuning hook: overrides one of the dispatcher's per-shape choices for all later calls in this process.
+ * No counterpart in the reference (whose only such knob is the `sms` argument).  knob = "ksplit" (k parts per tile),
+ * "wk16" / "wk" (waves per workgroup of the m <= 16 / m > 16 kernel: 4 or 8), "mb" (16-row blocks per wave: 2 or 4),
+ * "wm" / "wn" (shared-fragment kernel on/off, its column tiles per workgroup), "pair" (paired activation fetch on/off),
+ * "verbose" (print every launch's configuration to stderr); knob = NULL clears all overrides.  Unknown knob ->
+ * FP6M_ERR_ARG.  Not synchronised with GEMM calls running on other threads.  The library reads no environment
+ * variables on a call (FP6M_VERBOSE is looked up once at load time).
+ */
+int fp6m_tuning_set(const char* knob, int value);
+
 /* Minimum workspace length in 4-byte elements: n / 128 * max_par (fp6_marlin/fp6_marlin_cuda.cpp:62-63). */
 size_t fp6m_workspace_elems(int prob_n, int max_par);
 
 /*
- * Device-memory scratch the GEMM keeps per GPU for cross-workgroup partial sums.  It is allocated
- * on the first fp6m_mul on a device, or eagerly here (call once per device outside any region that
- * must not allocate).  No counterpart in the reference (which reduces through C in fp16).
+ * Device memory the GEMM keeps besides its operands, and what may run concurrently.
+ *
+ * Column tiles whose k range is shared by several workgroups are summed through fp32 partial tiles in device memory
+ * (the reference sums them through C in fp16 under the locks in `workspace`, fp6_marlin_cuda_kernel.cu:645-696).
+ * That scratch belongs to the workspace: every workspace address the library has seen on a device owns a 16 MiB
+ * region (plus 64 MiB for gathered activations once a call with a_cols has used it).  The concurrency rule is
+ * therefore the reference's, one call at a time per workspace (fp6_marlin_cuda.cpp:62-63): calls with different
+ * workspaces may overlap on different streams, also when replayed from HIP graphs; two overlapping calls must not
+ * share a workspace.
+ * A region is allocated (hipMalloc + hipMemset, both synchronous) by the first call with a workspace, or ahead of
+ * time by fp6m_init_workspace -- do that before HIP-graph capture or any other section that must not allocate.
+ * Share one workspace between calls that never overlap (all layers of a model on one stream).  The library holds at
+ * most FP6M_MAX_WORKSPACES regions per device: when another is needed it waits for the device
+ * (hipDeviceSynchronize) and frees them all, which fails inside a capture.  fp6m_release_workspace frees one region
+ * (call it before the workspace is freed), or all of a device's with workspace = NULL; it waits for the device first.
+ * No counterpart in the reference.
  */
+#define FP6M_MAX_WORKSPACES 128
+/* Looks up the device's compute-unit count; optional (the first GEMM call does it too).  Allocates nothing. */
 int fp6m_init(int dev);
-/* The same for the 64 MiB buffer that gathered activations pass through (a_cols of fp6m_mul_fused / fp6m_mul_rows):
- * allocated by the first gathering call on a device, or eagerly here.  No counterpart in the reference. */
-int fp6m_init_gather(int dev);
+/* Region of `workspace`; with_gather != 0 also allocates its gathered-activation buffer. */
+int fp6m_init_workspace(int dev, const void* workspace, int with_gather);
+int fp6m_release_workspace(int dev, const void* workspace);
 
 /*
  * FP16 -> FP6 (e3m2) row quantiser.  Replaces

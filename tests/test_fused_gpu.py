@@ -183,7 +183,7 @@ def test_graph_replays_of_fused_and_row_mix_calls(oracle):
     res = torch.randn((m, n), generator=g).half().to(dev())
     ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
     outs = [torch.empty((m, n), dtype=torch.half, device=dev()) for _ in range(3)]
-    fp6_marlin.init(0, gather=True)                                     # nothing may allocate during capture
+    fp6_marlin.init_workspace(ws, gather=True)                          # nothing may allocate during capture
 
     def work():
         fp6_marlin.mul(A, B, outs[0], s, ws, qc, -1, -1, -1, 16, gs)

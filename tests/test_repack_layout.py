@@ -8,7 +8,6 @@ test.py:62-72 give the owner's (k, n) elements; the MFMA operand order is the ke
 GPU part: the GEMM on the repacked words equals the GEMM on the reference words bit for bit, for all three kernels,
 both mixes, group and column scales.
 """
-import os
 
 import numpy as np
 import pytest
@@ -80,17 +79,12 @@ def gpu_case(oracle, m, k, n, qc, gs, env=None):
     assert torch.equal(Bn.cpu(), fp6_marlin.repack_gfx950_host(B.cpu(), k, n, qc))
     A = torch.randn((m, k), generator=torch.Generator().manual_seed(m)).half().to(dev)
     ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev)
-    for name, value in (env or {}).items():
-        os.environ[name] = str(value)
-    try:
+    with fp6_marlin.cabi.tuning(**{name[5:].lower(): value for name, value in (env or {}).items()}):
         want = torch.full((m, n), float("nan"), dtype=torch.half, device=dev)
         fp6_marlin.cabi.mul(A, B, want, sd, ws, qc, -1, -1, -1, 16, gs)
         got = torch.full((m, n), float("nan"), dtype=torch.half, device=dev)
         fp6_marlin.mul_fused(A, Bn, got, sd, ws, qc, gs, layout="gfx950")
         torch.cuda.synchronize()
-    finally:
-        for name in (env or {}):
-            os.environ.pop(name, None)
     assert int(ws.abs().sum()) == 0
     assert torch.equal(got, want)
     assert oracle.rel_err(got.cpu().numpy(), oracle.matmul_ref(A.cpu().numpy(), ref)) <= 1e-3

@@ -9,7 +9,6 @@ harness's two weight generators, and what pins the result:
 * the two-launch formulation the reference would need (column-mix `mul` on the two row ranges, added in fp32)
   within the same tolerance.
 """
-import os
 
 import numpy as np
 import pytest
@@ -51,16 +50,12 @@ def run(oracle, m, k, n, qr, ksplit=None, seed=0, **kw):
     A = torch.randn((m, k), generator=torch.Generator().manual_seed(m + seed)).half()
     ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
     outs = []
-    if ksplit is not None:
-        os.environ["FP6M_KSPLIT"] = str(ksplit)
-    try:
+    with fp6_marlin.cabi.tuning(ksplit=ksplit):
         for _ in range(2):
             C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
             fp6_marlin.mul_rows(A.to(dev()), B, C, s, ws, qr, **kw)
             torch.cuda.synchronize()
             outs.append(C)
-    finally:
-        os.environ.pop("FP6M_KSPLIT", None)
     assert int(ws.abs().sum()) == 0
     assert torch.equal(outs[0], outs[1]), "two identical calls differ"
     c = outs[0].cpu().numpy()
