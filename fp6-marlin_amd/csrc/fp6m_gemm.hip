@@ -85,8 +85,15 @@ struct Region {
 constexpr size_t kGatherBytes = size_t(64) << 20;
 constexpr int kMaxDevices = 64;
 constexpr int kMaxRegions = 128;    // per device
+// Partial-tile scratch of fp6m_mul_static, the entry point for callers that must not allocate: part of the loaded
+// code object, so every GPU the library runs on holds its own copy until the process ends.  In host code the
+// array's name is only a handle; its device address is looked up once per device (device_state) and kept there.
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
 struct DeviceState {
     int cus = 0;
+    float* static_scratch = nullptr;   // device address of this GPU's copy of g_static_scratch
     int nregions = 0;
     void* pack_temp = nullptr;      // kPackTempBytes for the on-GPU packer's flag and column maxima
     Region regions[kMaxRegions];
@@ -113,15 +120,23 @@ hipError_t on_device(int dev, F&& fn)
     return e;
 }
 
-// Compute units of the device (queried once; no allocation).  Callers hold g_scratch_mutex.
+// Compute units of the device and the address of its copy of the static scratch (both looked up once, with the
+// device current; no allocation).  Callers hold g_scratch_mutex.
 int device_state(int dev, DeviceState** out)
 {
     if (dev < 0 || dev >= kMaxDevices) return FP6M_ERR_ARG;
     DeviceState& d = g_devices[dev];
     if (!d.cus) {
         int cus = 0;
-        const hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        void* sym = nullptr;
+        const hipError_t e = on_device(dev, [&] {
+            hipError_t e2 = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e2 == hipSuccess) e2 = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_static_scratch));
+            return e2;
+        });
         if (e != hipSuccess) return hip_fail(e);
+        if (!sym) return hip_fail(hipErrorInvalidSymbol);
+        d.static_scratch = static_cast<float*>(sym);
         d.cus = cus > 0 ? cus : 256;
     }
     *out = &d;
@@ -367,10 +382,13 @@ struct Fusion {
     int quant_rows = 0;              // > 0: row mix (fp6m_mul_rows), the last quant_rows rows of k are FP6
     bool native = false;             // weight planes in the gfx950 order (FP6M_LAYOUT_GFX950)
 };
+// `fixed_scratch` (fp6m_mul_static): partial tiles go to the device's static scratch instead of the workspace's
+// region, nothing is allocated, and a launch whose split needs more than the array holds is refused rather than
+// given a smaller split.
 
 int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
                void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
-               int quant_cols, int group_size, const Fusion& fu)
+               int quant_cols, int group_size, const Fusion& fu, bool fixed_scratch = false)
 {
     if (prob_m < 0 || prob_n < 0 || prob_k < 0) return FP6M_ERR_ARG;
 
@@ -412,8 +430,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     hipStream_t st = static_cast<hipStream_t>(stream);
     DeviceState* device = nullptr;
     Region* region = nullptr;
-    const size_t scratch_bytes = kScratchBytes;
-    if (int rc = workspace_region(dev, workspace, fu.a_cols != nullptr, &device, &region)) return rc;
+    size_t scratch_bytes = kScratchBytes;
+    if (fixed_scratch) {
+        if (fu.a_cols) return FP6M_ERR_ARG;                           // the gathered activations need a region's buffer
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (int rc = device_state(dev, &device)) return rc;
+        scratch_bytes = kStaticScratchBytes;
+    } else if (int rc = workspace_region(dev, workspace, fu.a_cols != nullptr, &device, &region)) {
+        return rc;
+    }
     const int cus = device->cus;
 
     GemmArgs a;
@@ -422,7 +447,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.b_fp6_4 = a.b_fp6_2 + (size_t)prob_k * qc / 16;
     a.s_int4 = static_cast<const uint16_t*>(s);
     a.s_fp6 = a.s_int4 + (g128 ? (size_t)(prob_k / 128) * n4 : (size_t)n4);
-    a.scratch = region->partials;
+    a.scratch = fixed_scratch ? device->static_scratch : region->partials;
     a.counters = static_cast<int*>(workspace);
     a.n = prob_n;
     a.k = prob_k;
@@ -521,6 +546,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
+            if (fixed_scratch && ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > scratch_bytes) return FP6M_ERR_SCRATCH;
             while (ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > scratch_bytes) ks--;
             a.ksplit = (int)ks;
             a.rule[0] = a.rule[1] = make_rule(units, a.ksplit * wk);
@@ -609,6 +635,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
             const size_t slot_bytes = (size_t)cfg.wn * 16 * kTileN * sizeof(float);
+            if (fixed_scratch && ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > scratch_bytes) return FP6M_ERR_SCRATCH;
             while (ks > 1 && (size_t)(a.groups4 + 2 * a.groups6) * ks * slot_bytes > scratch_bytes) ks--;
             a.ks4 = (int)ks;
             a.ks6 = (int)ks6_of(ks, cfg.wk);
@@ -644,6 +671,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (sms > 0 && ks > sms) ks = sms;
             if (env_ks >= 1) ks = env_ks;
             if (ks < 1) ks = 1;
+            if (fixed_scratch && ks > 1 && (size_t)(a.tiles + a.tiles6) * mtiles * ks * tile_bytes > scratch_bytes) return FP6M_ERR_SCRATCH;
             while (ks > 1 && (size_t)(a.tiles + a.tiles6) * mtiles * ks * tile_bytes > scratch_bytes) ks--;   // (FP6 tiles: 2 ks)
             a.ksplit = (int)ks;
             // A grid of at most one workgroup per CU would leave every SIMD a single wave: give the workgroup eight
@@ -700,6 +728,14 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
 {
     return fp6m::mul_common(A, B, C, s, prob_m, prob_n, prob_k, workspace, dev, stream, thread_k, thread_n, sms, max_par,
                             quant_cols, group_size, fp6m::Fusion{});
+}
+
+int fp6m_mul_static(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+                    void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
+                    int quant_cols, int group_size)
+{
+    return fp6m::mul_common(A, B, C, s, prob_m, prob_n, prob_k, workspace, dev, stream, thread_k, thread_n, sms, max_par,
+                            quant_cols, group_size, fp6m::Fusion{}, true);
 }
 
 int fp6m_mul_fused(const void* A, int lda, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,

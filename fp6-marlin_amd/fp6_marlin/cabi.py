@@ -39,6 +39,8 @@ lib.fp6m_init_workspace.restype = _int
 lib.fp6m_release_workspace.argtypes = [_int, _vp]
 lib.fp6m_release_workspace.restype = _int
 lib.fp6m_mul.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _int, _int]
+lib.fp6m_mul_static.argtypes = lib.fp6m_mul.argtypes
+lib.fp6m_mul_static.restype = _int
 lib.fp6m_mul_fused.argtypes = [_vp, _int, _vp, _vp, _vp, _int, _int, _int, _vp, _int, _vp, _int, _int, _int, _int, _vp, _vp,
                                _vp, _vp, _int]
 lib.fp6m_repack_gfx950.argtypes = [_vp, _vp, _sz, _sz, _int, _int, _int]

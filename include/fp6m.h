@@ -75,6 +75,25 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
              int quant_cols, int group_size);
 
 /*
+ * fp6m_mul for callers that cannot allocate device memory (code under HIP-graph capture, tight serving loops,
+ * harnesses that forbid it).  No counterpart in the reference.  Same arguments, results and return codes as
+ * fp6m_mul, with these differences:
+ *   - the fp32 partial tiles of split column tiles go to a 16 MiB array that is part of the library's device code
+ *     (one copy per GPU, held until the process ends) instead of the workspace's region; the call allocates and
+ *     frees nothing.  fp6m_init(dev) beforehand also keeps the one-time lookup of the device's properties and of the
+ *     array's address out of the first call;
+ *   - a launch whose k split needs more partial-tile space than the array holds returns FP6M_ERR_SCRATCH (fp6m_mul
+ *     would shrink the split instead).  The need is (workgroups that share column tiles) x (rows per workgroup pass,
+ *     16 for m <= 16, else 32 or 64) x 128 columns x 4 bytes; the splits the dispatcher picks on a 256-CU device stay
+ *     below 10 MiB for every shape, so this only triggers for splits forced with fp6m_tuning_set or on larger devices;
+ *   - every call on a GPU shares that GPU's array: calls that overlap on one GPU race, whatever their workspaces
+ *     and streams.  `workspace` keeps its role (tile counters, zero on entry and on exit).
+ */
+int fp6m_mul_static(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n, int prob_k,
+                    void* workspace, int dev, void* stream, int thread_k, int thread_n, int sms, int max_par,
+                    int quant_cols, int group_size);
+
+/*
  * The packed words in the order this GPU's kernels would choose, next to the reference's.  Same bits; what moves is
  * the 16-byte (4-bit plane, INT4 words) or 8-byte (2-bit plane) granule that one lane consumes per k-block of 16 rows:
  *   reference  [k-block][64-column group g][fragment owner t = 4 l + i]          (weight_prepacking.cpp:123-177,
