@@ -36,6 +36,7 @@
 #include "fp6m.h"
 #include "gemm_common.h"
 #include "gemm_m16.h"
+#include "gemm_sk.h"
 #include "gemm_mb.h"
 #include "gemm_wm.h"
 
@@ -64,9 +65,10 @@ thread_local int g_last_hip_error = 0;
 // Overrides of the dispatcher's choices, for tests and tuning runs (fp6m_tuning_set).  The product path reads no
 // environment variables; FP6M_VERBOSE alone is looked up once, when the library is loaded.
 constexpr int kUnset = INT32_MIN;
+const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset;
-    int verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset;
+    int verbose = g_env_verbose;
 };
 Tuning g_tuning;
 
@@ -79,7 +81,7 @@ Tuning g_tuning;
 // waits for the device and frees every region, which is safe because nothing is in flight then.
 struct Region {
     const void* workspace = nullptr;
-    float* partials = nullptr;      // kScratchBytes of partial tiles
+    float* partials = nullptr;      // kScratchBytes of partial tiles (m > 16, row mix), then kCellBytes of cells (m <= 16)
     uint16_t* gathered = nullptr;   // kGatherBytes, allocated by the first gathering call with this workspace
 };
 constexpr size_t kGatherBytes = size_t(64) << 20;
@@ -88,7 +90,8 @@ constexpr int kMaxRegions = 128;    // per device
 // Partial-tile scratch of fp6m_mul_static, the entry point for callers that must not allocate: part of the loaded
 // code object, so every GPU the library runs on holds its own copy until the process ends.  In host code the
 // array's name is only a handle; its device address is looked up once per device (device_state) and kept there.
-constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+constexpr size_t kStaticTileBytes = size_t(12) << 20;                  // partial tiles, then kCellBytes of cells
+constexpr size_t kStaticScratchBytes = kStaticTileBytes + kCellBytes;
 static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
 
 struct DeviceState {
@@ -175,8 +178,8 @@ int workspace_region(int dev, const void* workspace, bool want_gather, DeviceSta
         }
         void* mem = nullptr;
         const hipError_t e = on_device(dev, [&] {
-            hipError_t e2 = hipMalloc(&mem, kScratchBytes);
-            if (e2 == hipSuccess) e2 = hipMemset(mem, 0, kScratchBytes);
+            hipError_t e2 = hipMalloc(&mem, kScratchBytes + kCellBytes);
+            if (e2 == hipSuccess) e2 = hipMemset(mem, 0, kScratchBytes + kCellBytes);
             return e2;
         });
         if (e != hipSuccess) {
@@ -245,6 +248,21 @@ void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
         hipLaunchKernelGGL((gemm_m16_kernel<false, AROWS, WN, WK, D4, D6>), grid, dim3(64 * WN * WK), 0, stream, a);
 }
 
+// n / d as (n * magic) >> 40: exact for n < 2^24 and d < 2^16.
+inline unsigned long long magic40(long long d) { return ((1ULL << 40) + (unsigned long long)d - 1) / (unsigned long long)d; }
+
+// Share of a wave in units for a tile of `units` and a wish of at least `want`: a share shorter than a tile should
+// divide it, so that no wave crosses a tile boundary and restarts its pipeline for a few steps; if no divisor lies
+// within 1.5 x the wish the wish is taken as it is.
+inline long long pick_share(long long units, long long want)
+{
+    if (want < 1) want = 1;
+    if (want >= units) return want;
+    for (long long q = want; q < units && 2 * q <= 3 * want; q++)
+        if (units % q == 0) return q;
+    return want;
+}
+
 struct M16Config {
     int id, wn, wk;
 };
@@ -310,14 +328,13 @@ int fp6m_tuning_set(const char* knob, int value)
 {
     using fp6m::g_tuning;
     if (!knob) {                                                      // NULL: back to the dispatcher's own choices
-        const int verbose = g_tuning.verbose;
-        g_tuning = fp6m::Tuning{};
-        g_tuning.verbose = verbose;
+        g_tuning = fp6m::Tuning{};                                    // (`verbose` back to what FP6M_VERBOSE said at load time)
         return FP6M_OK;
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"verbose", &g_tuning.verbose}};
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs},
+        {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
             *k.field = value;
@@ -435,7 +452,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         if (fu.a_cols) return FP6M_ERR_ARG;                           // the gathered activations need a region's buffer
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
         if (int rc = device_state(dev, &device)) return rc;
-        scratch_bytes = kStaticScratchBytes;
+        scratch_bytes = kStaticTileBytes;
     } else if (int rc = workspace_region(dev, workspace, fu.a_cols != nullptr, &device, &region)) {
         return rc;
     }
@@ -556,8 +573,82 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: shared fragments, %d tile(s) x %d k slice(s), row tiles %d ks=%d grid=%ux%u\n",
                         a.m, prob_n, prob_k, wn, wk, mtiles, a.ksplit, grid.x, grid.y);
             fp6m::launch_wm(a, g128, wn, grid, st);
+        } else if (mb == 1 && !row_mix && a.m <= 4 && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24)) {
+            // m <= 4, weight mixed along n: one wave per workgroup, equal shares of every region's (tile, k unit)
+            // list (gemm_sk.h).
+            SkArgs sk;
+            sk.A = a.A;
+            sk.b_int4 = a.b_int4;
+            sk.b_fp6_2 = a.b_fp6_2;
+            sk.b_fp6_4 = a.b_fp6_4;
+            sk.s_int4 = a.s_int4;
+            sk.s_fp6 = a.s_fp6;
+            sk.C = a.C;
+            sk.cells = reinterpret_cast<unsigned long long*>(reinterpret_cast<unsigned char*>(a.scratch) + scratch_bytes);
+            sk.m = a.m;
+            sk.n = a.n;
+            sk.k = a.k;
+            sk.n4 = a.n4;
+            sk.qc = a.qc;
+            sk.tiles6 = a.tiles6;
+            sk.native = a.native;
+            sk.fused = a.fused;
+            sk.c_cols = a.c_cols;
+            sk.bias = a.bias;
+            sk.residual = a.residual;
+            sk.timeline = nullptr;
+#ifdef FP6M_TIMELINE
+            sk.timeline = a.timeline;
+#endif
+            const long long tiles4 = a.tiles - a.tiles6;
+            const long long u4 = units, u6 = prob_k / 64;              // FP6 tiles have no group scales: 64-row units
+            // Waves: eight per CU keep enough loads in flight; a wave gets at least one unit.  `want` is the INT4
+            // share that gives about that many waves; an FP6 unit of 64 rows is 6 KiB against 8 (4) KiB of an
+            // INT4 unit with (without) group scales and costs more per byte, so the FP6 share counts the same
+            // (half as many) units.
+            const long long bytes4 = tiles4 * u4 * (g128 ? 8 : 4), bytes6 = (long long)a.tiles6 * u6 * 6;   // KiB
+            long long waves_wanted = 8LL * cus;
+            if (tune.wgs != kUnset && tune.wgs > 0) waves_wanted = tune.wgs;
+            long long want4 = ((bytes4 + bytes6) / (g128 ? 8 : 4) + waves_wanted - 1) / waves_wanted;
+            // Bounds: at most kMaxParts waves on one tile; `sms` caps the waves that share a tile (1: whole tiles
+            // only), a forced split cuts every tile into that many parts; and without room for the cells of every
+            // tile nothing is shared.
+            const bool cells_fit = (size_t)prob_n * a.m * sizeof(unsigned long long) <= kCellBytes;
+            auto share = [&](long long units_r, long long want) {
+                long long q = pick_share(units_r, want);
+                if (env_ks >= 1) q = units_r / (env_ks < units_r ? env_ks : units_r);   // (may not divide: shares then cross tiles)
+                if (q * kMaxParts < units_r) q = pick_share(units_r, (units_r + kMaxParts - 1) / kMaxParts);
+                if (sms > 1 && q * sms < units_r) q = pick_share(units_r, (units_r + sms - 1) / sms);
+                if ((sms == 1 || !cells_fit) && q < units_r) q = units_r;
+                return q;
+            };
+            const long long q4 = share(u4, want4), q6 = share(u6, g128 ? want4 : (want4 + 1) / 2);
+            const long long n4u = tiles4 * u4, n6u = (long long)a.tiles6 * u6;
+            const long long w4 = tiles4 ? (n4u + q4 - 1) / q4 : 0, w6 = a.tiles6 ? (n6u + q6 - 1) / q6 : 0;
+            sk.waves = (int)(w4 + w6);
+            sk.waves6 = (int)w6;
+            sk.units4 = (int)u4;
+            sk.units6 = (int)u6;
+            sk.q4 = w4 ? (int)(n4u / w4) : 1;
+            sk.r4 = w4 ? (int)(n4u % w4) : 0;
+            sk.q6 = w6 ? (int)(n6u / w6) : 1;
+            sk.r6 = w6 ? (int)(n6u % w6) : 0;
+            sk.magic_u4 = magic40(u4);
+            sk.magic_u6 = magic40(u6);
+            sk.magic_q4 = magic40(sk.q4);
+            sk.magic_q4p = magic40(sk.q4 + 1);
+            sk.magic_q6 = magic40(sk.q6);
+            sk.magic_q6p = magic40(sk.q6 + 1);
+            if (tune.verbose)
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: one-wave workgroups %lld (FP6) + %lld (INT4), units per tile %lld / %lld, "
+                        "units per wave %d / %d\n", a.m, prob_n, prob_k, w6, w4, u6, u4, sk.q6, sk.q4);
+            dim3 grid((unsigned)sk.waves, 1);
+            if (g128)
+                hipLaunchKernelGGL((gemm_sk_kernel<true>), grid, dim3(64), 0, st, sk);
+            else
+                hipLaunchKernelGGL((gemm_sk_kernel<false>), grid, dim3(64), 0, st, sk);
         } else if (mb == 1) {
-            // m <= 16.  Each region (FP6, INT4) has its own number of k parts (workgroups) per tile group;
+            // m <= 16 (the row mix, and 5 to 16 rows of the column mix).  Each region (FP6, INT4) has its own number of k parts (workgroups) per tile group;
             // FP6 steps cost about twice an INT4 step, so the FP6 region is split twice as finely.  The
             // split is bounded so that every wave keeps at least one k unit, partial-sum traffic stays
             // well below the weight stream and the partial tiles fit the scratch.

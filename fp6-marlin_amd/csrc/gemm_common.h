@@ -125,7 +125,6 @@ __device__ __forceinline__ void preload_args(const GemmArgs& p)
     asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
                         "s"(p.div[0].d), "s"(p.div[0].magic), "s"(p.div[1].d), "s"(p.div[1].magic), "s"(p.fused));
 }
-
 // Epilogue of fp6m_mul_fused for the two adjacent packed columns a lane owns: C[row, c_cols[col]] =
 // fp16(v + bias[c_cols[col]] + residual[row, c_cols[col]]), everything added in fp32 and rounded once.
 // The lane's destination columns and bias are looked up once (FusedCols), the rows then only add and store.
@@ -134,7 +133,8 @@ struct FusedCols {
     int c0, c1;
     float b0, b1;
 };
-__device__ __forceinline__ FusedCols fused_cols(const GemmArgs& p, int col)
+template <typename Args>
+__device__ __forceinline__ FusedCols fused_cols(const Args& p, int col)
 {
     FusedCols f;
     f.c0 = col;
@@ -153,7 +153,8 @@ __device__ __forceinline__ FusedCols fused_cols(const GemmArgs& p, int col)
     }
     return f;
 }
-__device__ __forceinline__ void store_fused(const GemmArgs& p, const FusedCols& f, size_t row, float v0, float v1)
+template <typename Args>
+__device__ __forceinline__ void store_fused(const Args& p, const FusedCols& f, size_t row, float v0, float v1)
 {
     v0 += f.b0;
     v1 += f.b1;
@@ -164,6 +165,17 @@ __device__ __forceinline__ void store_fused(const GemmArgs& p, const FusedCols& 
     }
     p.C[r + f.c0] = __builtin_bit_cast(uint16_t, (_Float16)v0);
     p.C[r + f.c1] = __builtin_bit_cast(uint16_t, (_Float16)v1);
+}
+
+// One of the two: element e (0 / 1) of the lane's column pair.
+template <typename Args>
+__device__ __forceinline__ void store_fused_one(const Args& p, const FusedCols& f, size_t row, int e, float v)
+{
+    const int col = e ? f.c1 : f.c0;
+    v += e ? f.b1 : f.b0;
+    const size_t at = row * (size_t)p.n + col;
+    if (p.residual) v += (float)__builtin_bit_cast(_Float16, p.residual[at]);
+    p.C[at] = __builtin_bit_cast(uint16_t, (_Float16)v);
 }
 
 // ------------------------------------------------------------------------------------------------ tile bookkeeping
@@ -199,7 +211,8 @@ struct PlaneGeometry {
     size_t row4, row2;       // bytes from one k-block of the tile to the next
     size_t tile4, tile2;     // byte offset of the tile's first k-block
 };
-__device__ __forceinline__ PlaneGeometry plane_geometry(const GemmArgs& p, const TileInfo& ti)
+template <typename Args>
+__device__ __forceinline__ PlaneGeometry plane_geometry(const Args& p, const TileInfo& ti)
 {
     PlaneGeometry g;
     if (p.native) {

@@ -40,8 +40,8 @@ struct StepRegs {
 };
 
 // AROWS = rows of A the ring holds (4 or 16).
-template <bool FP6, bool G128, int DEPTH, int AROWS>
-__device__ __forceinline__ void stream_tile(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
+template <bool FP6, bool G128, int DEPTH, int AROWS, typename Args>
+__device__ __forceinline__ void stream_tile(const Args& p, const TileInfo& ti, unsigned char* ring,
                                             int step_begin, int step_end, f4 (&acc)[1][8])
 {
     static_assert(DEPTH >= 3, "needs two steps of look-ahead");

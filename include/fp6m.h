@@ -78,14 +78,16 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
  * fp6m_mul for callers that cannot allocate device memory (code under HIP-graph capture, tight serving loops,
  * harnesses that forbid it).  No counterpart in the reference.  Same arguments, results and return codes as
  * fp6m_mul, with these differences:
- *   - the fp32 partial tiles of split column tiles go to a 16 MiB array that is part of the library's device code
- *     (one copy per GPU, held until the process ends) instead of the workspace's region; the call allocates and
- *     frees nothing.  fp6m_init(dev) beforehand also keeps the one-time lookup of the device's properties and of the
+ *   - what column tiles shared by several workgroups are summed through (fp32 partial tiles for m > 16, 64-bit
+ *     accumulate-and-count cells for m <= 16) lives in a 20 MiB array that is part of the library's device code (one
+ *     copy per GPU, held until the process ends) instead of the workspace's region; the call allocates and frees
+ *     nothing.  fp6m_init(dev) beforehand also keeps the one-time lookup of the device's properties and of the
  *     array's address out of the first call;
- *   - a launch whose k split needs more partial-tile space than the array holds returns FP6M_ERR_SCRATCH (fp6m_mul
- *     would shrink the split instead).  The need is (workgroups that share column tiles) x (rows per workgroup pass,
- *     16 for m <= 16, else 32 or 64) x 128 columns x 4 bytes; the splits the dispatcher picks on a 256-CU device stay
- *     below 10 MiB for every shape, so this only triggers for splits forced with fp6m_tuning_set or on larger devices;
+ *   - a launch of more than 16 rows whose k split needs more than the 12 MiB the array has for partial tiles returns
+ *     FP6M_ERR_SCRATCH (fp6m_mul would shrink the split instead).  The need is (workgroups that share column tiles) x
+ *     (32 or 64 rows) x 128 columns x 4 bytes; the splits the dispatcher picks on a 256-CU device stay below 10 MiB
+ *     for every shape, so this only triggers for splits forced with fp6m_tuning_set or on larger devices.  Launches
+ *     of up to 16 rows never fail this way: without room for their cells (n * m * 8 bytes > 8 MiB) no tile is shared;
  *   - every call on a GPU shares that GPU's array: calls that overlap on one GPU race, whatever their workspaces
  *     and streams.  `workspace` keeps its role (tile counters, zero on entry and on exit).
  */
@@ -168,7 +170,7 @@ size_t fp6m_workspace_elems(int prob_n, int max_par);
  *
  * Column tiles whose k range is shared by several workgroups are summed through fp32 partial tiles in device memory
  * (the reference sums them through C in fp16 under the locks in `workspace`, fp6_marlin_cuda_kernel.cu:645-696).
- * That scratch belongs to the workspace: every workspace address the library has seen on a device owns a 16 MiB
+ * That scratch belongs to the workspace: every workspace address the library has seen on a device owns a 24 MiB
  * region (plus 64 MiB for gathered activations once a call with a_cols has used it).  The concurrency rule is
  * therefore the reference's, one call at a time per workspace (fp6_marlin_cuda.cpp:62-63): calls with different
  * workspaces may overlap on different streams, also when replayed from HIP graphs; two overlapping calls must not

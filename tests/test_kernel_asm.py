@@ -33,6 +33,8 @@ def asm(tmp_path_factory):
 
 def kernels(asm):
     for m in re.finditer(r"^(_ZN4fp6m\w+):", asm, re.M):
+        if f".type\t{m.group(1)},@function" not in asm:                 # a data symbol (the static scratch array)
+            continue
         body = asm[m.start():asm.index(".Lfunc_end", m.start())]
         ins = [l.strip() for l in body.split("\n") if l.startswith("\t") and l.strip() and not l.strip().startswith((".", ";"))]
         yield m.group(1), ins
@@ -70,9 +72,9 @@ def test_no_valu_write_right_before_mfma_read(asm):
 
 
 def test_scalar_operands_of_asm_loads(asm):
-    assert not re.findall(r"global_load_lds_dwordx?4? v\d+, v", asm), "direct-to-LDS load with a vector base"
-    assert not re.findall(r"s_mov_b32 m0, v", asm), "M0 written from a VGPR"
-    assert not re.findall(r"global_load_dwordx2 v\[\d+:\d+\], v\d+, v", asm), "2-bit plane load with a vector base"
+    assert not re.findall(r"global_load_lds_dwordx?4? v\d+, v[\[\d]", asm), "direct-to-LDS load with a vector base"
+    assert not re.findall(r"s_mov_b32 m0, v\d", asm), "M0 written from a VGPR"
+    assert not re.findall(r"global_load_dwordx2 v\[\d+:\d+\], v\d+, v[\[\d]", asm), "2-bit plane load with a vector base"
     assert len(re.findall(r"global_load_lds_dwordx4 v\d+, s\[", asm)) > 20
 
 
@@ -98,15 +100,20 @@ def test_mfma_loops_keep_accumulators_in_place(asm):
 def test_kernel_arguments_are_loaded_in_one_batch(asm):
     """Scalar loads of kernel arguments between the top of a GEMM kernel and its first MFMA would each add a dependent
     round trip before the first weight load (measured: 0.4 us per launch when the slice tables were read by computed
-    index).  All of them must sit in the first few instructions, behind a single wait."""
+    index).  All of them must sit in the first few instructions, behind a single wait.  The decode kernel fetches its
+    argument block itself: four loads, one wait, and no other argument load anywhere."""
     seen = 0
     for name, ins in kernels(asm):
-        if "gemm_m16_kernel" not in name and "gemm_mb_kernel" not in name and "gemm_wm_kernel" not in name:
+        if not any(k in name for k in ("gemm_m16_kernel", "gemm_sk_kernel", "gemm_mb_kernel", "gemm_wm_kernel")):
             continue
         seen += 1
+        if "gemm_sk_kernel" in name:
+            loads = [n for n, l in enumerate(ins) if l.startswith("s_load") and "s[0:1]" in l]
+            assert loads == [0, 1, 2, 3] and ins[4].startswith("s_waitcnt lgkmcnt(0)"), f"{name}: {ins[:6]}"
+            continue
         first_mfma = next(n for n, l in enumerate(ins) if l.startswith("v_mfma"))
         late = [(n, l) for n, l in enumerate(ins[:first_mfma]) if l.startswith("s_load") and n > 16]
         # the code of the epilogue may be laid out ahead of the loops: its loads (fused-epilogue pointers) do not count
         late = [(n, l) for n, l in late if not re.search(r"0x(a8|b0|b8)$", l)]
         assert not late, f"{name}: kernel-argument loads after the prologue: {late[:4]}"
-    assert seen == 24
+    assert seen == 26

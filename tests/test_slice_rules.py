@@ -56,3 +56,52 @@ def test_multiply_high_quotient_is_exact():
         alln = np.arange(65536, dtype=np.uint64)
         magic = np.uint64((2 ** 32 + d - 1) // d)
         assert np.array_equal((alln * magic) >> np.uint64(32), alln // np.uint64(d)), d
+
+
+# ---------------------------------------------------------------- equal shares of the m <= 16 kernel (gemm_sk.h)
+
+def share(j, q, r):
+    """Units of workgroup j: the first r workgroups hold q + 1."""
+    begin = j * q + min(j, r)
+    return begin, begin + q + (1 if j < r else 0)
+
+
+def owner(x, q, r):
+    head = r * (q + 1)
+    return x // (q + 1) if x < head else r + (x - head) // q
+
+
+def test_equal_shares_cover_every_unit_once_and_owner_inverts_them():
+    rng = np.random.default_rng(0)
+    cases = [(30, 32, 256), (446, 64, 512), (2, 32, 6), (94, 32, 500), (446, 224, 384), (1, 5, 3), (7, 1, 7), (3, 9, 2)]
+    cases += [(int(rng.integers(1, 60)), int(rng.integers(1, 40)), 0) for _ in range(200)]
+    for tiles, units, wgs in cases:
+        total = tiles * units
+        if wgs == 0:
+            wgs = int(rng.integers(1, total + 1))
+        wgs = min(wgs, total)
+        q, r = divmod(total, wgs)
+        covered = np.zeros(total, dtype=np.int32)
+        touching = np.zeros(tiles, dtype=np.int32)
+        for j in range(wgs):
+            b, e = share(j, q, r)
+            assert e - b in (q, q + 1) and e > b
+            covered[b:e] += 1
+            assert all(owner(x, q, r) == j for x in (b, e - 1))
+            for t in range(b // units, (e - 1) // units + 1):        # the segments the kernel walks
+                touching[t] += 1
+        assert (covered == 1).all()
+        for t in range(tiles):                                      # what the kernel takes as a tile's number of parts
+            parts = owner((t + 1) * units - 1, q, r) - owner(t * units, q, r) + 1
+            assert parts == touching[t], (tiles, units, wgs, t)
+
+
+def test_forty_bit_reciprocal_division_is_exact_in_its_range():
+    rng = np.random.default_rng(1)
+    ds = np.unique(np.concatenate([np.arange(1, 300), rng.integers(1, 65536, 2000), [65535]])).astype(np.uint64)
+    ns = np.unique(np.concatenate([np.arange(0, 2000), rng.integers(0, 1 << 24, 4000), [(1 << 24) - 1]])).astype(np.uint64)
+    for d in ds.tolist():
+        magic = ((1 << 40) + d - 1) // d
+        assert magic < (1 << 41)
+        got = (ns * np.uint64(magic)) >> np.uint64(40)              # n < 2^24, magic < 2^41: no overflow of 64 bits
+        assert (got == ns // np.uint64(d)).all(), d

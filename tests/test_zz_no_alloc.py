@@ -48,11 +48,11 @@ def test_static_scratch_entry_matches_mul_on_consecutive_calls():
 def test_static_scratch_entry_refuses_what_does_not_fit():
     from fp6_marlin import cabi
     L = cabi.lib
-    m, k, n, qc, gs = 16, 4096, 57344, 256, 128
+    m, k, n, qc, gs = 64, 8192, 8192, 256, 128
     A, B, s = operands(m, k, n, qc, gs, 60)
     ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device="cuda")
     C = torch.zeros((m, n), dtype=torch.half, device="cuda")
-    with cabi.tuning(ksplit=8):                                          # 450 tiles x 8 parts x 8 KiB > 16 MiB
+    with cabi.tuning(ksplit=8):                                          # 66 tile slots x 8 parts x 32 KiB > 12 MiB
         assert call(L.fp6m_mul_static, A, B, C, s, ws, m, n, k, qc, gs) == cabi.ERR_SCRATCH
         assert call(L.fp6m_mul, A, B, C, s, ws, m, n, k, qc, gs) == cabi.OK      # the region-backed entry shrinks the split
     assert "use fp6m_mul" in cabi.strerror(cabi.ERR_SCRATCH)
