@@ -67,7 +67,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, exact = kUnset, share = kUnset, sk = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -251,13 +251,13 @@ void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 // n / d as (n * magic) >> 40: exact for n < 2^24 and d < 2^16.
 inline unsigned long long magic40(long long d) { return ((1ULL << 40) + (unsigned long long)d - 1) / (unsigned long long)d; }
 
-// Share of a wave in units for a tile of `units` and a wish of at least `want`: a share shorter than a tile should
-// divide it, so that no wave crosses a tile boundary and restarts its pipeline for a few steps; if no divisor lies
-// within 1.5 x the wish the wish is taken as it is.
+// Share of a wave in units for a tile of `units` and a wish of at least `want`.  A short share should divide the tile,
+// so that no wave crosses a tile boundary for a few steps (taken if a divisor lies within 1.5 x the wish); for long
+// shares the boundary costs nothing worth a longer share (the next tile's words are fetched ahead).
 inline long long pick_share(long long units, long long want)
 {
     if (want < 1) want = 1;
-    if (want >= units) return want;
+    if (want >= units || want >= 8) return want;
     for (long long q = want; q < units && 2 * q <= 3 * want; q++)
         if (units % q == 0) return q;
     return want;
@@ -333,7 +333,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"exact", &g_tuning.exact}, {"share", &g_tuning.share}, {"sk", &g_tuning.sk},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -573,9 +573,13 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: shared fragments, %d tile(s) x %d k slice(s), row tiles %d ks=%d grid=%ux%u\n",
                         a.m, prob_n, prob_k, wn, wk, mtiles, a.ksplit, grid.x, grid.y);
             fp6m::launch_wm(a, g128, wn, grid, st);
-        } else if (mb == 1 && !row_mix && a.m <= 4 && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24)) {
-            // m <= 4, weight mixed along n: one wave per workgroup, equal shares of every region's (tile, k unit)
-            // list (gemm_sk.h).
+        } else if (mb == 1 && !row_mix && (tune.sk != kUnset ? tune.sk != 0 && a.m <= 4 : a.m == 1) && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24) &&
+                   (long long)prob_k * prob_n / 2 < (1LL << 32)) {
+            // One row (decode), weight mixed along n: one wave per workgroup, equal shares of every region's (tile,
+            // k unit) list (gemm_sk.h).  The kernel takes up to four rows, but every wave adds its part of a shared
+            // tile with one atomic per element, and from two rows on that traffic costs more than the barriers and
+            // the partial-tile round trips of the workgroup kernel below (measured: 4096 x 4096 6.5 us at one row,
+            // 8.2 at two, 12.8 at four, against 8.2 - 8.3 there).
             SkArgs sk;
             sk.A = a.A;
             sk.b_int4 = a.b_int4;
@@ -602,14 +606,19 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
 #endif
             const long long tiles4 = a.tiles - a.tiles6;
             const long long u4 = units, u6 = prob_k / 64;              // FP6 tiles have no group scales: 64-row units
-            // Waves: eight per CU keep enough loads in flight; a wave gets at least one unit.  `want` is the INT4
-            // share that gives about that many waves; an FP6 unit of 64 rows is 6 KiB against 8 (4) KiB of an
-            // INT4 unit with (without) group scales and costs more per byte, so the FP6 share counts the same
-            // (half as many) units.
-            const long long bytes4 = tiles4 * u4 * (g128 ? 8 : 4), bytes6 = (long long)a.tiles6 * u6 * 6;   // KiB
-            long long waves_wanted = 8LL * cus;
+            // Waves (measured on MI355X over 17 shapes): shorter shares are faster as long as all waves are resident at
+            // once (twelve per CU by registers) and a tile is not cut into more than about 32 parts (every part is
+            // one atomic per output element); beyond either bound times rise steeply.  So: the shortest share that
+            // keeps the waves below eleven per CU and the parts of a tile at 32.  An FP6 unit (64 rows, 6 KiB)
+            // counts like an INT4 unit (8 KiB with group scales, 4 KiB without): fewer bytes, more work per byte.
+            long long waves_wanted = 11LL * cus;
             if (tune.wgs != kUnset && tune.wgs > 0) waves_wanted = tune.wgs;
+            const long long bytes4 = tiles4 * u4 * (g128 ? 8 : 4), bytes6 = (long long)a.tiles6 * u6 * 6;   // KiB
             long long want4 = ((bytes4 + bytes6) / (g128 ? 8 : 4) + waves_wanted - 1) / waves_wanted;
+            if (want4 < (u4 + 31) / 32) want4 = (u4 + 31) / 32;
+            long long want6 = g128 ? want4 : (want4 + 1) / 2;
+            if (want6 < (u6 + 31) / 32) want6 = (u6 + 31) / 32;
+            if (tune.share != kUnset && tune.share > 0) want4 = want6 = tune.share;
             // Bounds: at most kMaxParts waves on one tile; `sms` caps the waves that share a tile (1: whole tiles
             // only), a forced split cuts every tile into that many parts; and without room for the cells of every
             // tile nothing is shared.
@@ -622,9 +631,20 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if ((sms == 1 || !cells_fit) && q < units_r) q = units_r;
                 return q;
             };
-            const long long q4 = share(u4, want4), q6 = share(u6, g128 ? want4 : (want4 + 1) / 2);
+            const long long q4 = share(u4, want4), q6 = share(u6, want6);
             const long long n4u = tiles4 * u4, n6u = (long long)a.tiles6 * u6;
-            const long long w4 = tiles4 ? (n4u + q4 - 1) / q4 : 0, w6 = a.tiles6 ? (n6u + q6 - 1) / q6 : 0;
+            long long w4 = tiles4 ? (n4u + q4 - 1) / q4 : 0, w6 = a.tiles6 ? (n6u + q6 - 1) / q6 : 0;
+            if (tune.exact != kUnset && tune.exact > 0 && sms <= 0 && env_ks < 1 && cells_fit) {
+                // exactly `waves_wanted` waves, dealt to the regions by bytes; shares as they come
+                w6 = a.tiles6 ? (waves_wanted * bytes6 * 3 / 2 + (bytes4 + bytes6 * 3 / 2) / 2) / (bytes4 + bytes6 * 3 / 2) : 0;
+                if (a.tiles6 && w6 < 1) w6 = 1;
+                if (w6 > n6u) w6 = n6u;
+                w4 = tiles4 ? waves_wanted - w6 : 0;
+                if (tiles4 && w4 < 1) w4 = 1;
+                if (w4 > n4u) w4 = n4u;
+                if (w4 && n4u / w4 * kMaxParts < u4) w4 = n4u / ((u4 + kMaxParts - 1) / kMaxParts);
+                if (w6 && n6u / w6 * kMaxParts < u6) w6 = n6u / ((u6 + kMaxParts - 1) / kMaxParts);
+            }
             sk.waves = (int)(w4 + w6);
             sk.waves6 = (int)w6;
             sk.units4 = (int)u4;

@@ -281,6 +281,19 @@ __device__ __forceinline__ void dma4(const void* gsrc, unsigned char* lds_dst)
 {
     __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 4, 0, 0);
 }
+// (the same with the destination already an LDS-space pointer)
+__device__ __forceinline__ void dma16(const void* gsrc, FP6M_AS3 unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 0);
+}
+__device__ __forceinline__ void dma16_stream(const void* gsrc, FP6M_AS3 unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 16, 0, 2);
+}
+__device__ __forceinline__ void dma4(const void* gsrc, FP6M_AS3 unsigned char* lds_dst)
+{
+    __builtin_amdgcn_global_load_lds((const FP6M_AS1 void*)gsrc, (FP6M_AS3 void*)lds_dst, 4, 0, 0);
+}
 __device__ __forceinline__ uint32_t lds_addr(const void* ptr) { return (uint32_t)(uintptr_t)(const FP6M_AS3 void*)ptr; }
 
 // Direct-to-LDS loads in their scalar-base form: global address = sbase + voff + OFF, LDS address =

@@ -125,128 +125,385 @@ __device__ __forceinline__ int sk_owner(uint32_t x, int q, int r, unsigned long 
     return x < head ? (int)mul_shift40(magic_qp, x) : r + (int)mul_shift40(magic_q, x - head);
 }
 
-// End of a segment.  `parts` = waves that share the tile (1: this segment is the whole tile); s0, s1 = the scales
-// of the lane's two columns (1 where group scales were applied in the loop).
-__device__ __forceinline__ void wave_finish_sk(const SkArgs& p, const TileInfo& ti, int parts, f4 (&acc)[1][8], float s0,
-                                               float s1, unsigned char* ring)
+// A shared tile's elements this wave has added to and not yet looked at: the atomics' results come back while the
+// wave is already streaming its next segment.
+struct PendingCells {
+    unsigned long long* cell;      // this lane's cell of row 0 (even column; the odd one 64 cells on)
+    unsigned long long old[4][2];
+    float v[4][2];
+    int parts;                     // 0: nothing pending
+    int col0;                      // the tile's first column in C
+};
+
+// The wave's whole share in one software pipeline.  This is stream_tile (gemm_m16.h) for at most four rows of A with
+// two changes.  The fetch side walks the share's steps across tile boundaries by itself (at a tile's last step the
+// pointers move to the next tile's first), so when the multiply side finishes a segment the words of the next one
+// are already in the ring or on their way: a wave pays the latency of a first load once, not once per segment.  And
+// because the ring is never drained in between, a segment's accumulators are turned into rows in a small slab of
+// their own behind the ring.
+template <bool FP6, bool G128>
+__device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigned char* ring)
 {
+    constexpr int DEPTH = FP6 ? 3 : 4;
+    constexpr int AROWS = 4;
+    constexpr bool kGroup = G128 && !FP6;                 // group scales apply to INT4 tiles only
+    constexpr bool kColumnScale = FP6 || !G128;
+    constexpr int unit_steps = kGroup ? 4 : 2;
+    constexpr int kPairSlots = pair_slots(DEPTH);         // step pairs of A alive at once
+    constexpr int kPair = pair_bytes(AROWS);
+    constexpr int kSlot = FP6 ? 3072 : 2048;              // a step's packed words
+    constexpr int kWordOps = FP6 ? 3 : 2;                 // direct-to-LDS loads of the packed words per step
+    constexpr int kAOps = 1;                              // ... and of A per pair of steps
+    constexpr int kReads = FP6 ? 8 : 6;                   // LDS reads per step
+    constexpr int kUnroll = kGroup ? 4 : 2;               // steps per loop trip (segments are multiples of it)
     typedef float f2 __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x;
-    const int c = lane & 15, q = lane >> 4;
-    const int nrows = p.m;                                               // <= 4
-    // MFMA fragments -> fp32 rows in the drained ring (lane c holds row c of the tile's 16), read back with lane L
-    // owning columns 2L, 2L+1.  LDS operations of one wave execute in order: no barrier is needed.
-    float* slab = reinterpret_cast<float*>(ring);
-    if (c < nrows) {
-        float* mine = slab + c * kRedStride + 64 * (q >> 1) + 4 * (q & 1);
-#pragma unroll
-        for (int t = 0; t < 8; t++) *reinterpret_cast<f4*>(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[0][t];
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    float v0[4], v1[4];
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const f2 t = *reinterpret_cast<const f2*>(slab + (r < nrows ? r : 0) * kRedStride + 2 * lane);
-        v0[r] = t[0] * s0;
-        v1[r] = t[1] * s1;
-    }
-    FP6M_MARK(p, 3);
+    const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
+    const int nrows = p.m;                                // <= 4
 
-    uint16_t* c_out = p.C + ti.col0 + 2 * lane;
-    const FusedCols fcols = fused_cols(p, ti.col0 + 2 * lane);
-    if (parts == 1) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            if (r >= nrows) continue;
-            if (p.fused) {
-                store_fused(p, fcols, (size_t)r, v0[r], v1[r]);
-            } else {
-                const h2 o = {(_Float16)v0[r], (_Float16)v1[r]};
-                *reinterpret_cast<h2*>(c_out + (size_t)r * p.n) = o;
-            }
-        }
-        return;
-    }
+    DequantConsts kc;
+    kc.lo = vgpr_const(0x000f000fu);
+    kc.hi = vgpr_const(0x00f000f0u);
+    kc.ex = vgpr_const(0x64006400u);
+    kc.top2 = vgpr_const(0xc0c0c0c0u);
+    kc.exp_man = vgpr_const(0x9f009f00u);
 
-    // Shared tile: one returning atomic per element (cells of a row: 64 of the even columns, then 64 of the odd).
-    unsigned long long* cell = p.cells + (size_t)ti.tile * nrows * kTileN + lane;
-    unsigned long long add[4][2], old[4][2];
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        add[r][0] = cell_contribution(v0[r]);
-        add[r][1] = cell_contribution(v1[r]);
-        if (r < nrows) {
-            old[r][0] = __hip_atomic_fetch_add(cell + r * kTileN, add[r][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            old[r][1] = __hip_atomic_fetch_add(cell + r * kTileN + 64, add[r][1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    FP6M_MARK(p, 4);
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        if (r >= nrows) continue;
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            if ((int)(old[r][e] >> 56) != parts - 1) continue;           // somebody else arrives last at this element
-            const float v = cell_total(old[r][e], add[r][e], parts);
-            __hip_atomic_store(cell + r * kTileN + 64 * e, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (p.fused) {
-                store_fused_one(p, fcols, (size_t)r, e, v);
-            } else {
-                c_out[(size_t)r * p.n + e] = __builtin_bit_cast(uint16_t, (_Float16)v);
-            }
-        }
-    }
-    FP6M_MARK(p, 6);
-}
-
-template <bool FP6, bool G128>
-__device__ __forceinline__ void sk_wave(const SkArgs& p, int j, unsigned char* ring)
-{
-    constexpr int unit_steps = G128 && !FP6 ? 4 : 2;
-    constexpr int DEPTH = FP6 ? 3 : 4;
-    constexpr bool kColumnScale = FP6 || !G128;
+    // ---- the share
     const int q = FP6 ? p.q6 : p.q4, r = FP6 ? p.r6 : p.r4;
     const int units = FP6 ? p.units6 : p.units4;
+    const int tile_steps = units * unit_steps;
     uint32_t u = (uint32_t)j * (uint32_t)q + (uint32_t)(j < r ? j : r);
     const uint32_t u_end = u + (uint32_t)q + (j < r ? 1u : 0u);
-    TileInfo ti;
-    ti.fp6 = FP6;
-    ti.mtile = 0;
-    ti.part = 0;
-    ti.a_step0 = 0;
-    ti.region_n = FP6 ? p.qc : p.n4;
-    ti.tcol = (int)mul_shift40(FP6 ? p.magic_u6 : p.magic_u4, u);
+    int tcol = (int)mul_shift40(FP6 ? p.magic_u6 : p.magic_u4, u);
+    const int region_n = FP6 ? p.qc : p.n4;
+
+    // ---- fetch side (lane = position in the slot).  Uniform 64-bit bases advance on the scalar unit; each lane
+    // only contributes a constant 32-bit offset.
+    const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
+    const size_t kblocks = (size_t)p.k / 16;
+    const size_t row4 = p.native ? 1024 : (size_t)region_n * 8, row2 = row4 / 2;
+    const size_t tile_stride4 = p.native ? kblocks * 1024 : 1024, tile_stride2 = tile_stride4 / 2;
+    const unsigned char* plane4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4);
+    const unsigned char* plane2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2);
+    // Fetch position: tile, step inside it, steps not yet fetched; as 32-bit byte offsets from the planes' bases
+    // (the host sends planes of 4 GiB and more to the other kernel), all advanced without branches.
+    int i_tcol = tcol;
+    int i_step = ((int)u - tcol * units) * unit_steps;
+    int i_left = (int)(u_end - u) * unit_steps;
+    const uint32_t step4 = 2 * (uint32_t)row4, step2 = 2 * (uint32_t)row2;
+    uint32_t off4 = (uint32_t)i_tcol * (uint32_t)tile_stride4 + (uint32_t)i_step * step4;
+    uint32_t off2 = (uint32_t)i_tcol * (uint32_t)tile_stride2 + (uint32_t)i_step * step2;
+    const int lg = lane & 31;
+    const uint32_t v2 = (uint32_t)((lane >> 5) * row2) + (lg ^ (lg >> 4)) * 16;
+    // A: the lower half of the wave brings rows 0 .. 3, eight lanes per row (see stream_tile); rows past m re-read
+    // row m-1, so the lanes that take part never depend on m.
+    const bool a_lane = lane < 32;
+    uint32_t vap;
+    {
+        const int prow = (lane >> 3) & 3, pch = lane & 7;
+        const int row = prow < nrows ? prow : nrows - 1;
+        vap = (uint32_t)row * (uint32_t)p.k * 2 + 16 * ((pch & 4) | ((pch & 3) ^ ((prow >> 1) & 3)));
+    }
+    const unsigned char* a0 = reinterpret_cast<const unsigned char*>(p.A);
+    uint32_t offa = (uint32_t)i_step * 64;
+    FP6M_AS3 unsigned char* a_ring = ring + DEPTH * kSlot;
+    int pair_in = 0;
+    const unsigned char* gs0 = reinterpret_cast<const unsigned char*>(p.s_int4);
+    const uint32_t gs_row = (uint32_t)p.n4 * 2;          // bytes from one group's scales to the next
+    const uint32_t vgs = 4 * lane;
+    FP6M_AS3 unsigned char* gs_ring = a_ring + kPairSlots * kPair;
+    int gs_in = 0;                                        // group-scale slab the next fetch fills (two alternate)
+
+    // `even`: the step fetched is the first of its pair (a compile-time fact at every call).  Returns whether a
+    // load of group scales went out.  Once the share's last step has been fetched, further calls repeat it.
+    auto issue = [&](int slot, bool even) {
+        FP6M_AS3 unsigned char* dst = ring + slot * kSlot;
+        if (even) {
+            if (a_lane) dma16(a0 + offa + vap, a_ring + pair_in * kPair);
+            pair_in = pair_in + 1 == kPairSlots ? 0 : pair_in + 1;
+            offa += i_left > 2 ? 128u : 0u;               // (the share's last pair is repeated)
+        }
+        dma16_stream(plane4 + off4 + v4, dst);
+        dma16_stream(plane4 + off4 + (uint32_t)row4 + v4, dst + 1024);
+        if (FP6) dma16_stream(plane2 + off2 + v2, dst + 2048);
+        const bool scales = kGroup && (i_step & 3) == 0;  // (never again once the position stops at the last, odd step)
+        if (scales) {
+            dma4(gs0 + (uint32_t)i_tcol * (kTileN * 2) + (uint32_t)(i_step >> 2) * gs_row + vgs, gs_ring + gs_in * 256);
+            gs_in ^= 1;
+        }
+        // the position moves on the scalar unit: next step, or the first step of the share's next tile
+        const bool more = i_left > 1;
+        const bool next_tile = more && i_step + 1 == tile_steps;
+        i_left -= more ? 1 : 0;
+        i_step = next_tile ? 0 : i_step + (more ? 1 : 0);
+        i_tcol += next_tile ? 1 : 0;
+        off4 = next_tile ? (uint32_t)i_tcol * (uint32_t)tile_stride4 : off4 + (more ? step4 : 0u);
+        off2 = next_tile ? (uint32_t)i_tcol * (uint32_t)tile_stride2 : off2 + (more ? step2 : 0u);
+        offa = next_tile ? 0u : offa;
+        return scales;
+    };
+    static_assert(!kGroup || DEPTH == 4, "the steps whose waits count a load of group scales are written out for depth 4");
+    constexpr int kWaitOdd = newer_step_ops(kWordOps, kAOps, 1, DEPTH - 2);
+    constexpr int kWaitEven = newer_step_ops(kWordOps, kAOps, 0, DEPTH - 2);
+
+    // ---- read side (lane = MFMA identity)
+    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;   // whose granule of the k-block this lane needs
+    const uint32_t ring_lds = (uint32_t)(uintptr_t)ring;
+    const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
+    const int gr2 = owner >> 1;
+    const uint32_t rd2 = ring_lds + 2048 + (gr2 ^ (gr2 >> 4)) * 16 + (owner & 1) * 8;
+    const int ar = c & (AROWS - 1);                       // rows beyond AROWS re-read a valid row; their sums are never stored
+    uint32_t rda[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+        rda[d] = (uint32_t)(uintptr_t)a_ring + (8 * ar + (d ^ ((ar >> 1) & 3))) * 16 + 4 * i;
+    const uint32_t rdgs = (uint32_t)(uintptr_t)gs_ring + (64 * (i >> 1) + 4 * (i & 1)) * 2;
+    int gs_rd = 0;
+    // behind the ring: 4 rows of kRedStride floats (an LDS-space pointer: no generic-address arithmetic)
+    FP6M_AS3 float* slab = (FP6M_AS3 float*)(ring + wave_lds_bytes(4, 3, 4));
+
+    auto fetch = [&](StepRegs& rg, int slot, int pair_slot, bool odd) {
+        const uint32_t so = slot * kSlot;
+        if (FP6) {
+            asm volatile(
+                "ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\t"
+                "ds_read_b64 %2, %5\n\tds_read_b64 %3, %5 offset:512"
+                : "=&v"(rg.q0), "=&v"(rg.q1), "=&v"(rg.t0), "=&v"(rg.t1) : "v"(rd4 + so), "v"(rd2 + so) : "memory");
+        } else {
+            asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024"
+                         : "=&v"(rg.q0), "=&v"(rg.q1) : "v"(rd4 + so) : "memory");
+        }
+        const uint32_t ao = pair_slot * kPair;
+        if (odd)                                // the second step of a pair: the other half of every row's line
+            asm volatile("ds_read_b32 %0, %4 offset:64\n\tds_read_b32 %1, %5 offset:64\n\t"
+                         "ds_read_b32 %2, %6 offset:64\n\tds_read_b32 %3, %7 offset:64"
+                         : "=&v"(rg.a[0]), "=&v"(rg.a[1]), "=&v"(rg.a[2]), "=&v"(rg.a[3])
+                         : "v"(rda[0] + ao), "v"(rda[1] + ao), "v"(rda[2] + ao), "v"(rda[3] + ao) : "memory");
+        else
+            asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7"
+                         : "=&v"(rg.a[0]), "=&v"(rg.a[1]), "=&v"(rg.a[2]), "=&v"(rg.a[3])
+                         : "v"(rda[0] + ao), "v"(rda[1] + ao), "v"(rda[2] + ao), "v"(rda[3] + ao) : "memory");
+    };
+    auto settle = [&](StepRegs& rg) {
+        asm volatile("" : "+v"(rg.q0), "+v"(rg.q1), "+v"(rg.a[0]), "+v"(rg.a[1]), "+v"(rg.a[2]), "+v"(rg.a[3]));
+        if (FP6) asm volatile("" : "+v"(rg.t0), "+v"(rg.t1));
+    };
+    auto compute = [&](const StepRegs& rg, f4 (&dst)[8], bool fresh) {
+        const h8 av = __builtin_bit_cast(h8, u4{rg.a[0], rg.a[1], rg.a[2], rg.a[3]});
+        const f4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            h2 r0[4], r1[4];
+            if (FP6) {
+                dequant_fp6_fast(rg.t0[jj >> 1] << (4 * (jj & 1)), rg.q0[jj], kc, r0);
+                dequant_fp6_fast(rg.t1[jj >> 1] << (4 * (jj & 1)), rg.q1[jj], kc, r1);
+            } else {
+                dequant_int4_fast(rg.q0[jj], kc, r0);
+                dequant_int4_fast(rg.q1[jj], kc, r1);
+            }
+            const h8 w_lo = join(r0[0], r0[1], r1[0], r1[1]);  // columns 16j + l
+            const h8 w_hi = join(r0[2], r0[3], r1[2], r1[3]);  // columns 16j + 8 + l
+            dst[2 * jj + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, av, fresh ? zero : dst[2 * jj + 0], 0, 0, 0);
+            dst[2 * jj + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, av, fresh ? zero : dst[2 * jj + 1], 0, 0, 0);
+        }
+    };
+
+    // ---- what has been added to shared tiles and not yet looked at
+    PendingCells pend;
+    pend.parts = 0;
+    auto settle_pending = [&]() {
+        if (pend.parts == 0) return;                                     // (uniform)
+        const FusedCols fcols = fused_cols(p, pend.col0 + 2 * lane);
+        uint16_t* c_out = p.C + pend.col0 + 2 * lane;
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            if (rr >= nrows) continue;
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                if ((int)(pend.old[rr][e] >> 56) != pend.parts - 1) continue;   // somebody else arrives last at this element
+                const float v = cell_total(pend.old[rr][e], cell_contribution(pend.v[rr][e]), pend.parts);
+                __hip_atomic_store(pend.cell + rr * kTileN + 64 * e, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (p.fused)
+                    store_fused_one(p, fcols, (size_t)rr, e, v);
+                else
+                    c_out[(size_t)rr * p.n + e] = __builtin_bit_cast(uint16_t, (_Float16)v);
+            }
+        }
+        pend.parts = 0;
+    };
+
+    // Pipeline: while step s is being computed, the LDS reads of step s+1 are in flight and the
+    // direct-to-LDS loads of steps s+2 .. s+DEPTH-1 are outstanding.
+    int slot_in = 0;
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; d++) {
+        issue(slot_in, (d & 1) == 0);
+        slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+    }
+    StepRegs regs[2];
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));         // step 0 has landed; step 1 is the oldest newer one
+    FP6M_MARK(p, 1);
+    fetch(regs[0], 0, 0, false);
+    int slot_rd = 1;                                      // slot of the step whose LDS reads come next
+    int pair_rd = 0;                                      // A ring slot of the pair that step belongs to
+    bool scales_in_flight = false;
+    f4 grp[8];
+    f4 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+
+    // Waves that share a SIMD are served oldest first, which lets the older one run ahead and leaves the younger
+    // one to stream alone afterwards, with half the loads in flight.  A wave therefore lowers its own priority
+    // as it gets through its share: whoever is further behind goes first, and the waves of a SIMD finish together.
+    const int share_steps = (int)(u_end - u) * unit_steps;
+    const int prio_step = (share_steps / 4 + kUnroll - 1) / kUnroll * kUnroll;
+    int steps_done = 0;
+    __builtin_amdgcn_s_setprio(3);
     while (u < u_end) {                                                  // (uniform) one segment per trip
-        const int kb = (int)u - ti.tcol * units;
+        const int kb = (int)u - tcol * units;
         const int left = (int)(u_end - u);
         const int len = units - kb < left ? units - kb : left;           // units of this tile in my share
-        ti.tile = FP6 ? ti.tcol : p.tiles6 + ti.tcol;
-        ti.col0 = (FP6 ? p.n4 : 0) + ti.tcol * kTileN;
+        const int tile = FP6 ? tcol : p.tiles6 + tcol;
+        const int col0 = (FP6 ? p.n4 : 0) + tcol * kTileN;
         h2 sv = {(_Float16)1.0f, (_Float16)1.0f};
-        if (kColumnScale) {                                              // fetched now, used after the loop
-            const int nr = ti.tcol * kTileN + 2 * (int)threadIdx.x;      // even column inside the region
+        if (kColumnScale) {                                              // fetched now, used after the segment
+            const int nr = tcol * kTileN + 2 * lane;                     // even column inside the region
             sv = *reinterpret_cast<const h2*>((FP6 ? p.s_fp6 : p.s_int4) + (nr & ~31) + scale_slot(nr & 31));
         }
-        f4 acc[1][8];
+        const int seg_steps = len * unit_steps;
+#pragma unroll 1
+        for (int s = 0; s < seg_steps; s += kUnroll) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) acc[0][t] = f4{0.f, 0.f, 0.f, 0.f};
-        stream_tile<FP6, G128, DEPTH, 4>(p, ti, ring, kb * unit_steps, (kb + len) * unit_steps, acc);
+            for (int uu = 0; uu < kUnroll; uu++) {
+                const bool scales = issue(slot_in, ((uu + DEPTH - 1) & 1) == 0);
+                slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+                if (kGroup && uu == 1) scales_in_flight = scales;         // the fetch of the step four on: a multiple of four
+                const bool one_more = kGroup && (uu == 1 || uu == 2) && scales_in_flight;
+                if (uu & 1) {                                             // the next step has landed
+                    if (one_more)
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd + 1));
+                    else
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));
+                } else {
+                    if (one_more)
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven + 1));
+                    else
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven));
+                }
+                if (uu & 1) pair_rd = pair_rd + 1 == kPairSlots ? 0 : pair_rd + 1;   // the next step opens a pair
+                fetch(regs[(uu + 1) & 1], slot_rd, pair_rd, (uu & 1) == 0);
+                slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
+                __builtin_amdgcn_s_waitcnt(lgkmcnt_only(kReads));         // reads of this step (older) are done
+                settle(regs[uu & 1]);
+                if (kGroup)
+                    compute(regs[uu & 1], grp, uu == 0);
+                else
+                    compute(regs[uu & 1], acc, false);
+            }
+            if (kGroup) {
+                // end of a 128-row group: fold it into the running sum with its scales (fp32)
+                const uint32_t ga = rdgs + gs_rd * 256;
+                gs_rd ^= 1;
+                u2 sc[8];
+                asm volatile(
+                    "ds_read_b64 %0, %8\n\tds_read_b64 %1, %8 offset:16\n\tds_read_b64 %2, %8 offset:32\n\t"
+                    "ds_read_b64 %3, %8 offset:48\n\tds_read_b64 %4, %8 offset:64\n\tds_read_b64 %5, %8 offset:80\n\t"
+                    "ds_read_b64 %6, %8 offset:96\n\tds_read_b64 %7, %8 offset:112\n\ts_waitcnt lgkmcnt(0)"
+                    : "=&v"(sc[0]), "=&v"(sc[1]), "=&v"(sc[2]), "=&v"(sc[3]), "=&v"(sc[4]), "=&v"(sc[5]), "=&v"(sc[6]),
+                      "=&v"(sc[7])
+                    : "v"(ga) : "memory");
+                settle(regs[0]);                              // lgkmcnt(0) also completed the look-ahead reads
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    const h2 lo = as_h2(sc[t][0]), hi = as_h2(sc[t][1]);
+                    acc[t][0] += (float)lo[0] * grp[t][0];
+                    acc[t][1] += (float)lo[1] * grp[t][1];
+                    acc[t][2] += (float)hi[0] * grp[t][2];
+                    acc[t][3] += (float)hi[1] * grp[t][3];
+                }
+            }
+            steps_done += kUnroll;
+            if (steps_done == prio_step) __builtin_amdgcn_s_setprio(2);
+            else if (steps_done == 2 * prio_step) __builtin_amdgcn_s_setprio(1);
+            else if (steps_done == 3 * prio_step) __builtin_amdgcn_s_setprio(0);
+        }
         FP6M_MARK(p, 2);
+
+        // ---- end of the segment: the look-ahead reads of the next step stay in flight, the ring is not touched
+        __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
+        settle(regs[0]);
         int parts = 1;
         if (len < units) {
-            const uint32_t t0 = (uint32_t)ti.tcol * (uint32_t)units;
+            const uint32_t t0 = (uint32_t)tcol * (uint32_t)units;
             const unsigned long long mq = FP6 ? p.magic_q6 : p.magic_q4, mqp = FP6 ? p.magic_q6p : p.magic_q4p;
             parts = sk_owner(t0 + units - 1, q, r, mq, mqp) - sk_owner(t0, q, r, mq, mqp) + 1;
         }
+        settle_pending();                                                // the previous segment's atomics are long back
+        // MFMA fragments -> fp32 rows in the slab (lane c holds row c of the tile's 16), read back with lane L owning
+        // columns 2L, 2L+1.  LDS operations of one wave execute in order: no barrier is needed.
+        const float rescale = FP6 ? 4096.0f : 1.0f;                      // the deferred e3m2 exponent re-bias
+        if (c < nrows) {
+            FP6M_AS3 float* mine = slab + c * kRedStride + 64 * (i >> 1) + 4 * (i & 1);
+#pragma unroll
+            for (int t = 0; t < 8; t++) *(FP6M_AS3 f4*)(mine + 16 * (t >> 1) + 8 * (t & 1)) = acc[t];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const float s0 = (float)sv[0] * rescale, s1 = (float)sv[1] * rescale;
+        float v0[4], v1[4];
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            const f2 t = *(const FP6M_AS3 f2*)(slab + (rr < nrows ? rr : 0) * kRedStride + 2 * lane);
+            v0[rr] = t[0] * s0;
+            v1[rr] = t[1] * s1;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+        FP6M_MARK(p, 3);
+        if (parts == 1) {
+            const FusedCols fcols = fused_cols(p, col0 + 2 * lane);
+            uint16_t* c_out = p.C + col0 + 2 * lane;
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                if (rr >= nrows) continue;
+                if (p.fused) {
+                    store_fused(p, fcols, (size_t)rr, v0[rr], v1[rr]);
+                } else {
+                    const h2 o = {(_Float16)v0[rr], (_Float16)v1[rr]};
+                    *reinterpret_cast<h2*>(c_out + (size_t)rr * p.n) = o;
+                }
+            }
+        } else {
+            // Shared tile: one returning atomic per element (cells of a row: 64 of the even columns, then 64 of the odd)
+            pend.cell = p.cells + (size_t)tile * nrows * kTileN + lane;
+            pend.parts = parts;
+            pend.col0 = col0;
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+                pend.v[rr][0] = v0[rr];
+                pend.v[rr][1] = v1[rr];
+                if (rr < nrows) {
+                    pend.old[rr][0] = __hip_atomic_fetch_add(pend.cell + rr * kTileN, cell_contribution(v0[rr]), __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT);
+                    pend.old[rr][1] = __hip_atomic_fetch_add(pend.cell + rr * kTileN + 64, cell_contribution(v1[rr]),
+                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            FP6M_MARK(p, 4);
+        }
         u += len;
-        wave_finish_sk(p, ti, parts, acc, (float)sv[0], (float)sv[1], ring);
-        ti.tcol++;
+        tcol++;
     }
+    // Redundant tail prefetches and look-ahead reads may still be in flight.
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+    settle(regs[0]);
+    settle(regs[1]);
+    settle_pending();
+    FP6M_MARK(p, 6);
 }
 
-constexpr int kSkWaveLds = wave_lds_bytes(4, 3, 4);
+constexpr int kSkWaveLds = wave_lds_bytes(4, 3, 4) + 4 * kRedStride * 4;   // ring, then the four-row slab
 
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
 template <bool G128>
@@ -264,9 +521,9 @@ __global__ __launch_bounds__(64, 3) void gemm_sk_kernel(const SkArgs in_kernarg_
 #endif
     const int logical = xcd_contiguous_id(blockIdx.x, p.waves);
     if (logical < p.waves6)                                              // the FP6 region's waves come first
-        sk_wave<true, G128>(p, logical, smem);
+        sk_wave<true, G128>(p, logical, (FP6M_AS3 unsigned char*)smem);
     else
-        sk_wave<false, G128>(p, logical - p.waves6, smem);
+        sk_wave<false, G128>(p, logical - p.waves6, (FP6M_AS3 unsigned char*)smem);
     FP6M_MARK(p, 7);
 }
 

@@ -219,6 +219,33 @@ def test_decode_kernel_with_eight_waves_per_workgroup(oracle):
     run(oracle, 1, 10240, 8192, qc=256, gs=128)                         # the dispatcher's own choice of it
 
 
+def test_one_wave_decode_kernel(oracle):
+    """The decode kernel (one wave per workgroup, equal shares of the (tile, k unit) list, parts of a tile added into
+    64-bit cells): the dispatcher uses it for one row; here also forced for two to four rows, with shares that divide
+    a tile, shares that cross tile boundaries (3 units of 16, exact wave counts), whole tiles (sms = 1), one part per
+    unit, FP6-only and INT4-only problems, both scale modes; and the workgroup kernel forced for one row."""
+    for m in (1, 2, 3, 4):
+        e = {"FP6M_SK": 1}
+        run(oracle, m, 512, 2048, qc=256, gs=128, env=e)
+        run(oracle, m, 512, 2048, qc=256, env=e)
+        run(oracle, m, 768, 1024, qc=128, gs=128, env=dict(e, FP6M_SHARE=3))      # 8 units per tile: shares cross tiles
+        run(oracle, m, 768, 1024, qc=128, env=dict(e, FP6M_SHARE=5))
+        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=37, FP6M_EXACT=1))
+        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=1000, FP6M_EXACT=1))
+        run(oracle, m, 512, 2048, qc=256, gs=128, sms=1, env=e)                   # whole tiles, no cells
+        run(oracle, m, 512, 2048, qc=256, gs=128, sms=3, env=e)
+        run(oracle, m, 512, 2048, qc=256, ksplit=16, env=e)
+        run(oracle, m, 512, 1024, qc=512, env=e)                                  # all FP6
+        run(oracle, m, 640, 1024, qc=-1, gs=128, env=dict(e, FP6M_SHARE=1))       # all INT4, one unit per wave
+        run(oracle, m, 256, 64, 64, 256, qc=-1, env=e)                            # a single unit
+    run(oracle, 1, 512, 2048, qc=256, gs=128, env={"FP6M_SK": 0})                 # one row on the workgroup kernel
+    run(oracle, 1, 768, 1024, qc=128, env={"FP6M_SK": 0})
+    for gs in (-1, 128):
+        one_hot_case(oracle, 4, 768, 1024, 256, gs, {"sk": 1, "share": 3})
+        one_hot_case(oracle, 1, 768, 1024, 256, gs)
+        one_hot_case(oracle, 1, 768, 1024, 256, gs, {"sk": 0})
+
+
 def test_max_par_chunks_m(oracle):
     """m-tiles beyond max_par go to further launches (fp6_marlin_cuda_kernel.cu:917-948)."""
     run(oracle, 300, 512, 512, qc=256, max_par=2)

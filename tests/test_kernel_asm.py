@@ -95,6 +95,10 @@ def test_mfma_loops_keep_accumulators_in_place(asm):
     # (group scales or not) x ((MB 2, MB 4, MB 4 with paired A fetches) x (4, 8 k slices) + (one, two tiles per workgroup))
     assert seen == 16
     assert not re.findall(r"\.vgpr_spill_count:\s+[1-9]", asm), "a kernel spills VGPRs"
+    # nothing may live in private memory either: a pointer that the compiler keeps on the stack costs the decode loop a
+    # scratch load and a full `s_waitcnt vmcnt(0)` per step (seen once with pointers advanced under uniform branches)
+    assert not re.findall(r"\.private_segment_fixed_size:\s+[1-9]", asm), "a kernel uses scratch memory"
+    assert "scratch_load" not in asm and "scratch_store" not in asm
 
 
 def test_kernel_arguments_are_loaded_in_one_batch(asm):
