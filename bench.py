@@ -33,8 +33,9 @@ for _p in (ROOT, os.path.join(ROOT, "fp6-marlin_amd")):
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline workload (mean of its four GEMMs): FETCH_SIZE + WRITE_SIZE from two
 # `rocprofv3 --pmc` runs of `bench.py --traffic-probe`, each scaled by what the same counter reads for a
-# 256 MiB device copy (x2.000 and x1.000); figures in profiles/gemm_m16_kernel_decode7b_hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27062631
+# 256 MiB device copy (x2.000 and x1.000); figures in profiles/gemm_sk_kernel_decode7b_hbm_traffic.txt.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 29070438
+TRAFFIC_PROFILE = "profiles/gemm_sk_kernel_decode7b_hbm_traffic.txt"
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLAMA7B = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
 LLAMA70B = [(8192, 10240), (8192, 8192), (8192, 57344), (28672, 8192)]
@@ -136,20 +137,26 @@ def cpu_baseline(torch):
 
 
 def graphed(torch, step, layers, steps):
-    """fn(i) for time_region that replays a HIP graph of `layers` consecutive steps (launch-bound loops
-    belong in graphs); steps that do not fill a whole graph run eagerly."""
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        for i in range(layers):
-            step(i)
-    whole = steps // layers
+    """fn(i) for time_region that replays HIP graphs of `layers` consecutive steps (launch-bound loops belong in
+    graphs); steps that do not fill a whole graph are replayed from a second, shorter graph, so that every timed
+    step runs the same way."""
+    whole, rest = divmod(steps, layers)
+    graph = None
+    if whole:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(layers):
+                step(i)
+    tail = None
+    if rest:
+        tail = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(tail):
+            for i in range(rest):
+                step(i)
 
     def run(i):
-        if i < whole:
-            graph.replay()
-        else:
-            step(i - whole)
-    return run, whole + (steps - whole * layers)
+        (graph if i < whole else tail).replay()
+    return run, whole + (1 if rest else 0)
 
 
 def headline(args):
@@ -200,18 +207,24 @@ def headline(args):
                    "m": m, "quant_cols": qc, "group_size": gs, "weight_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "fp6m::gemm_m16_kernel<true, 4, 1, WK, 4, 3> (WK = 4 or 8 waves per workgroup, chosen per shape)", "us_per_launch": round(per_launch * 1e6, 3),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in " + TRAFFIC_PROFILE +
+                                       ", not measured in this run",
+                     "kernel": "fp6m::gemm_sk_kernel<true>", "us_per_launch": round(per_launch * 1e6, 3),
                      "bytes_per_launch": step_bytes // launches_per_step},
         "cpu_baseline": cpu_baseline(torch),
         "fp16_hipblaslt": {"ms_per_step": round(wall16 / args.steps * 1e3, 5),
+                           "GBs": round(sum(2 * k * n for k, n in LLAMA7B) * args.steps / wall16 / 1e9, 1),
                            "speedup": round(wall16 / wall, 3)},
     }
     del model
     torch.cuda.empty_cache()
-    # the other two regimes BASELINE's metric names, one shape each (same protocol as --sweep)
-    out["other_regimes"] = [measure_shape(torch, fp6_marlin, gen, tag, mm, k, n, qc, gs, calls_target=60)
-                            for tag, mm, k, n in (("70B M=16 (HBM-bound)", 16, 8192, 57344),
-                                                  ("M=128 (MFMA-bound)", 128, 8192, 8192))]
+    # the other regimes BASELINE's metric names (same protocol as --sweep): the 70B layer shapes at M = 1 and 16 and
+    # the batch sweep on 8192 x 8192, each next to the fp16 GEMM of the same shape
+    if not args.headline_only:
+        regimes = [(f"70B M={mm}", mm, k, n) for mm in (1, 16) for (k, n) in LLAMA70B]
+        regimes += [(f"batch sweep M={mm}", mm, 8192, 8192) for mm in (2, 4, 8, 32, 64, 128, 256, 512, 1024)]
+        out["other_regimes"] = [measure_shape(torch, fp6_marlin, gen, tag, mm, k, n, qc, gs, calls_target=60)
+                                for tag, mm, k, n in regimes]
     print(json.dumps(out), flush=True)
 
 
@@ -266,7 +279,7 @@ def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100
     row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "layout": layout, "us": round(t * 1e6, 2),
            "weight_GBs": round(nbytes / t / 1e9, 1), "hbm_frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
            "TFLOPs": round(2 * m * k * n / t / 1e12, 2), "mfma_frac": round(2 * m * k * n / t / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-           "fp16_us": round(t16 * 1e6, 2), "speedup_vs_fp16": round(t16 / t, 2)}
+           "fp16_us": round(t16 * 1e6, 2), "fp16_GBs": round(2 * k * n / t16 / 1e9, 1), "speedup_vs_fp16": round(t16 / t, 2)}
     del probs, w16
     torch.cuda.empty_cache()
     return row
@@ -461,6 +474,7 @@ def main():
     ap.add_argument("--fused", type=str, default=None, help="m,k,n[,quant_cols,group_size]: time mul_fused against mul + torch kernels")
     ap.add_argument("--rows", type=str, default=None, help="m,k,n[,quant_rows]: time the row-mixed GEMM against two mul calls and an addition")
     ap.add_argument("--pack", type=str, default=None, help="k,n[,quant_cols,group_size]: time the on-GPU weight packer")
+    ap.add_argument("--headline-only", action="store_true", help="skip the other regimes' rows of the JSON line")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 256 MiB device copy, then one layer of GEMMs")
