@@ -82,6 +82,26 @@ class Problem:
         torch.matmul(self.A, self.W16, out=self.C)
 
 
+SETTLE_MS = 50.0
+
+
+def settle(torch, fn, calls, ms=SETTLE_MS):
+    """Replay the workload about to be timed for at least `ms` milliseconds (untimed) and return the number of calls.
+    An MI355X that has been idle (tensor set-up on the host, graph capture) needs tens of milliseconds of the same kind
+    of load to reach the clocks it sustains under it: measured on 8192 x 57344 at M=1, 50-58 us per launch right after
+    an idle period against 43-45 us after 20 ms of the same launches (an unrelated fp16 matmul loop does not do it,
+    and leaves the memory-bound launches slower).  Every timed region here -- the quantised GEMM and the fp16
+    baseline alike -- starts from the steady state a serving loop is in."""
+    n = 0
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for i in range(calls):
+            fn(i)
+        torch.cuda.synchronize()
+        n += calls
+    return n
+
+
 def time_region(torch, fn, iters):
     """Wall clock (synchronised on both sides) and HIP-event time of `iters` calls of fn(i)."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -177,22 +197,23 @@ def headline(args):
         for p in model[i % layers]:
             p.run_fp16(torch)
 
-    for i in range(args.warmup):
+    # (graphs are captured before the warm-up steps: capturing leaves the GPU idle for milliseconds, and the first
+    # launches after that run slower)
+    if args.warmup:
+        step(0)                                                          # (the first of the warm-up steps loads the kernels)
+        torch.cuda.synchronize()
+    fn, calls = (step, args.steps) if args.no_graph else graphed(torch, step, layers, args.steps)
+    for i in range(1, args.warmup):
         step(i)
+    settled = settle(torch, fn, calls)
+    wall, ev = time_region(torch, fn, calls)
+    step_fp16(0)
     torch.cuda.synchronize()
-    if args.no_graph:
-        wall, ev = time_region(torch, step, args.steps)
-    else:
-        fn, calls = graphed(torch, step, layers, args.steps)
-        wall, ev = time_region(torch, fn, calls)
-    for i in range(max(2, args.warmup // 4)):
+    fn16, calls16 = (step_fp16, args.steps) if args.no_graph else graphed(torch, step_fp16, layers, args.steps)
+    for i in range(1, max(2, args.warmup // 4)):
         step_fp16(i)
-    torch.cuda.synchronize()
-    if args.no_graph:
-        wall16, _ = time_region(torch, step_fp16, args.steps)
-    else:
-        fn16, calls16 = graphed(torch, step_fp16, layers, args.steps)
-        wall16, _ = time_region(torch, fn16, calls16)
+    settle(torch, fn16, calls16)
+    wall16, _ = time_region(torch, fn16, calls16)
 
     gbs = step_bytes * args.steps / wall / 1e9
     per_launch = ev / (args.steps * launches_per_step)
@@ -201,6 +222,8 @@ def headline(args):
         "metric": "weight-stream GB/s (M=1-16), TFLOP/s (M=128), speedup vs fp16 hipBLASLt",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall / args.steps * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "warmup_settle": f"after the {args.warmup} warm-up steps the same steps were replayed untimed for {SETTLE_MS:.0f} ms "
+                         f"({settled} graph replays) so that the clocks are those of a running serving loop",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "decode M=1, Llama-2-7B layer shapes 4096x12288 4096x4096 4096x22016 11008x4096, "
                                "INT4 g128 + 256 FP6 columns, one step = one layer (4 GEMMs), 8 layers cycled",
@@ -266,14 +289,15 @@ def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100
     def f16(i):
         torch.matmul(probs[0].A, w16[i % len(w16)], out=probs[0].C)
 
-    for i in range(10):
-        f(i)
-        f16(i)
+    f(0)                                                                 # (first call: scratch region, lazy module load)
+    f16(0)
     torch.cuda.synchronize()
     iters, iters16 = copies * max(1, calls_target // copies), len(w16) * max(1, calls_target // len(w16))
     fn, calls = graphed(torch, f, copies, iters)
-    _, ev = time_region(torch, fn, calls)
     fn16, calls16 = graphed(torch, f16, len(w16), iters16)
+    settle(torch, fn, calls)                                             # warm-up right before each timed region
+    _, ev = time_region(torch, fn, calls)
+    settle(torch, fn16, calls16)
     _, ev16 = time_region(torch, fn16, calls16)
     t, t16 = ev / iters, ev16 / iters16
     row = {"tag": tag, "m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "layout": layout, "us": round(t * 1e6, 2),
@@ -355,6 +379,7 @@ def fused_bench(args):
             f(i)
         torch.cuda.synchronize()
         fn, calls = graphed(torch, f, copies, iters)
+        settle(torch, fn, calls)
         _, ev = time_region(torch, fn, calls)
         row[name + "_us"] = round(ev / iters * 1e6, 2)
     print(json.dumps(row), flush=True)
@@ -400,6 +425,7 @@ def rows_bench(args):
             f(i)
         torch.cuda.synchronize()
         fn, calls = graphed(torch, f, copies, iters)
+        settle(torch, fn, calls)
         _, ev = time_region(torch, fn, calls)
         row[name + "_us"] = round(ev / iters * 1e6, 2)
     t = row["mul_rows_us"] * 1e-6

@@ -251,16 +251,20 @@ void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 // n / d as (n * magic) >> 40: exact for n < 2^24 and d < 2^16.
 inline unsigned long long magic40(long long d) { return ((1ULL << 40) + (unsigned long long)d - 1) / (unsigned long long)d; }
 
-// Share of a wave in units for a tile of `units` and a wish of at least `want`.  A short share should divide the tile,
-// so that no wave crosses a tile boundary for a few steps (taken if a divisor lies within 1.5 x the wish); for long
-// shares the boundary costs nothing worth a longer share (the next tile's words are fetched ahead).
+// Share of a wave in units for a tile of `units` and a wish of at least `want`: a divisor of the tile within
+// 1.5 x the wish if there is one, so that no wave crosses a tile boundary (the smallest for short shares, the
+// largest from six units on, where fewer parts per tile weighed more in the measurements), else the wish itself.
 inline long long pick_share(long long units, long long want)
 {
     if (want < 1) want = 1;
-    if (want >= units || want >= 8) return want;
+    if (want >= units) return want;
+    long long best = 0;
     for (long long q = want; q < units && 2 * q <= 3 * want; q++)
-        if (units % q == 0) return q;
-    return want;
+        if (units % q == 0) {
+            best = q;
+            if (want < 6) break;
+        }
+    return best ? best : want;
 }
 
 struct M16Config {

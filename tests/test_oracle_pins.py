@@ -196,13 +196,63 @@ def test_int4_quantize_closed_form(oracle):
         g = 256 if gs == -1 else gs
         assert s.shape == (256 // g, 64)
         amax = np.abs(w.reshape(256 // g, g, 64)).max(axis=1)
-        assert np.allclose(s.astype(np.float64), amax.astype(np.float64) * 2 / 15, rtol=2e-3)
+        assert np.allclose(s.astype(np.float64), amax.astype(np.float64) * 2 / 15, rtol=2e-3)   # (bit for bit: next test)
         srep = np.repeat(s, g, axis=0)
         assert np.array_equal(ref, ((codes.astype(np.float16) - np.float16(8)) * srep).astype(np.float16))
         assert codes.min() >= 0 and codes.max() <= 15
         assert np.abs(ref.astype(np.float64) - w.astype(np.float64)).max() <= srep.astype(np.float64).max() * 0.51 + 1e-6
         # the column maximum maps to +/-7.5 -> code 0/1 or 15/16 clamp: extremes are reached
         assert codes.max() == 15 or codes.min() <= 1
+
+
+def test_int4_scale_and_codes_against_numpy_binary16(oracle):
+    """The harness computes in torch CPU half arithmetic (test.py:88-92): every operation takes binary16 operands, is
+    carried out in binary32 and rounded back to binary16.  The same steps in numpy, each rounding written out, must
+    give the scale and the codes bit for bit: s = fp16(fp32(amax) * fp32(2/15)), code = clamp(rint(fp16(fp32(w) /
+    fp32(s))) + 8, 0, 15)."""
+    rng = np.random.default_rng(9)
+    w = rng.normal(0, 0.02, (256, 96)).astype(np.float16)
+    w[5, 3] = np.float16(0.3)                                            # an outlier: most of its column rounds to code 8
+    for gs in (-1, 128):
+        codes, s, ref = oracle.int4_quantize(w, gs)
+        g = 256 if gs == -1 else gs
+        amax = np.abs(w).reshape(256 // g, g, 96).max(axis=1)
+        s_np = (amax.astype(np.float32) * np.float32(2 / 15)).astype(np.float16)
+        assert np.array_equal(s.view(np.uint16), s_np.view(np.uint16))
+        srep = np.repeat(s_np, g, axis=0)
+        ratio = (w.astype(np.float32) / srep.astype(np.float32)).astype(np.float16)
+        want = np.clip(np.rint(ratio.astype(np.float32)).astype(np.int32) + 8, 0, 15)
+        assert np.array_equal(codes.astype(np.int32), want)
+        ref_np = ((want - 8).astype(np.float16).astype(np.float32) * srep.astype(np.float32)).astype(np.float16)
+        assert np.array_equal(ref.view(np.uint16), ref_np.view(np.uint16))
+
+
+def test_int4_rounding_ties(oracle):
+    """Constructed ties: with max|w| = 15/128 the scale is exactly 2^-6, so w = t * 2^-6 sits exactly half way between
+    two codes for t = +-0.5 ... +-7.5.  torch.round (test.py:90) rounds half to even, and the clamp (test.py:92) cuts
+    +8 to code 15: the expected codes below are written out by hand."""
+    import torch
+    import fp6_marlin
+    ties = [0.5, 1.5, 2.5, 3.5, 4.5, 5.5, 6.5, 7.5]
+    even = [0, 2, 2, 4, 4, 6, 6, 8]                                      # nearest even integer of each tie
+    expect = {}
+    for t, e in zip(ties, even):
+        expect[t] = min(e + 8, 15)
+        expect[-t] = max(-e + 8, 0)
+    col = [t for t in ties] + [-t for t in ties]
+    k = 128
+    w = np.zeros((k, 64), dtype=np.float16)
+    for c in range(64):
+        w[: len(col), c] = (np.array(col, dtype=np.float64) / 64).astype(np.float16)     # t * 2^-6: exact in binary16
+    assert np.abs(w).max() == np.float16(15 / 128)
+    for gs in (-1, 128):
+        codes, s, ref = oracle.int4_quantize(w, gs)
+        assert (s == np.float16(2 ** -6)).all()
+        for r, t in enumerate(col):
+            assert (codes[r] == expect[t]).all(), (t, codes[r, 0], expect[t])
+        assert (codes[len(col):] == 8).all()
+        c2, s2, r2 = fp6_marlin.int4_quantize(torch.from_numpy(w), gs)  # the shipped host routine agrees on the ties
+        assert np.array_equal(c2.numpy(), codes) and np.array_equal(s2.numpy(), s) and np.array_equal(r2.numpy(), ref)
 
 
 # --------------------------------------------------------------------------- wire format (MX)
