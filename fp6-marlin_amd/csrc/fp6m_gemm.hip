@@ -67,7 +67,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, exact = kUnset, share = kUnset, sk = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, sk = kUnset, cap = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -251,22 +251,6 @@ void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 // n / d as (n * magic) >> 40: exact for n < 2^24 and d < 2^16.
 inline unsigned long long magic40(long long d) { return ((1ULL << 40) + (unsigned long long)d - 1) / (unsigned long long)d; }
 
-// Share of a wave in units for a tile of `units` and a wish of at least `want`: a divisor of the tile within
-// 1.5 x the wish if there is one, so that no wave crosses a tile boundary (the smallest for short shares, the
-// largest from six units on, where fewer parts per tile weighed more in the measurements), else the wish itself.
-inline long long pick_share(long long units, long long want)
-{
-    if (want < 1) want = 1;
-    if (want >= units) return want;
-    long long best = 0;
-    for (long long q = want; q < units && 2 * q <= 3 * want; q++)
-        if (units % q == 0) {
-            best = q;
-            if (want < 6) break;
-        }
-    return best ? best : want;
-}
-
 struct M16Config {
     int id, wn, wk;
 };
@@ -337,7 +321,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"exact", &g_tuning.exact}, {"share", &g_tuning.share}, {"sk", &g_tuning.sk},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -578,7 +562,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         a.m, prob_n, prob_k, wn, wk, mtiles, a.ksplit, grid.x, grid.y);
             fp6m::launch_wm(a, g128, wn, grid, st);
         } else if (mb == 1 && !row_mix && (tune.sk != kUnset ? tune.sk != 0 && a.m <= 4 : a.m == 1) && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24) &&
-                   (long long)prob_k * prob_n / 2 < (1LL << 32)) {
+                   (long long)prob_k * prob_n / 2 < (1LL << 32) && (long long)(prob_n / 128) * max_par >= 2) {
             // One row (decode), weight mixed along n: one wave per workgroup, equal shares of every region's (tile,
             // k unit) list (gemm_sk.h).  The kernel takes up to four rows, but every wave adds its part of a shared
             // tile with one atomic per element, and from two rows on that traffic costs more than the barriers and
@@ -599,8 +583,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             sk.n4 = a.n4;
             sk.qc = a.qc;
             sk.tiles6 = a.tiles6;
-            sk.native = a.native;
-            sk.fused = a.fused;
+            sk.flags = (a.native ? 1 : 0) | (a.fused ? 2 : 0);
             sk.c_cols = a.c_cols;
             sk.bias = a.bias;
             sk.residual = a.residual;
@@ -610,62 +593,86 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
 #endif
             const long long tiles4 = a.tiles - a.tiles6;
             const long long u4 = units, u6 = prob_k / 64;              // FP6 tiles have no group scales: 64-row units
-            // Waves (measured on MI355X over 17 shapes): shorter shares are faster as long as all waves are resident at
-            // once (twelve per CU by registers) and a tile is not cut into more than about 32 parts (every part is
-            // one atomic per output element); beyond either bound times rise steeply.  So: the shortest share that
-            // keeps the waves below eleven per CU and the parts of a tile at 32.  An FP6 unit (64 rows, 6 KiB)
-            // counts like an INT4 unit (8 KiB with group scales, 4 KiB without): fewer bytes, more work per byte.
+            // Chunks and waves (measured on MI355X over 17 shapes).  Shorter chunks are faster as long as every chunk
+            // has a wave of its own resident at once (twelve waves per CU fit by registers; eleven are used) and a
+            // tile is not cut into more than 32 chunks (more made the adds to one cell queue up).  Chunks beyond the
+            // waves are drawn from the counters and processed correctly, but every draw and every further chunk's
+            // adds are returning atomics that the wave's loads queue behind, so that is the overflow path for
+            // problems too large for one chunk per wave, not the plan.  Hence: the shortest chunk that keeps the
+            // chunks below eleven per CU and a tile's at 32, moved to a divisor of the tile within 1.5 x if there is
+            // one (the largest from six units on, where fewer chunks per tile weighed more).  An FP6 unit (64 rows,
+            // 6 KiB) counts like an INT4 unit (8 KiB with group scales, 4 KiB without): fewer bytes, more work per
+            // byte.  Further bounds: a chunk has at least as many steps as the fetch side runs ahead (three; an INT4
+            // unit without group scales has two); `sms` caps the chunks of a tile (1: whole tiles only), a forced
+            // split cuts every tile into that many; and without room for the cells of every tile nothing is shared.
             long long waves_wanted = 11LL * cus;
+            if (tune.cap != kUnset && tune.cap > 0) waves_wanted = tune.cap;
             if (tune.wgs != kUnset && tune.wgs > 0) waves_wanted = tune.wgs;
-            const long long bytes4 = tiles4 * u4 * (g128 ? 8 : 4), bytes6 = (long long)a.tiles6 * u6 * 6;   // KiB
-            long long want4 = ((bytes4 + bytes6) / (g128 ? 8 : 4) + waves_wanted - 1) / waves_wanted;
-            if (want4 < (u4 + 31) / 32) want4 = (u4 + 31) / 32;
+            const long long work4 = tiles4 * u4, work6 = (long long)a.tiles6 * u6;
+            long long want4 = (work4 + work6 + waves_wanted - 1) / waves_wanted;
             long long want6 = g128 ? want4 : (want4 + 1) / 2;
-            if (want6 < (u6 + 31) / 32) want6 = (u6 + 31) / 32;
-            if (tune.share != kUnset && tune.share > 0) want4 = want6 = tune.share;
-            // Bounds: at most kMaxParts waves on one tile; `sms` caps the waves that share a tile (1: whole tiles
-            // only), a forced split cuts every tile into that many parts; and without room for the cells of every
-            // tile nothing is shared.
+            if (tune.wgs != kUnset) want4 = want6 = 1;                 // (tests: few waves, many chunks each)
             const bool cells_fit = (size_t)prob_n * a.m * sizeof(unsigned long long) <= kCellBytes;
-            auto share = [&](long long units_r, long long want) {
-                long long q = pick_share(units_r, want);
-                if (env_ks >= 1) q = units_r / (env_ks < units_r ? env_ks : units_r);   // (may not divide: shares then cross tiles)
-                if (q * kMaxParts < units_r) q = pick_share(units_r, (units_r + kMaxParts - 1) / kMaxParts);
-                if (sms > 1 && q * sms < units_r) q = pick_share(units_r, (units_r + sms - 1) / sms);
-                if ((sms == 1 || !cells_fit) && q < units_r) q = units_r;
+            auto chunk_units = [&](long long units_r, long long want, long long min_units) {
+                long long q = want > (units_r + 31) / 32 ? want : (units_r + 31) / 32;
+                if (q < units_r) {                                     // a divisor of the tile nearby
+                    long long best = 0;
+                    for (long long d = q; d < units_r && 2 * d <= 3 * q; d++)
+                        if (units_r % d == 0) {
+                            best = d;
+                            if (q < 6) break;
+                        }
+                    if (best) q = best;
+                }
+                if (tune.share != kUnset && tune.share > 0) q = tune.share;
+                if (env_ks >= 1) q = (units_r + env_ks - 1) / env_ks;
+                if (sms > 1 && q * sms < units_r) q = (units_r + sms - 1) / sms;
+                if (q < min_units) q = min_units;
+                if (q * kMaxParts < units_r) q = (units_r + kMaxParts - 1) / kMaxParts;
+                while (q < units_r && units_r % q != 0 && units_r % q < min_units) q++;   // (a tile's last chunk too)
+                if (sms == 1 || !cells_fit || q > units_r) q = units_r;
                 return q;
             };
-            const long long q4 = share(u4, want4), q6 = share(u6, want6);
-            const long long n4u = tiles4 * u4, n6u = (long long)a.tiles6 * u6;
-            long long w4 = tiles4 ? (n4u + q4 - 1) / q4 : 0, w6 = a.tiles6 ? (n6u + q6 - 1) / q6 : 0;
-            if (tune.exact != kUnset && tune.exact > 0 && sms <= 0 && env_ks < 1 && cells_fit) {
-                // exactly `waves_wanted` waves, dealt to the regions by bytes; shares as they come
-                w6 = a.tiles6 ? (waves_wanted * bytes6 * 3 / 2 + (bytes4 + bytes6 * 3 / 2) / 2) / (bytes4 + bytes6 * 3 / 2) : 0;
+            const long long q4 = chunk_units(u4, want4, g128 ? 1 : 2), q6 = chunk_units(u6, want6, 1);
+            const long long cpt4 = (u4 + q4 - 1) / q4, cpt6 = (u6 + q6 - 1) / q6;
+            const long long chunks4 = tiles4 * cpt4, chunks6 = (long long)a.tiles6 * cpt6;
+            // Waves: one per chunk, up to the number aimed at, which is dealt to the regions by their chunks.
+            long long w6 = chunks6, w4 = chunks4;
+            if (w4 + w6 > waves_wanted) {
+                w6 = a.tiles6 ? (waves_wanted * chunks6 + (chunks4 + chunks6) / 2) / (chunks4 + chunks6) : 0;
                 if (a.tiles6 && w6 < 1) w6 = 1;
-                if (w6 > n6u) w6 = n6u;
                 w4 = tiles4 ? waves_wanted - w6 : 0;
                 if (tiles4 && w4 < 1) w4 = 1;
-                if (w4 > n4u) w4 = n4u;
-                if (w4 && n4u / w4 * kMaxParts < u4) w4 = n4u / ((u4 + kMaxParts - 1) / kMaxParts);
-                if (w6 && n6u / w6 * kMaxParts < u6) w6 = n6u / ((u6 + kMaxParts - 1) / kMaxParts);
+                if (w4 > chunks4) w4 = chunks4;
+                if (w6 > chunks6) w6 = chunks6;
             }
             sk.waves = (int)(w4 + w6);
             sk.waves6 = (int)w6;
             sk.units4 = (int)u4;
             sk.units6 = (int)u6;
-            sk.q4 = w4 ? (int)(n4u / w4) : 1;
-            sk.r4 = w4 ? (int)(n4u % w4) : 0;
-            sk.q6 = w6 ? (int)(n6u / w6) : 1;
-            sk.r6 = w6 ? (int)(n6u % w6) : 0;
-            sk.magic_u4 = magic40(u4);
-            sk.magic_u6 = magic40(u6);
-            sk.magic_q4 = magic40(sk.q4);
-            sk.magic_q4p = magic40(sk.q4 + 1);
-            sk.magic_q6 = magic40(sk.q6);
-            sk.magic_q6p = magic40(sk.q6 + 1);
+            sk.q4 = (int)q4;
+            sk.cpt4 = (int)cpt4;
+            sk.q6 = (int)q6;
+            sk.cpt6 = (int)cpt6;
+            sk.magic_cpt4 = magic40(cpt4);
+            sk.magic_cpt6 = magic40(cpt6);
+            sk.total4 = chunks4 > w4 ? (int)chunks4 : 0;               // 0: one chunk per wave, no counter traffic
+            sk.total6 = chunks6 > w6 ? (int)chunks6 : 0;
+            sk.counters = a.counters;
+            // Counters: atomics on one address complete one after the other, about 0.3 us apart, and a wave's loads
+            // queue behind its own draw, so no more than four waves share a counter (with 64 counters for 2560 waves
+            // the first data arrived up to 15 us late).  They come out of the workspace the caller must provide
+            // (prob_n / 128 * max_par elements): a quarter of it at most for the FP6 region.
+            const long long ws_elems = (long long)(prob_n / 128) * max_par;
+            long long groups6 = a.tiles6 ? (w6 + 3) / 4 : 0;
+            if (groups6 > ws_elems / 4) groups6 = ws_elems / 4 > 0 ? ws_elems / 4 : 1;
+            long long groups4 = tiles4 ? (w4 + 3) / 4 : 0;
+            if (groups4 > ws_elems - groups6) groups4 = ws_elems - groups6;
+            if (groups4 > 65535) groups4 = 65535;
+            sk.groups = (int)(groups4 | (groups6 << 16));
             if (tune.verbose)
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: one-wave workgroups %lld (FP6) + %lld (INT4), units per tile %lld / %lld, "
-                        "units per wave %d / %d\n", a.m, prob_n, prob_k, w6, w4, u6, u4, sk.q6, sk.q4);
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: one-wave workgroups %lld (FP6) + %lld (INT4), chunks %lld of %lld units + "
+                        "%lld of %lld units\n", a.m, prob_n, prob_k, w6, w4, chunks6, q6, chunks4, q4);
             dim3 grid((unsigned)sk.waves, 1);
             if (g128)
                 hipLaunchKernelGGL((gemm_sk_kernel<true>), grid, dim3(64), 0, st, sk);

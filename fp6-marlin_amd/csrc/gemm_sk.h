@@ -11,12 +11,16 @@ namespace fp6m {
 //
 // Partition.  The reference's striped scheduler (fp6_marlin_cuda_kernel.cu:343-408) gives every CTA the same
 // number of (k tile, n tile) units and lets a CTA run over the end of one column slice into the next; the property
-// is that every SM streams the same number of bytes whatever the tile count.  Same property here at the
-// granularity of a wave: a workgroup is ONE wave, and the (tile, k unit) pairs of a region, tile-major, are cut
-// into one contiguous share per wave, equal to within one unit.  A wave walks its share segment by segment (a
-// segment = its part of one tile).  The host picks the number of waves; shares shorter than a tile are chosen to
-// divide it, so that only long shares ever cross a tile boundary.  INT4 and FP6 tiles are separate regions with
-// their own unit length and share.  Nothing in the kernel synchronises waves: no barrier, no LDS shared
+// is that every SM streams the same number of bytes whatever the tile count.  Here the property is reached
+// dynamically, at the granularity of a wave: a workgroup is ONE wave, every tile's k range is cut into chunks of
+// a few k units, and the chunks of a region, tile-major, form one list.  Wave j starts on chunk j; whenever a wave's
+// fetches reach the end of a chunk it moves on to the chunk it drew from a counter in `workspace` one chunk
+// earlier (one agent-scope atomic by one lane, its latency hidden behind a whole chunk).  Equal static shares left a
+// third of the run to a thinning tail of waves (those that share a SIMD with an older wave, or got their first
+// data late, finish up to twice as late as the first); with chunks every wave works until the list is empty.  The
+// counter is zero before and after the launch: each wave draws exactly one number past the end of the list, and the
+// wave that draws the last of them writes the zero back.  INT4 and FP6 tiles are separate regions with their own
+// unit length, chunk size, waves and counter.  Nothing in the kernel synchronises waves: no barrier, no LDS shared
 // between them.
 //
 // Reduction.  A segment that covers its tile's whole k range is scaled and stored.  Otherwise the tile is shared,
@@ -58,33 +62,41 @@ struct SkArgs {
     int tiles6;               // FP6 tiles come first in the tile list
     int waves, waves6;        // all waves; the FP6 region's come first
     int units4, units6;       // k units per tile (INT4: 128 rows with group scales, else 64; FP6: 64 rows)
-    int q4, r4, q6, r6;       // shares: wave j of a region owns q units from j * q + min(j, r) on, one more if j < r
-    int native, fused;
-    // block 2: n / d as (n * magic) >> 40 for d = units4, units6, q4, q4 + 1, q6, q6 + 1 (exact for n < 2^24, d < 2^16)
-    unsigned long long magic_u4, magic_u6, magic_q4, magic_q4p, magic_q6, magic_q6p;
+    int q4, cpt4, q6, cpt6;   // chunk: q units (the last of a tile may be shorter); chunks per tile
+    int flags;                // bit 0: planes in the gfx950 order, bit 1: fused epilogue work
+    int groups;               // counters (= sub-lists of chunks) of the INT4 region | of the FP6 region << 16
+    // block 2
+    unsigned long long magic_cpt4, magic_cpt6;   // n / cpt as (n * magic) >> 40 (exact for n < 2^24, cpt < 2^16)
+    int total4, total6;       // chunks of each region (0: the region's waves own one chunk each and draw nothing)
+    int* counters;            // the INT4 region's, then the FP6 region's; zero on entry, zero on exit
     const int32_t* c_cols;    // optional epilogue work (fp6m_mul_fused), as in GemmArgs
     const uint16_t* bias;
-    // block 3 (two more scalar loads)
     const uint16_t* residual;
     unsigned long long* timeline;   // performance debugging builds only
     static constexpr int k4 = 0;    // (the row mix does not come here)
 };
-static_assert(sizeof(SkArgs) == 208 && offsetof(SkArgs, m) == 64 && offsetof(SkArgs, magic_u4) == 128 &&
-              offsetof(SkArgs, residual) == 192, "three 64-byte blocks and a tail");
+// What the fused-epilogue helpers of gemm_common.h read.
+struct SkEpilogue {
+    int fused, n;
+    const int32_t* c_cols;
+    const uint16_t* bias;
+    const uint16_t* residual;
+    uint16_t* C;
+};
+static_assert(sizeof(SkArgs) == 192 && offsetof(SkArgs, m) == 64 && offsetof(SkArgs, magic_cpt4) == 128,
+              "three 64-byte blocks");
 
 __device__ __forceinline__ SkArgs load_sk_args()
 {
     typedef uint32_t u16v __attribute__((ext_vector_type(16)));
-    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
     u16v b0, b1, b2;
-    u4v b3;
     const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile(
-        "s_load_dwordx16 %0, %4, 0x0\n\ts_load_dwordx16 %1, %4, 0x40\n\ts_load_dwordx16 %2, %4, 0x80\n\t"
-        "s_load_dwordx4 %3, %4, 0xc0\n\ts_waitcnt lgkmcnt(0)"
-        : "=&s"(b0), "=&s"(b1), "=&s"(b2), "=&s"(b3) : "s"(ka));
+        "s_load_dwordx16 %0, %3, 0x0\n\ts_load_dwordx16 %1, %3, 0x40\n\ts_load_dwordx16 %2, %3, 0x80\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&s"(b0), "=&s"(b1), "=&s"(b2) : "s"(ka));
     struct Words {
-        uint32_t w[52];
+        uint32_t w[48];
     } raw;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
@@ -92,8 +104,6 @@ __device__ __forceinline__ SkArgs load_sk_args()
         raw.w[16 + i] = b1[i];
         raw.w[32 + i] = b2[i];
     }
-#pragma unroll
-    for (int i = 0; i < 4; i++) raw.w[48 + i] = b3[i];
     return __builtin_bit_cast(SkArgs, raw);
 }
 
@@ -118,13 +128,6 @@ __device__ __forceinline__ float cell_total(unsigned long long old, unsigned lon
     return (float)(long long)sum * (1.0f / (float)(1ll << kCellFracBits));
 }
 
-// Wave that owns unit x of a region whose shares are (q, r): the first r waves hold q + 1 units.
-__device__ __forceinline__ int sk_owner(uint32_t x, int q, int r, unsigned long long magic_q, unsigned long long magic_qp)
-{
-    const uint32_t head = (uint32_t)r * (uint32_t)(q + 1);
-    return x < head ? (int)mul_shift40(magic_qp, x) : r + (int)mul_shift40(magic_q, x - head);
-}
-
 // A shared tile's elements this wave has added to and not yet looked at: the atomics' results come back while the
 // wave is already streaming its next segment.
 struct PendingCells {
@@ -135,12 +138,13 @@ struct PendingCells {
     int col0;                      // the tile's first column in C
 };
 
-// The wave's whole share in one software pipeline.  This is stream_tile (gemm_m16.h) for at most four rows of A with
-// two changes.  The fetch side walks the share's steps across tile boundaries by itself (at a tile's last step the
-// pointers move to the next tile's first), so when the multiply side finishes a segment the words of the next one
-// are already in the ring or on their way: a wave pays the latency of a first load once, not once per segment.  And
-// because the ring is never drained in between, a segment's accumulators are turned into rows in a small slab of
-// their own behind the ring.
+// All chunks of a wave in one software pipeline.  This is stream_tile (gemm_m16.h) for at most four rows of A with
+// two changes.  The fetch side walks from chunk to chunk by itself (past a chunk's last step its position moves to the
+// first step of the next chunk), so when the multiply side finishes a chunk the words of the next one are already in
+// the ring or on their way: a wave pays the latency of a first load once, not once per chunk.  And because the ring
+// is never drained in between, a chunk's accumulators are turned into rows in a small slab of their own behind the
+// ring.  A chunk has at least as many steps as the fetch side runs ahead (DEPTH - 1), so the fetch side is never
+// more than one chunk ahead of the multiply side.
 template <bool FP6, bool G128>
 __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigned char* ring)
 {
@@ -168,28 +172,52 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     kc.top2 = vgpr_const(0xc0c0c0c0u);
     kc.exp_man = vgpr_const(0x9f009f00u);
 
-    // ---- the share
-    const int q = FP6 ? p.q6 : p.q4, r = FP6 ? p.r6 : p.r4;
+    // ---- chunks
+    const int q = FP6 ? p.q6 : p.q4, cpt = FP6 ? p.cpt6 : p.cpt4;
     const int units = FP6 ? p.units6 : p.units4;
-    const int tile_steps = units * unit_steps;
-    uint32_t u = (uint32_t)j * (uint32_t)q + (uint32_t)(j < r ? j : r);
-    const uint32_t u_end = u + (uint32_t)q + (j < r ? 1u : 0u);
-    int tcol = (int)mul_shift40(FP6 ? p.magic_u6 : p.magic_u4, u);
+    const unsigned long long magic_cpt = FP6 ? p.magic_cpt6 : p.magic_cpt4;
+    const int total = FP6 ? p.total6 : p.total4;          // 0: one chunk per wave, nothing to draw
+    const int region_waves = FP6 ? p.waves6 : p.waves - p.waves6;
     const int region_n = FP6 ? p.qc : p.n4;
+    // chunk id -> tile of the region, first unit, units
+    auto chunk_tile = [&](int ch) { return (int)mul_shift40(magic_cpt, (uint32_t)ch); };
+    auto chunk_len = [&](int kb) { return units - kb < q ? units - kb : q; };
+    // A single counter would see every wave's first draw at the same moment (thousands of atomics on one address:
+    // tens of microseconds).  The list is therefore dealt into `groups` sub-lists (chunk c belongs to sub-list
+    // c mod groups) with a counter each, and wave j draws from sub-list j mod groups: consecutive waves sit on the
+    // same XCD, so every sub-list's waves are spread over the whole chip.
+    const int groups = FP6 ? p.groups >> 16 : p.groups & 0xffff;
+    const int group = j % groups;
+    const int group_waves = (region_waves - group + groups - 1) / groups;   // waves j' = group mod groups
+    const int group_total = (total - group + groups - 1) / groups;          // chunks of the sub-list
+    int* counter = p.counters + (FP6 ? (p.groups & 0xffff) : 0) + group;
+    // The next chunk of this wave: drawn by lane 0 with an atomic the compiler does not see (it would wait for every
+    // load in flight before handing the result out); the result is used a whole chunk later, when waits for newer
+    // loads have long covered it: a chunk issues at least seven loads, the waits let at most six stay in flight.
+    uint32_t drawn = 0;                                   // (lane 0) value of the counter before this wave's draw
+    auto draw = [&]() {
+        if (lane == 0)
+            asm volatile("global_atomic_add %0, %1, %2, off sc0 sc1" : "=&v"(drawn) : "v"(counter), "v"(1u) : "memory");
+    };
+    bool more_chunks = total != 0;                        // false once a draw has come back past the end of the list
+    if (more_chunks) draw();
 
     // ---- fetch side (lane = position in the slot).  Uniform 64-bit bases advance on the scalar unit; each lane
     // only contributes a constant 32-bit offset.
     const uint32_t v4 = (lane ^ ((lane >> 4) & 3)) * 16;
     const size_t kblocks = (size_t)p.k / 16;
-    const size_t row4 = p.native ? 1024 : (size_t)region_n * 8, row2 = row4 / 2;
-    const size_t tile_stride4 = p.native ? kblocks * 1024 : 1024, tile_stride2 = tile_stride4 / 2;
+    const bool native = (p.flags & 1) != 0;
+    const SkEpilogue ep = {(p.flags >> 1) & 1, p.n, p.c_cols, p.bias, p.residual, p.C};
+    const size_t row4 = native ? 1024 : (size_t)region_n * 8, row2 = row4 / 2;
+    const size_t tile_stride4 = native ? kblocks * 1024 : 1024, tile_stride2 = tile_stride4 / 2;
     const unsigned char* plane4 = reinterpret_cast<const unsigned char*>(FP6 ? p.b_fp6_4 : p.b_int4);
     const unsigned char* plane2 = reinterpret_cast<const unsigned char*>(p.b_fp6_2);
-    // Fetch position: tile, step inside it, steps not yet fetched; as 32-bit byte offsets from the planes' bases
-    // (the host sends planes of 4 GiB and more to the other kernel), all advanced without branches.
-    int i_tcol = tcol;
-    int i_step = ((int)u - tcol * units) * unit_steps;
-    int i_left = (int)(u_end - u) * unit_steps;
+    // Fetch position: chunk, tile, step inside the tile, steps of the chunk not yet fetched; as 32-bit byte offsets
+    // from the planes' bases (the host sends planes of 4 GiB and more to the other kernel).
+    int f_chunk = j;
+    int i_tcol = chunk_tile(j);
+    int i_step = (j - i_tcol * cpt) * q * unit_steps;
+    int i_left = chunk_len((j - i_tcol * cpt) * q) * unit_steps;
     const uint32_t step4 = 2 * (uint32_t)row4, step2 = 2 * (uint32_t)row2;
     uint32_t off4 = (uint32_t)i_tcol * (uint32_t)tile_stride4 + (uint32_t)i_step * step4;
     uint32_t off2 = (uint32_t)i_tcol * (uint32_t)tile_stride2 + (uint32_t)i_step * step2;
@@ -215,31 +243,51 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     int gs_in = 0;                                        // group-scale slab the next fetch fills (two alternate)
 
     // `even`: the step fetched is the first of its pair (a compile-time fact at every call).  Returns whether a
-    // load of group scales went out.  Once the share's last step has been fetched, further calls repeat it.
+    // load of group scales went out.  With the current chunk used up, the position first moves to the wave's next
+    // chunk (and the chunk after that is drawn); with no chunk left, the last step is fetched again.
     auto issue = [&](int slot, bool even) {
+        if (i_left == 0 && more_chunks) {                 // (uniform)
+            asm volatile("" : "+v"(drawn));
+            const int drawn_index = group_waves + (int)__builtin_amdgcn_readfirstlane(drawn);   // position in the sub-list
+            const int next = group + groups * drawn_index;
+            if (drawn_index < group_total) {
+                f_chunk = next;
+                i_tcol = chunk_tile(next);
+                const int kb = (next - i_tcol * cpt) * q;
+                i_step = kb * unit_steps;
+                i_left = chunk_len(kb) * unit_steps;
+                off4 = (uint32_t)i_tcol * (uint32_t)tile_stride4 + (uint32_t)i_step * step4;
+                off2 = (uint32_t)i_tcol * (uint32_t)tile_stride2 + (uint32_t)i_step * step2;
+                offa = (uint32_t)i_step * 64;
+                draw();
+            } else {
+                more_chunks = false;
+                // every wave draws exactly one number past the end; whoever draws the last of them leaves the
+                // counter at zero for the next launch
+                if (lane == 0 && drawn_index == group_total + group_waves - 1)
+                    __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
         FP6M_AS3 unsigned char* dst = ring + slot * kSlot;
         if (even) {
             if (a_lane) dma16(a0 + offa + vap, a_ring + pair_in * kPair);
             pair_in = pair_in + 1 == kPairSlots ? 0 : pair_in + 1;
-            offa += i_left > 2 ? 128u : 0u;               // (the share's last pair is repeated)
+            offa += i_left > 2 ? 128u : 0u;               // (a chunk's last pair stays, for the repeats at the very end)
         }
         dma16_stream(plane4 + off4 + v4, dst);
         dma16_stream(plane4 + off4 + (uint32_t)row4 + v4, dst + 1024);
         if (FP6) dma16_stream(plane2 + off2 + v2, dst + 2048);
-        const bool scales = kGroup && (i_step & 3) == 0;  // (never again once the position stops at the last, odd step)
+        const bool scales = kGroup && (i_step & 3) == 0 && i_left > 0;   // (not for the repeats)
         if (scales) {
             dma4(gs0 + (uint32_t)i_tcol * (kTileN * 2) + (uint32_t)(i_step >> 2) * gs_row + vgs, gs_ring + gs_in * 256);
             gs_in ^= 1;
         }
-        // the position moves on the scalar unit: next step, or the first step of the share's next tile
+        // on to the chunk's next step; after its last step the position stays (i_left == 0)
         const bool more = i_left > 1;
-        const bool next_tile = more && i_step + 1 == tile_steps;
-        i_left -= more ? 1 : 0;
-        i_step = next_tile ? 0 : i_step + (more ? 1 : 0);
-        i_tcol += next_tile ? 1 : 0;
-        off4 = next_tile ? (uint32_t)i_tcol * (uint32_t)tile_stride4 : off4 + (more ? step4 : 0u);
-        off2 = next_tile ? (uint32_t)i_tcol * (uint32_t)tile_stride2 : off2 + (more ? step2 : 0u);
-        offa = next_tile ? 0u : offa;
+        i_left -= i_left > 0 ? 1 : 0;
+        i_step += more ? 1 : 0;
+        off4 += more ? step4 : 0u;
+        off2 += more ? step2 : 0u;
         return scales;
     };
     static_assert(!kGroup || DEPTH == 4, "the steps whose waits count a load of group scales are written out for depth 4");
@@ -247,7 +295,7 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     constexpr int kWaitEven = newer_step_ops(kWordOps, kAOps, 0, DEPTH - 2);
 
     // ---- read side (lane = MFMA identity)
-    const int owner = p.native ? lane : 32 * sigma + 4 * l + i;   // whose granule of the k-block this lane needs
+    const int owner = native ? lane : 32 * sigma + 4 * l + i;     // whose granule of the k-block this lane needs
     const uint32_t ring_lds = (uint32_t)(uintptr_t)ring;
     const uint32_t rd4 = ring_lds + (owner ^ ((owner >> 4) & 3)) * 16;
     const int gr2 = owner >> 1;
@@ -313,7 +361,7 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     pend.parts = 0;
     auto settle_pending = [&]() {
         if (pend.parts == 0) return;                                     // (uniform)
-        const FusedCols fcols = fused_cols(p, pend.col0 + 2 * lane);
+        const FusedCols fcols = fused_cols(ep, pend.col0 + 2 * lane);
         uint16_t* c_out = p.C + pend.col0 + 2 * lane;
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
@@ -323,8 +371,8 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
                 if ((int)(pend.old[rr][e] >> 56) != pend.parts - 1) continue;   // somebody else arrives last at this element
                 const float v = cell_total(pend.old[rr][e], cell_contribution(pend.v[rr][e]), pend.parts);
                 __hip_atomic_store(pend.cell + rr * kTileN + 64 * e, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (p.fused)
-                    store_fused_one(p, fcols, (size_t)rr, e, v);
+                if (ep.fused)
+                    store_fused_one(ep, fcols, (size_t)rr, e, v);
                 else
                     c_out[(size_t)rr * p.n + e] = __builtin_bit_cast(uint16_t, (_Float16)v);
             }
@@ -352,17 +400,11 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
 #pragma unroll
     for (int t = 0; t < 8; t++) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
 
-    // Waves that share a SIMD are served oldest first, which lets the older one run ahead and leaves the younger
-    // one to stream alone afterwards, with half the loads in flight.  A wave therefore lowers its own priority
-    // as it gets through its share: whoever is further behind goes first, and the waves of a SIMD finish together.
-    const int share_steps = (int)(u_end - u) * unit_steps;
-    const int prio_step = (share_steps / 4 + kUnroll - 1) / kUnroll * kUnroll;
-    int steps_done = 0;
-    __builtin_amdgcn_s_setprio(3);
-    while (u < u_end) {                                                  // (uniform) one segment per trip
-        const int kb = (int)u - tcol * units;
-        const int left = (int)(u_end - u);
-        const int len = units - kb < left ? units - kb : left;           // units of this tile in my share
+    int c_chunk = j;                                      // the chunk the multiply side is on
+    while (true) {                                                       // (uniform) one chunk per trip
+        const int tcol = chunk_tile(c_chunk);
+        const int kb = (c_chunk - tcol * cpt) * q;
+        const int len = chunk_len(kb);
         const int tile = FP6 ? tcol : p.tiles6 + tcol;
         const int col0 = (FP6 ? p.n4 : 0) + tcol * kTileN;
         h2 sv = {(_Float16)1.0f, (_Float16)1.0f};
@@ -422,23 +464,14 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
                     acc[t][3] += (float)hi[1] * grp[t][3];
                 }
             }
-            steps_done += kUnroll;
-            if (steps_done == prio_step) __builtin_amdgcn_s_setprio(2);
-            else if (steps_done == 2 * prio_step) __builtin_amdgcn_s_setprio(1);
-            else if (steps_done == 3 * prio_step) __builtin_amdgcn_s_setprio(0);
         }
         FP6M_MARK(p, 2);
 
-        // ---- end of the segment: the look-ahead reads of the next step stay in flight, the ring is not touched
+        // ---- end of the chunk: the look-ahead reads of the next step stay in flight, the ring is not touched
         __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
         settle(regs[0]);
-        int parts = 1;
-        if (len < units) {
-            const uint32_t t0 = (uint32_t)tcol * (uint32_t)units;
-            const unsigned long long mq = FP6 ? p.magic_q6 : p.magic_q4, mqp = FP6 ? p.magic_q6p : p.magic_q4p;
-            parts = sk_owner(t0 + units - 1, q, r, mq, mqp) - sk_owner(t0, q, r, mq, mqp) + 1;
-        }
-        settle_pending();                                                // the previous segment's atomics are long back
+        const int parts = cpt;                                           // chunks (= waves) that share the tile
+        settle_pending();                                                // the previous chunk's atomics are long back
         // MFMA fragments -> fp32 rows in the slab (lane c holds row c of the tile's 16), read back with lane L owning
         // columns 2L, 2L+1.  LDS operations of one wave execute in order: no barrier is needed.
         const float rescale = FP6 ? 4096.0f : 1.0f;                      // the deferred e3m2 exponent re-bias
@@ -462,13 +495,13 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
         for (int t = 0; t < 8; t++) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
         FP6M_MARK(p, 3);
         if (parts == 1) {
-            const FusedCols fcols = fused_cols(p, col0 + 2 * lane);
+            const FusedCols fcols = fused_cols(ep, col0 + 2 * lane);
             uint16_t* c_out = p.C + col0 + 2 * lane;
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) {
                 if (rr >= nrows) continue;
-                if (p.fused) {
-                    store_fused(p, fcols, (size_t)rr, v0[rr], v1[rr]);
+                if (ep.fused) {
+                    store_fused(ep, fcols, (size_t)rr, v0[rr], v1[rr]);
                 } else {
                     const h2 o = {(_Float16)v0[rr], (_Float16)v1[rr]};
                     *reinterpret_cast<h2*>(c_out + (size_t)rr * p.n) = o;
@@ -492,8 +525,8 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
             }
             FP6M_MARK(p, 4);
         }
-        u += len;
-        tcol++;
+        if (f_chunk == c_chunk) break;                                   // the fetch side found no further chunk
+        c_chunk = f_chunk;                                               // (it is never more than one chunk ahead)
     }
     // Redundant tail prefetches and look-ahead reads may still be in flight.
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));

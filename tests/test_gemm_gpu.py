@@ -220,28 +220,34 @@ def test_decode_kernel_with_eight_waves_per_workgroup(oracle):
 
 
 def test_one_wave_decode_kernel(oracle):
-    """The decode kernel (one wave per workgroup, equal shares of the (tile, k unit) list, parts of a tile added into
-    64-bit cells): the dispatcher uses it for one row; here also forced for two to four rows, with shares that divide
-    a tile, shares that cross tile boundaries (3 units of 16, exact wave counts), whole tiles (sms = 1), one part per
-    unit, FP6-only and INT4-only problems, both scale modes; and the workgroup kernel forced for one row."""
+    """The decode kernel (one wave per workgroup, every tile's k range cut into chunks that the waves draw from a
+    counter, parts of a tile added into 64-bit cells): the dispatcher uses it for one row; here also forced for two to
+    four rows, with few waves (every wave draws many chunks), as many waves as chunks (nothing to draw), chunks that
+    do not divide a tile, whole tiles (sms = 1), FP6-only and INT4-only problems, both scale modes; and the
+    workgroup kernel forced for one row."""
     for m in (1, 2, 3, 4):
         e = {"FP6M_SK": 1}
         run(oracle, m, 512, 2048, qc=256, gs=128, env=e)
         run(oracle, m, 512, 2048, qc=256, env=e)
-        run(oracle, m, 768, 1024, qc=128, gs=128, env=dict(e, FP6M_SHARE=3))      # 8 units per tile: shares cross tiles
-        run(oracle, m, 768, 1024, qc=128, env=dict(e, FP6M_SHARE=5))
-        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=37, FP6M_EXACT=1))
-        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=1000, FP6M_EXACT=1))
+        run(oracle, m, 768, 1024, qc=128, gs=128, env=dict(e, FP6M_SHARE=3))      # 8 units per tile: chunks of 3, 3, 2
+        run(oracle, m, 768, 1024, qc=128, env=dict(e, FP6M_SHARE=5))              # 16 units per tile: 5, 5, 5, 1 -> 6, 6, 4
+        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=7))       # seven waves for 150 chunks
+        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=37, FP6M_SHARE=2))
+        run(oracle, m, 1024, 2048, qc=256, env=dict(e, FP6M_WGS=100))
+        run(oracle, m, 1024, 2048, qc=256, gs=128, env=dict(e, FP6M_WGS=100000))  # a wave per chunk
         run(oracle, m, 512, 2048, qc=256, gs=128, sms=1, env=e)                   # whole tiles, no cells
+        run(oracle, m, 512, 2048, qc=256, gs=128, sms=1, env=dict(e, FP6M_WGS=3)) # ... drawn by three waves
         run(oracle, m, 512, 2048, qc=256, gs=128, sms=3, env=e)
         run(oracle, m, 512, 2048, qc=256, ksplit=16, env=e)
         run(oracle, m, 512, 1024, qc=512, env=e)                                  # all FP6
-        run(oracle, m, 640, 1024, qc=-1, gs=128, env=dict(e, FP6M_SHARE=1))       # all INT4, one unit per wave
+        run(oracle, m, 512, 1024, qc=512, env=dict(e, FP6M_WGS=5))
+        run(oracle, m, 640, 1024, qc=-1, gs=128, env=dict(e, FP6M_SHARE=1))       # all INT4, one unit per chunk
+        run(oracle, m, 768, 192, 64, 256, qc=-1, env=dict(e, FP6M_SHARE=2))       # three units per tile, no group scales
         run(oracle, m, 256, 64, 64, 256, qc=-1, env=e)                            # a single unit
     run(oracle, 1, 512, 2048, qc=256, gs=128, env={"FP6M_SK": 0})                 # one row on the workgroup kernel
     run(oracle, 1, 768, 1024, qc=128, env={"FP6M_SK": 0})
     for gs in (-1, 128):
-        one_hot_case(oracle, 4, 768, 1024, 256, gs, {"sk": 1, "share": 3})
+        one_hot_case(oracle, 4, 768, 1024, 256, gs, {"sk": 1, "share": 3, "wgs": 11})
         one_hot_case(oracle, 1, 768, 1024, 256, gs)
         one_hot_case(oracle, 1, 768, 1024, 256, gs, {"sk": 0})
 
