@@ -610,8 +610,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (tune.wgs != kUnset && tune.wgs > 0) waves_wanted = tune.wgs;
             const long long work4 = tiles4 * u4, work6 = (long long)a.tiles6 * u6;
             long long want4 = (work4 + work6 + waves_wanted - 1) / waves_wanted;
-            long long want6 = g128 ? want4 : (want4 + 1) / 2;
-            if (tune.wgs != kUnset) want4 = want6 = 1;                 // (tests: few waves, many chunks each)
+            long long want6 = 1;
+            if (tune.wgs != kUnset) want4 = 1;                         // (tests: few waves, many chunks each)
             const bool cells_fit = (size_t)prob_n * a.m * sizeof(unsigned long long) <= kCellBytes;
             auto chunk_units = [&](long long units_r, long long want, long long min_units) {
                 long long q = want > (units_r + 31) / 32 ? want : (units_r + 31) / 32;
@@ -633,9 +633,19 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if (sms == 1 || !cells_fit || q > units_r) q = units_r;
                 return q;
             };
-            const long long q4 = chunk_units(u4, want4, g128 ? 1 : 2), q6 = chunk_units(u6, want6, 1);
-            const long long cpt4 = (u4 + q4 - 1) / q4, cpt6 = (u6 + q6 - 1) / q6;
-            const long long chunks4 = tiles4 * cpt4, chunks6 = (long long)a.tiles6 * cpt6;
+            long long q4, q6, cpt4, cpt6, chunks4, chunks6;
+            for (;; want4++) {                                         // (a last, shorter chunk per tile may push the count over)
+                want6 = g128 ? want4 : (want4 + 1) / 2;
+                q4 = chunk_units(u4, want4, g128 ? 1 : 2);
+                q6 = chunk_units(u6, want6, 1);
+                cpt4 = (u4 + q4 - 1) / q4;
+                cpt6 = (u6 + q6 - 1) / q6;
+                chunks4 = tiles4 * cpt4;
+                chunks6 = (long long)a.tiles6 * cpt6;
+                if (chunks4 + chunks6 <= waves_wanted || want4 >= u4 || tune.wgs != kUnset || tune.share != kUnset ||
+                    env_ks >= 1 || sms > 0)
+                    break;
+            }
             // Waves: one per chunk, up to the number aimed at, which is dealt to the regions by their chunks.
             long long w6 = chunks6, w4 = chunks4;
             if (w4 + w6 > waves_wanted) {
