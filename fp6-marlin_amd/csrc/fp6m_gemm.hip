@@ -67,7 +67,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, sk = kUnset, cap = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -321,7 +321,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -595,7 +595,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             const long long u4 = units, u6 = prob_k / 64;              // FP6 tiles have no group scales: 64-row units
             // Chunks and waves (measured on MI355X over 17 shapes).  Shorter chunks are faster as long as every chunk
             // has a wave of its own resident at once (twelve waves per CU fit by registers; eleven are used) and a
-            // tile is not cut into more than 32 chunks (more made the adds to one cell queue up).  Chunks beyond the
+            // tile is not cut into more than 32 chunks (more made the adds to one cell queue up; the few FP6 tiles, whose
+            // steps take twice as long, may have up to 64 as k grows, so that their waves do not finish last: 43 took
+            // 11008 x 4096 from 9.9 to 8.8 us and 56 took 28672 x 8192 from 25.2 to 24.7, while 64 chunks of one or two
+            // units cost 4096 x 4096 and 8192 x 8192 half a microsecond: short chunks all finish at the same time).  Chunks beyond the
             // waves are drawn from the counters and processed correctly, but every draw and every further chunk's
             // adds are returning atomics that the wave's loads queue behind, so that is the overflow path for
             // problems too large for one chunk per wave, not the plan.  Hence: the shortest chunk that keeps the
@@ -613,8 +616,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             long long want6 = 1;
             if (tune.wgs != kUnset) want4 = 1;                         // (tests: few waves, many chunks each)
             const bool cells_fit = (size_t)prob_n * a.m * sizeof(unsigned long long) <= kCellBytes;
-            auto chunk_units = [&](long long units_r, long long want, long long min_units) {
-                long long q = want > (units_r + 31) / 32 ? want : (units_r + 31) / 32;
+            auto chunk_units = [&](long long units_r, long long want, long long min_units, long long max_chunks) {
+                const long long floor_q = (units_r + max_chunks - 1) / max_chunks;
+                long long q = want > floor_q ? want : floor_q;
                 if (q < units_r) {                                     // a divisor of the tile nearby
                     long long best = 0;
                     for (long long d = q; d < units_r && 2 * d <= 3 * q; d++)
@@ -625,6 +629,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     if (best) q = best;
                 }
                 if (tune.share != kUnset && tune.share > 0) q = tune.share;
+                if (max_chunks != 32 && tune.share6 != kUnset && tune.share6 > 0) q = tune.share6;
                 if (env_ks >= 1) q = (units_r + env_ks - 1) / env_ks;
                 if (sms > 1 && q * sms < units_r) q = (units_r + sms - 1) / sms;
                 if (q < min_units) q = min_units;
@@ -633,11 +638,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if (sms == 1 || !cells_fit || q > units_r) q = units_r;
                 return q;
             };
+            const long long max_chunks6 = 32 + u6 / 16 < 64 ? 32 + u6 / 16 : 64;
             long long q4, q6, cpt4, cpt6, chunks4, chunks6;
             for (;; want4++) {                                         // (a last, shorter chunk per tile may push the count over)
                 want6 = g128 ? want4 : (want4 + 1) / 2;
-                q4 = chunk_units(u4, want4, g128 ? 1 : 2);
-                q6 = chunk_units(u6, want6, 1);
+                q4 = chunk_units(u4, want4, g128 ? 1 : 2, 32);
+                q6 = chunk_units(u6, want6, 1, max_chunks6);
                 cpt4 = (u4 + q4 - 1) / q4;
                 cpt6 = (u6 + q6 - 1) / q6;
                 chunks4 = tiles4 * cpt4;
