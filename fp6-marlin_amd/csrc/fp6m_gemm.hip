@@ -67,7 +67,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -321,7 +321,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -519,21 +519,22 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         a.C = static_cast<uint16_t*>(C) + (size_t)rows0 * prob_n;
         a.residual = fu.residual ? fu.residual + (size_t)rows0 * prob_n : nullptr;
         a.m = prob_m - rows0 < mtiles * rows_per_tile ? prob_m - rows0 : mtiles * rows_per_tile;
-        if (fu.a_cols) {
-            // the launch's rows of A, gathered into the per-device buffer (stream order keeps the launches apart)
+        a.A = static_cast<const uint16_t*>(A) + (size_t)rows0 * (fu.a_cols ? fu.lda : prob_k);
+        // fp6m_mul_fused's activation gather as a pass of its own: the launch's rows of A, gathered into the region's
+        // buffer (stream order keeps the launches apart), become the GEMM's A.  Every kernel but the decode kernel
+        // (which gathers by itself) starts with it.
+        auto gather_pass = [&]() {
+            if (!fu.a_cols) return;
             dim3 ggrid((unsigned)((prob_k / 2 + 255) / 256), (unsigned)a.m);
-            hipLaunchKernelGGL(gather_a_kernel, ggrid, dim3(256), 0, st,
-                               static_cast<const uint16_t*>(A) + (size_t)rows0 * fu.lda, fu.lda, fu.a_cols,
-                               region->gathered, prob_k);
+            hipLaunchKernelGGL(gather_a_kernel, ggrid, dim3(256), 0, st, a.A, fu.lda, fu.a_cols, region->gathered, prob_k);
             a.A = region->gathered;
-        } else {
-            a.A = static_cast<const uint16_t*>(A) + (size_t)rows0 * prob_k;
-        }
+        };
 
         const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
         const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
         const long long env_ks = tune.ksplit != kUnset ? tune.ksplit : 0;
         if (shared_frags) {
+            gather_pass();
             // two tiles per workgroup also share the A slabs: pays once the weights are large enough that
             // halving the grid still fills the chip (measured: 8192 x 16384 and up)
             int wn = weights >= (128LL << 20) ? 2 : 1;
@@ -569,7 +570,6 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // the partial-tile round trips of the workgroup kernel below (measured: 4096 x 4096 6.5 us at one row,
             // 8.2 at two, 12.8 at four, against 8.2 - 8.3 there).
             SkArgs sk;
-            sk.A = a.A;
             sk.b_int4 = a.b_int4;
             sk.b_fp6_2 = a.b_fp6_2;
             sk.b_fp6_4 = a.b_fp6_4;
@@ -674,6 +674,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             sk.magic_cpt6 = magic40(cpt6);
             sk.total4 = chunks4 > w4 ? (int)chunks4 : 0;               // 0: one chunk per wave, no counter traffic
             sk.total6 = chunks6 > w6 ? (int)chunks6 : 0;
+            // The activation gather: by the kernel itself for one row and one chunk per wave (two dependent loads per
+            // step pair and lane, hidden behind the weights' own latency), else by the pass.  From two rows on the
+            // kernel's extra loads (one per row, lane and pair) cost what the pass costs.
+            const bool gather_inside = fu.a_cols && a.m == 1 && !sk.total4 && !sk.total6 && (tune.gather == kUnset || tune.gather != 0);
+            if (!gather_inside) gather_pass();
+            sk.A = a.A;
+            sk.a_cols = gather_inside ? fu.a_cols : nullptr;
+            sk.lda = gather_inside ? fu.lda : 0;
+            sk.pad = 0;
             sk.counters = a.counters;
             // Counters: atomics on one address complete one after the other, about 0.3 us apart, and a wave's loads
             // queue behind its own draw, so no more than four waves share a counter (with 64 counters for 2560 waves
@@ -690,11 +699,18 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: one-wave workgroups %lld (FP6) + %lld (INT4), chunks %lld of %lld units + "
                         "%lld of %lld units\n", a.m, prob_n, prob_k, w6, w4, chunks6, q6, chunks4, q4);
             dim3 grid((unsigned)sk.waves, 1);
-            if (g128)
-                hipLaunchKernelGGL((gemm_sk_kernel<true>), grid, dim3(64), 0, st, sk);
+            // variants: group scales or not; one chunk per wave with or without the gather, or chunks drawn from counters
+            void (*kernel)(const SkArgs) = nullptr;
+            const bool draw = sk.total4 || sk.total6;
+            if (gather_inside)
+                kernel = g128 ? gemm_sk_kernel<true, 1, false> : gemm_sk_kernel<false, 1, false>;
+            else if (draw)
+                kernel = g128 ? gemm_sk_kernel<true, 0, true> : gemm_sk_kernel<false, 0, true>;
             else
-                hipLaunchKernelGGL((gemm_sk_kernel<false>), grid, dim3(64), 0, st, sk);
+                kernel = g128 ? gemm_sk_kernel<true, 0, false> : gemm_sk_kernel<false, 0, false>;
+            hipLaunchKernelGGL(kernel, grid, dim3(64), 0, st, sk);
         } else if (mb == 1) {
+            gather_pass();
             // m <= 16 (the row mix, and 5 to 16 rows of the column mix).  Each region (FP6, INT4) has its own number of k parts (workgroups) per tile group;
             // FP6 steps cost about twice an INT4 step, so the FP6 region is split twice as finely.  The
             // split is bounded so that every wave keeps at least one k unit, partial-sum traffic stays
@@ -797,6 +813,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x);
             launch_m16_any(cfg, a, g128, grid, st);
         } else {
+            gather_pass();
             // m > 16: a task is one workgroup (one tile x four k slices) on one row tile and k part.
             // Split k only as far as needed to give every CU a workgroup; partial tiles are 16*MB rows
             // of fp32, so the split is also capped by their traffic relative to the weight stream.

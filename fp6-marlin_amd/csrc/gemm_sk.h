@@ -43,8 +43,8 @@ constexpr unsigned long long kCellSumMask = kCellOne - 1;
 constexpr int kMaxParts = 255;                              // 255 * (2^47 + 2^46) < 2^56
 constexpr size_t kCellBytes = size_t(8) << 20;              // cells of one workspace: n * m * 8 bytes at most
 
-// Kernel arguments, laid out as three 64-byte blocks that the kernel fetches itself with three scalar loads
-// behind one wait (left to the compiler, the loads of the fields come in several dependent batches, each a
+// Kernel arguments, laid out as three 64-byte blocks and a 16-byte one that the kernel fetches itself with four
+// scalar loads behind one wait (left to the compiler, the loads of the fields come in several dependent batches, each a
 // round trip to a cold line before the wave's first weight load).
 struct SkArgs {
     // block 0
@@ -73,6 +73,10 @@ struct SkArgs {
     const uint16_t* bias;
     const uint16_t* residual;
     unsigned long long* timeline;   // performance debugging builds only
+    // block 3 (16 bytes): the activation gather of fp6m_mul_fused, done by the kernel itself (GR > 0)
+    const int32_t* a_cols;    // column kk of the GEMM's A is column a_cols[kk] (clamped) of the caller's matrix
+    int lda;                  // the caller's row length
+    int pad;
     static constexpr int k4 = 0;    // (the row mix does not come here)
 };
 // What the fused-epilogue helpers of gemm_common.h read.
@@ -83,20 +87,22 @@ struct SkEpilogue {
     const uint16_t* residual;
     uint16_t* C;
 };
-static_assert(sizeof(SkArgs) == 192 && offsetof(SkArgs, m) == 64 && offsetof(SkArgs, magic_cpt4) == 128,
-              "three 64-byte blocks");
+static_assert(sizeof(SkArgs) == 208 && offsetof(SkArgs, m) == 64 && offsetof(SkArgs, magic_cpt4) == 128 &&
+                  offsetof(SkArgs, a_cols) == 192,
+              "three 64-byte blocks and one of 16 bytes");
 
 __device__ __forceinline__ SkArgs load_sk_args()
 {
     typedef uint32_t u16v __attribute__((ext_vector_type(16)));
     u16v b0, b1, b2;
+    u4 b3;
     const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile(
-        "s_load_dwordx16 %0, %3, 0x0\n\ts_load_dwordx16 %1, %3, 0x40\n\ts_load_dwordx16 %2, %3, 0x80\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&s"(b0), "=&s"(b1), "=&s"(b2) : "s"(ka));
+        "s_load_dwordx16 %0, %4, 0x0\n\ts_load_dwordx16 %1, %4, 0x40\n\ts_load_dwordx16 %2, %4, 0x80\n\t"
+        "s_load_dwordx4 %3, %4, 0xc0\n\ts_waitcnt lgkmcnt(0)"
+        : "=&s"(b0), "=&s"(b1), "=&s"(b2), "=&s"(b3) : "s"(ka));
     struct Words {
-        uint32_t w[48];
+        uint32_t w[52];
     } raw;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
@@ -104,6 +110,8 @@ __device__ __forceinline__ SkArgs load_sk_args()
         raw.w[16 + i] = b1[i];
         raw.w[32 + i] = b2[i];
     }
+#pragma unroll
+    for (int i = 0; i < 4; i++) raw.w[48 + i] = b3[i];
     return __builtin_bit_cast(SkArgs, raw);
 }
 
@@ -145,7 +153,20 @@ struct PendingCells {
 // is never drained in between, a chunk's accumulators are turned into rows in a small slab of their own behind the
 // ring.  A chunk has at least as many steps as the fetch side runs ahead (DEPTH - 1), so the fetch side is never
 // more than one chunk ahead of the multiply side.
-template <bool FP6, bool G128>
+//
+// GR > 0: the activation gather (fp6m_mul_fused's a_cols) happens here instead of in a pass of its own.  A step pair
+// covers 64 columns of A, one per lane: the lane loads the pair's entry of the map (a dword, coalesced), then, with
+// the map entry as the address, its element of each of the GR rows (ushort loads), and writes them into the pair's
+// slot of the A ring where the direct-to-LDS load would have put them (ds_write_b16).  All three are scheduled by
+// the loop's own waits: the element loads and the next map load close the load group of the pair's first step, so
+// the wait that lets a step's words be read also covers them, the write to LDS follows that wait and precedes the
+// LDS reads of the pair (LDS operations of a wave execute in order), and the next element loads follow the write,
+// so one register per row suffices.  The map entry is fetched one pair earlier than the elements; the two dependent
+// loads hit the L2 and together take less time than the first weights take to come from memory.  Only with one
+// chunk per wave (the host sees to it).
+// DRAW = false: every wave has exactly one chunk (the host's plan whenever the chunks fit the waves); the code
+// that draws further chunks is left out, which frees a fifth of the registers.
+template <bool FP6, bool G128, int GR, bool DRAW>
 __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigned char* ring)
 {
     constexpr int DEPTH = FP6 ? 3 : 4;
@@ -157,7 +178,8 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     constexpr int kPair = pair_bytes(AROWS);
     constexpr int kSlot = FP6 ? 3072 : 2048;              // a step's packed words
     constexpr int kWordOps = FP6 ? 3 : 2;                 // direct-to-LDS loads of the packed words per step
-    constexpr int kAOps = 1;                              // ... and of A per pair of steps
+    constexpr int kAOps = GR > 0 ? 0 : 1;                 // ... and of A in front of a pair of steps
+    constexpr int kGatherOps = GR > 0 ? GR + 1 : 0;       // loads that close the group of a pair's first step (GR > 0)
     constexpr int kReads = FP6 ? 8 : 6;                   // LDS reads per step
     constexpr int kUnroll = kGroup ? 4 : 2;               // steps per loop trip (segments are multiples of it)
     typedef float f2 __attribute__((ext_vector_type(2)));
@@ -176,7 +198,8 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     const int q = FP6 ? p.q6 : p.q4, cpt = FP6 ? p.cpt6 : p.cpt4;
     const int units = FP6 ? p.units6 : p.units4;
     const unsigned long long magic_cpt = FP6 ? p.magic_cpt6 : p.magic_cpt4;
-    const int total = FP6 ? p.total6 : p.total4;          // 0: one chunk per wave, nothing to draw
+    static_assert(GR == 0 || !DRAW, "the gather follows one chunk");
+    const int total = !DRAW ? 0 : (FP6 ? p.total6 : p.total4);    // 0: one chunk per wave, nothing to draw
     const int region_waves = FP6 ? p.waves6 : p.waves - p.waves6;
     const int region_n = FP6 ? p.qc : p.n4;
     // chunk id -> tile of the region, first unit, units
@@ -269,7 +292,7 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
             }
         }
         FP6M_AS3 unsigned char* dst = ring + slot * kSlot;
-        if (even) {
+        if (GR == 0 && even) {
             if (a_lane) dma16(a0 + offa + vap, a_ring + pair_in * kPair);
             pair_in = pair_in + 1 == kPairSlots ? 0 : pair_in + 1;
             offa += i_left > 2 ? 128u : 0u;               // (a chunk's last pair stays, for the repeats at the very end)
@@ -291,8 +314,48 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
         return scales;
     };
     static_assert(!kGroup || DEPTH == 4, "the steps whose waits count a load of group scales are written out for depth 4");
+    // Loads that may be outstanding when the step after the current one must have landed: those of the DEPTH - 2
+    // newest steps, the first of them odd / even in its pair.  With the gather, the newest step's closing loads
+    // have not been issued yet at that point (they follow the wait), those of the one before have.
     constexpr int kWaitOdd = newer_step_ops(kWordOps, kAOps, 1, DEPTH - 2);
-    constexpr int kWaitEven = newer_step_ops(kWordOps, kAOps, 0, DEPTH - 2);
+    constexpr int kWaitEven = newer_step_ops(kWordOps, kAOps, 0, DEPTH - 2) + (DEPTH - 2 >= 2 ? kGatherOps : 0);
+    static_assert(GR == 0 || DEPTH == 3 || DEPTH == 4, "where the gather's loads sit among the counted ones");
+
+    // ---- gather (GR > 0): lane = column of the pair
+    uint32_t midx = 0, gval[GR > 0 ? GR : 1] = {};
+    const unsigned char* maps = reinterpret_cast<const unsigned char*>(p.a_cols);
+    const unsigned char* arow[GR > 0 ? GR : 1];
+    uint32_t wofs[GR > 0 ? GR : 1];
+#pragma unroll
+    for (int r = 0; r < (GR > 0 ? GR : 1); r++) {
+        const int row = r < nrows ? r : nrows - 1;
+        arow[r] = a0 + (size_t)row * (size_t)p.lda * 2;
+        // position of column `lane` of the pair in row r of a slot: see the swizzle of the fetch side above
+        wofs[r] = (uint32_t)(uintptr_t)a_ring +
+                  (8 * r + 4 * (lane >> 5) + (((lane >> 3) & 3) ^ ((r >> 1) & 3))) * 16 + 2 * (lane & 7);
+    }
+    // byte offsets into the map of the pair whose entry is loaded next / of the chunk's last pair (a wave has one
+    // chunk; past its end the last pair is loaded again, like the words)
+    uint32_t m_off = (uint32_t)i_step * 128, m_last = m_off + (uint32_t)(i_left / 2 - 1) * 256;
+    const int lda_max = p.lda - 1;
+    auto load_map = [&](uint32_t& dst) {
+        asm volatile("global_load_dword %0, %1, %2" : "=&v"(dst) : "v"(m_off + 4 * (uint32_t)lane), "s"(maps) : "memory");
+        m_off += m_off < m_last ? 256u : 0u;
+    };
+    auto load_vals = [&](uint32_t& idx) {
+        asm volatile("" : "+v"(idx));
+        int col = (int)idx;
+        col = col < 0 ? 0 : (col > lda_max ? lda_max : col);
+        const uint32_t vo = 2 * (uint32_t)col;
+#pragma unroll
+        for (int r = 0; r < GR; r++)
+            asm volatile("global_load_ushort %0, %1, %2" : "=&v"(gval[r]) : "v"(vo), "s"(arow[r]) : "memory");
+    };
+    auto write_vals = [&](int pair_slot) {
+#pragma unroll
+        for (int r = 0; r < GR; r++)
+            asm volatile("ds_write_b16 %0, %1" : : "v"(wofs[r] + pair_slot * kPair), "v"(gval[r]) : "memory");
+    };
 
     // ---- read side (lane = MFMA identity)
     const int owner = native ? lane : 32 * sigma + 4 * l + i;     // whose granule of the k-block this lane needs
@@ -383,13 +446,32 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     // Pipeline: while step s is being computed, the LDS reads of step s+1 are in flight and the
     // direct-to-LDS loads of steps s+2 .. s+DEPTH-1 are outstanding.
     int slot_in = 0;
+    uint32_t midx0 = 0;
+    if constexpr (GR > 0) {
+        load_map(midx0);
+        load_map(midx);
+    }
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; d++) {
         issue(slot_in, (d & 1) == 0);
         slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
     }
+    constexpr int kPrologueOps = (DEPTH - 1) * kWordOps + (kGroup ? 1 : 0);   // (a chunk's first step starts a group)
     StepRegs regs[2];
-    __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));         // step 0 has landed; step 1 is the oldest newer one
+    if constexpr (GR > 0) {
+        // The map entries of the first two pairs were the oldest loads (see below): wait for them only, fetch the
+        // first pair's elements, and wait for those, which also completes the words of the steps fetched ahead.
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(kPrologueOps));
+        load_vals(midx0);
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+        write_vals(0);
+        if (DEPTH - 1 > 2) {                                   // the second pair's first step is among those fetched ahead
+            load_vals(midx);
+            load_map(midx);
+        }
+    } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitOdd));     // step 0 has landed; step 1 is the oldest newer one
+    }
     FP6M_MARK(p, 1);
     fetch(regs[0], 0, 0, false);
     int slot_rd = 1;                                      // slot of the step whose LDS reads come next
@@ -433,6 +515,13 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
                         __builtin_amdgcn_s_waitcnt(vmcnt_only(kWaitEven));
                 }
                 if (uu & 1) pair_rd = pair_rd + 1 == kPairSlots ? 0 : pair_rd + 1;   // the next step opens a pair
+                if constexpr (GR > 0) {
+                    if (uu & 1) write_vals(pair_rd);                       // its elements have landed with its words
+                    if (((uu + DEPTH - 1) & 1) == 0) {                     // the step just fetched opens a pair: close its group
+                        load_vals(midx);
+                        load_map(midx);
+                    }
+                }
                 fetch(regs[(uu + 1) & 1], slot_rd, pair_rd, (uu & 1) == 0);
                 slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
                 __builtin_amdgcn_s_waitcnt(lgkmcnt_only(kReads));         // reads of this step (older) are done
@@ -532,6 +621,11 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
     settle(regs[0]);
     settle(regs[1]);
+    if constexpr (GR > 0) {
+        asm volatile("" : "+v"(midx));
+#pragma unroll
+        for (int r = 0; r < GR; r++) asm volatile("" : "+v"(gval[r]));
+    }
     settle_pending();
     FP6M_MARK(p, 6);
 }
@@ -539,7 +633,7 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
 constexpr int kSkWaveLds = wave_lds_bytes(4, 3, 4) + 4 * kRedStride * 4;   // ring, then the four-row slab
 
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
-template <bool G128>
+template <bool G128, int GR, bool DRAW>
 __global__ __launch_bounds__(64, 3) void gemm_sk_kernel(const SkArgs in_kernarg_segment)
 {
     __shared__ __attribute__((aligned(16))) unsigned char smem[kSkWaveLds];
@@ -554,9 +648,9 @@ __global__ __launch_bounds__(64, 3) void gemm_sk_kernel(const SkArgs in_kernarg_
 #endif
     const int logical = xcd_contiguous_id(blockIdx.x, p.waves);
     if (logical < p.waves6)                                              // the FP6 region's waves come first
-        sk_wave<true, G128>(p, logical, (FP6M_AS3 unsigned char*)smem);
+        sk_wave<true, G128, GR, DRAW>(p, logical, (FP6M_AS3 unsigned char*)smem);
     else
-        sk_wave<false, G128>(p, logical - p.waves6, (FP6M_AS3 unsigned char*)smem);
+        sk_wave<false, G128, GR, DRAW>(p, logical - p.waves6, (FP6M_AS3 unsigned char*)smem);
     FP6M_MARK(p, 7);
 }
 

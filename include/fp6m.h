@@ -117,8 +117,9 @@ int fp6m_repack_gfx950(const int32_t* in, int32_t* out, size_t k, size_t n, int 
  * any bias / residual addition to separate kernels of the caller.
  *   A, lda    device fp16 [m, lda] row-major.  Without a_cols, lda must equal prob_k.
  *   a_cols    device int32 [prob_k] or NULL: row kk of the packed weight multiplies column a_cols[kk] of A
- *             (0 <= a_cols[kk] < lda).  The gathered rows pass through a 64 MiB buffer of the call's workspace that the first
- *             such call allocates; min(prob_m, 64 * max_par) * prob_k * 2 bytes must fit (else FP6M_ERR_ARG).
+ *             (0 <= a_cols[kk] < lda).  With one row the decode kernel fetches A through the map itself; otherwise a
+ *             pass of its own gathers the rows into a 64 MiB buffer of the call's workspace, which the first call with a_cols
+ *             allocates; min(prob_m, 64 * max_par) * prob_k * 2 bytes must fit (else FP6M_ERR_ARG).
  *   c_cols    device int32 [prob_n] or NULL: packed column j (INT4 columns first, then the FP6 columns) is written
  *             to column c_cols[j] of C; must be a permutation of 0 .. prob_n-1.
  *   bias      device fp16 [prob_n] or NULL, indexed by C column.
@@ -156,7 +157,8 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * No counterpart in the reference (whose only such knob is the `sms` argument).  knob = "ksplit" (k parts per tile),
  * "wk16" / "wk" (waves per workgroup of the m <= 16 / m > 16 kernel: 4 or 8), "mb" (16-row blocks per wave: 2 or 4),
  * "wm" / "wn" (shared-fragment kernel on/off, its column tiles per workgroup), "pair" (paired activation fetch on/off),
- * "sk" (the one-wave decode kernel on for m <= 4 / off), "share" / "share6" (k units per chunk of its work list, both regions / the FP6 region only), "wgs" (its waves),
+ * "sk" (the one-wave decode kernel on for m <= 4 / off), "share" / "share6" (k units per chunk of its work list, both regions / the FP6 region only), "wgs" (its waves), "gather" (its own
+ * activation gather on / off),
  * "verbose" (print every launch's configuration to stderr); knob = NULL clears all overrides.  Unknown knob ->
  * FP6M_ERR_ARG.  Not synchronised with GEMM calls running on other threads.  The library reads no environment
  * variables on a call (FP6M_VERBOSE is looked up once at load time).

@@ -73,6 +73,35 @@ def test_scatter_and_gather_are_exact_reorders(oracle, m):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("k,n,qc,gs", [(4096, 4096, 256, 128), (4096, 4096, 256, -1), (1024, 768, 256, 128), (2048, 512, -1, 128),
+                                       (2048, 512, -1, -1), (1024, 384, 384, -1), (11008, 1024, 128, 128), (8192, 2048, 256, -1)])
+def test_one_row_gather_inside_the_decode_kernel(oracle, k, n, qc, gs):
+    """One row: the decode kernel gathers A itself (no pass of its own).  Bit for bit the result of `mul` on the
+    materialised row, and of the same call with the gather forced into the separate pass; map entries outside the row
+    are clamped to it, as the pass does."""
+    import fp6_marlin
+    print(f"case gather inside k={k} n={n} qc={qc} gs={gs}", flush=True)
+    ref, B, s = packed(oracle, k, n, qc, gs, seed=k + n)
+    g = torch.Generator().manual_seed(k)
+    lda = k + 192
+    A_wide = torch.randn((1, lda), generator=g).half().to(dev())
+    a_cols = torch.randperm(lda, generator=g)[:k].to(torch.int32)
+    a_cols[5], a_cols[k - 3] = -7, lda + 11                        # clamped to columns 0 and lda - 1
+    clamped = a_cols.clamp(0, lda - 1).long().to(dev())
+    a_cols = a_cols.to(dev())
+    want = plain(fp6_marlin, A_wide[:, clamped].contiguous(), B, s, n, qc, gs)
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+    for inside in (1, 0, 1):
+        C = torch.full((1, n), float("nan"), dtype=torch.half, device=dev())
+        with fp6_marlin.cabi.tuning(gather=inside):
+            fp6_marlin.mul_fused(A_wide, B, C, s, ws, qc, gs, a_cols=a_cols)
+        torch.cuda.synchronize()
+        assert torch.equal(C, want), inside
+        assert int(ws.abs().sum()) == 0
+    err = oracle.rel_err(want.cpu().numpy(), oracle.matmul_ref(A_wide[:, clamped].cpu().numpy(), ref))
+    assert err <= TOL
+
+
 @pytest.mark.parametrize("m", [3, 16, 40, 130])
 def test_bias_and_residual_round_once(oracle, m):
     """Integer-valued products: the bias-free output x is exact, so the fused result must be fp16(x + b + r)
