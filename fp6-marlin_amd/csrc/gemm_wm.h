@@ -12,15 +12,21 @@ namespace fp6m {
 // each) x two k slices of ONE tile: the four waves of a k slice fetch the tile's words once, each
 // dequantises a quarter of a step's operand fragments (one 16-column group) into LDS, and all four multiply
 // from there.  One workgroup barrier per step publishes the fragments and hands ring slots back to the
-// fetches; A stays private to its wave.  LDS per k slice: three slots (words [+ 2-bit plane], four 4 KiB A
-// slabs), two 8 KiB fragment buffers, two rows of group scales.
+// fetches; A stays private to its wave.  LDS per k slice: a ring of five steps of words [+ 2-bit plane], a ring of
+// three steps of A (four 4 KiB slabs each), two 8 KiB fragment buffers, two rows of group scales.
 
 constexpr int kWmRows = 4;                                           // row tiles per workgroup
 // WN adjacent tiles x (2 / WN) k slices: with WN = 2 the two tiles' waves also share the A slabs.
-template <int WN> constexpr int wm_slot_max() { return WN * 3072 + kWmRows * 4096; }
-template <int WN> constexpr int wm_frag_off() { return 3 * wm_slot_max<WN>(); }
+// LDS of a k slice: a ring of kWmWordDepth steps of packed words (3 KiB per tile and step), a ring of kWmADepth steps
+// of A (a 4 KiB slab per row tile), two fragment buffers per tile, two rows of group scales per tile.  The words are
+// small and come from memory, so they are fetched four steps ahead; A comes from the L2 and takes most of the LDS, so
+// it is fetched two steps ahead.
+constexpr int kWmWordDepth = 5, kWmADepth = 3;
+template <int WN> constexpr int wm_a_off() { return kWmWordDepth * WN * 3072; }
+template <int WN> constexpr int wm_frag_off() { return wm_a_off<WN>() + kWmADepth * kWmRows * 4096; }
 template <int WN> constexpr int wm_scale_off() { return wm_frag_off<WN>() + WN * 2 * 8192; }
-template <int WN> constexpr int wm_slice_lds() { return wm_scale_off<WN>() + WN * 512; }
+template <int WN> constexpr int wm_filler_off() { return wm_scale_off<WN>() + WN * 512; }   // 256 bytes nobody reads
+template <int WN> constexpr int wm_slice_lds() { return wm_filler_off<WN>() + 256; }
 constexpr int kWmRegion = 16 * kRedStride * 4;                       // one wave's 16-row block in the epilogue
 template <int WN> constexpr int wm_lds() { return max3((2 / WN) * wm_slice_lds<WN>(), 8 * kWmRegion, 0) + 64; }
 static_assert(wm_lds<1>() <= 160 * 1024 && wm_lds<2>() <= 160 * 1024, "LDS of one CU");
@@ -36,22 +42,26 @@ struct WmState {
 // two blocks of the next step; block 0 waits fragment by fragment.
 template <int BLK = 0>
 struct WmBlocks {
-    template <int phase, typename Hook>
+    // VMW: before the first read of the next step's A, wait until at most VMW vector-memory loads (the ones issued
+    // after that A) are outstanding.
+    template <int phase, int VMW, typename Hook>
     static __device__ __forceinline__ void run(WmState& st, f4 (&acc)[4][8], Hook&& hook)
     {
         if constexpr (BLK < 4) {
             constexpr int nb = BLK + 2;
             uint32_t (&dst)[4] = st.abuf[(phase + nb) & 3];
-            if constexpr (nb < 4)
+            if constexpr (nb < 4) {
                 lds_read_a4<nb * 1024>(dst, st.addr_cur);
-            else
+            } else {
+                if constexpr (nb == 4) __builtin_amdgcn_s_waitcnt(vmcnt_only(VMW));
                 lds_read_a4<(nb - 4) * 1024>(dst, st.addr_next);
+            }
             if constexpr (BLK > 0) __builtin_amdgcn_s_waitcnt(lgkmcnt_only(8));
             uint32_t (&src)[4] = st.abuf[(phase + BLK) & 3];
             asm volatile("" : "+v"(src[0]), "+v"(src[1]), "+v"(src[2]), "+v"(src[3]));
             const h8 av = __builtin_bit_cast(h8, u4{src[0], src[1], src[2], src[3]});
             step<0>(st, acc, av, hook);
-            WmBlocks<BLK + 1>::template run<phase>(st, acc, hook);
+            WmBlocks<BLK + 1>::template run<phase, VMW>(st, acc, hook);
         }
     }
     template <int T, typename Hook>
@@ -74,10 +84,12 @@ template <bool FP6, bool G128, int WN>
 __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo& ti, unsigned char* slice, int wm, int wn,
                                                int step_begin, int step_end, int loop_end, f4 (&acc)[4][8])
 {
-    constexpr int MB = 4, WM = kWmRows, DEPTH = 3;
+    constexpr int MB = 4, WM = kWmRows;
     constexpr bool kGroup = G128 && !FP6;
-    constexpr int kWBytes = FP6 ? 3072 : 2048;
-    constexpr int kSlot = WN * kWBytes + WM * 4096;
+    constexpr int kWSlot = WN * 3072;                                // a step's words of the WN tiles (3 KiB each, FP6 or not)
+    constexpr int kASlot = WM * 4096;
+    constexpr int kALoads = WN == 1 ? 4 : 2;                         // direct-to-LDS loads of A per wave and step
+    constexpr int kGroupOps = kALoads + 1;                           // ... and one load of the words' side
     constexpr int kUnroll = kGroup ? 4 : 2;
     const int lane = threadIdx.x & 63;
     const int i = lane >> 4, c = lane & 15, sigma = c >> 3, l = c & 7;
@@ -118,30 +130,17 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
     const uint32_t vgs = 4 * lane;
     const uint32_t slice_lds = uniform32(lds_addr(slice));
     const uint32_t gs_lds = slice_lds + wm_scale_off<WN>() + uniform32(wn * 512);
-    const uint32_t w_off = uniform32(wn * kWBytes);                   // this tile's words inside a slot
-    const uint32_t a_off = uniform32(WN * kWBytes + wm * 4096);       // this row tile's slab (shared by the WN tiles)
+    const uint32_t w_off = uniform32(wn * 3072);                      // this tile's words inside a word slot
+    const uint32_t a_off = uniform32(wm_a_off<WN>() + wm * 4096);     // this row tile's slab (shared by the WN tiles)
 
-    int issued = step_begin;
+    // Every wave issues, per step, its loads of A for the step two on and then exactly ONE load of the words' side
+    // for the step four on (k-block 0 / k-block 1 / the 2-bit plane / the group scales; a wave whose share does not
+    // exist for this tile or step loads 256 bytes into a corner of LDS that nobody reads), so that the counts in the waits below
+    // are the same for every wave.
+    int issued_a = step_begin, issued_w = step_begin;
     const int last = step_end - 1;
-    auto issue = [&](int slot) {
-        const uint32_t dst = slice_lds + slot * kSlot;
-        if (wm == 0) {
-            set_m0(dst + w_off);
-            dma16_m0<0, true>(base4, v4);
-        }
-        if (wm == 1) {
-            set_m0(dst + w_off);
-            dma16_m0<1024, true>(base4, v4b);
-        }
-        if (FP6 && wm == 2) {
-            set_m0(dst + w_off + 2048);
-            dma16_m0<0, true>(base2, v2);
-        }
-        if (kGroup && wm == 3 && (issued & 3) == 0) {
-            set_m0(gs_lds + ((issued >> 2) & 1) * 256);
-            dma4_m0(base_gs + (size_t)(issued >> 2) * (size_t)uniform32(p.n4) * 2, vgs);
-        }
-        set_m0(dst + a_off);
+    auto issue_a = [&](int slot) {
+        set_m0(slice_lds + a_off + slot * kASlot);
         if (WN == 1 || wn == 0) {                                     // with two tiles, each loads half of the slab
             dma16_m0<0, false>(base_a, va[0]);
             dma16_m0<1024, false>(base_a, va[1]);
@@ -150,11 +149,34 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
             dma16_m0<2048, false>(base_a, va[2]);
             dma16_m0<3072, false>(base_a, va[3]);
         }
-        if (issued < last) {
-            issued++;
+        if (issued_a < last) {
+            issued_a++;
+            base_a += 64;
+        }
+    };
+    auto issue_w = [&](int slot) {
+        const uint32_t dst = slice_lds + slot * kWSlot + w_off;
+        if (wm == 0) {
+            set_m0(dst);
+            dma16_m0<0, true>(base4, v4);
+        } else if (wm == 1) {
+            set_m0(dst);
+            dma16_m0<1024, true>(base4, v4b);
+        } else if (FP6 && wm == 2) {
+            set_m0(dst + 2048);
+            dma16_m0<0, true>(base2, v2);
+        } else if (kGroup && wm == 3 && (issued_w & 3) == 0) {
+            set_m0(gs_lds + ((issued_w >> 2) & 1) * 256);
+            dma4_m0(base_gs + (size_t)(issued_w >> 2) * (size_t)uniform32(p.n4) * 2, vgs);
+        } else {
+            // (into LDS, not a register: a register nobody reads would be reused while the load is in flight)
+            set_m0(slice_lds + wm_filler_off<WN>());
+            dma4_m0(base4, vgs);
+        }
+        if (issued_w < last) {
+            issued_w++;
             base4 += 2 * row4;
             base2 += 2 * row2;
-            base_a += 64;
         }
     };
 
@@ -176,7 +198,7 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
     h2 gs_cur[2], part[2];
     h8 mine[2];
     auto fetch_raw = [&](int slot) {
-        const uint32_t so = slot * kSlot;
+        const uint32_t so = slot * kWSlot;
         asm volatile("ds_read_b32 %0, %2\n\tds_read_b32 %1, %2 offset:1024" : "=&v"(q0), "=&v"(q1) : "v"(rd4 + so) : "memory");
         if (FP6)
             asm volatile("ds_read_b32 %0, %2\n\tds_read_b32 %1, %2 offset:512" : "=&v"(t0), "=&v"(t1) : "v"(rd2 + so) : "memory");
@@ -234,14 +256,16 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
                      : : "v"(frag_wr + buf * 8192), "v"(mine[0]), "v"(mine[1]) : "memory");
     };
     auto slot_addrs = [&](uint32_t (&addr)[4], int slot) {
-        const uint32_t so = slot * kSlot;
+        const uint32_t so = slot * kASlot;
 #pragma unroll
         for (int d = 0; d < 4; d++) addr[d] = rda[d] + so;
     };
 
-    issue(0);
-    issue(1);
-    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                        // steps 0 and 1: this wave's loads ...
+    issue_a(0);
+    issue_a(1);
+#pragma unroll
+    for (int d = 0; d < kWmWordDepth - 1; d++) issue_w(d);
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));                        // the steps fetched ahead: this wave's loads ...
     __builtin_amdgcn_s_barrier();                                     // ... and everybody else's
     slot_addrs(st.addr_next, 0);
     fetch_raw(0);
@@ -253,26 +277,30 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
 #pragma unroll
     for (int ck = 0; ck < 4; ck++) chunk(ck);
     publish(0);                                                       // step_begin is even
-    int slot_in = 2, slot_rd = 1;
+    int a_in = 2, a_rd = 1, w_in = kWmWordDepth - 1, w_rd = 1;
 #pragma unroll 1
     for (int s = step_begin; s < loop_end; s += kUnroll) {
 #pragma unroll
         for (int u = 0; u < kUnroll; u++) {
-            // step s+u+1 has landed and the fragments of step s+u are written, for everybody; everybody has
-            // left step s+u-1, whose slot the loads of step s+u+2 overwrite and whose fragment buffer this
-            // step's dequantisation refills
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
+            // The words' side of step s+u+1 has landed (this wave's share: the loads of the last two steps, issued
+            // after it, may be outstanding) and the fragments of step s+u are written, for everybody; everybody has
+            // left step s+u-1, whose A slot the loads of step s+u+2 overwrite and whose fragment buffer this step's
+            // dequantisation refills (its word slot was read a step earlier still).
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(2 * kGroupOps) & lgkmcnt_only(0));
             __builtin_amdgcn_s_barrier();
-            issue(slot_in);
-            slot_in = slot_in + 1 == DEPTH ? 0 : slot_in + 1;
+            issue_a(a_in);
+            issue_w(w_in);
+            a_in = a_in + 1 == kWmADepth ? 0 : a_in + 1;
+            w_in = w_in + 1 == kWmWordDepth ? 0 : w_in + 1;
             if (s >= step_end) continue;                              // (uniform) only keeping step with the others
 #pragma unroll
             for (int d = 0; d < 4; d++) st.addr_cur[d] = st.addr_next[d];
-            slot_addrs(st.addr_next, slot_rd);
-            fetch_raw(slot_rd);
+            slot_addrs(st.addr_next, a_rd);
+            fetch_raw(w_rd);
             const bool next_group = kGroup && u == kUnroll - 1;       // step s+u+1 starts a 128-row group
             if (next_group) fetch_scales((s + u + 1) >> 2);
-            slot_rd = slot_rd + 1 == DEPTH ? 0 : slot_rd + 1;
+            a_rd = a_rd + 1 == kWmADepth ? 0 : a_rd + 1;
+            w_rd = w_rd + 1 == kWmWordDepth ? 0 : w_rd + 1;
             fetch_frags(u & 1);
             auto hook = [&](auto blk, auto t) {
                 constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
@@ -282,10 +310,9 @@ __device__ __forceinline__ void stream_tile_wm(const GemmArgs& p, const TileInfo
                 if constexpr (mslot >= 8 && mslot < 24 && (mslot & 3) == 0) chunk((mslot - 8) >> 2);
                 if constexpr (mslot == 31) publish((u + 1) & 1);
             };
-            if ((u & 1) == 0)
-                WmBlocks<>::template run<0>(st, acc, hook);
-            else
-                WmBlocks<>::template run<0>(st, acc, hook);
+            // the A of step s+u+1 was fetched a step ago: behind it in the queue are that step's load of the words'
+            // side and this step's loads
+            WmBlocks<>::template run<0, kGroupOps + 1>(st, acc, hook);
         }
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0) & lgkmcnt_only(0));
