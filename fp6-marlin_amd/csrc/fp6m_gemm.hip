@@ -481,11 +481,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
 #endif
 
     // Row blocks per workgroup pass: 32 rows up to m = 32, 64 rows (accumulators in 128 VGPRs, two
-    // workgroups per CU) beyond.  128-row blocks (accumulators in AGPRs, one wave per SIMD) measured 10-15 %
-    // faster for m >= 512 but left the register allocator no slack, and were dropped.
+    // workgroups per CU) beyond; 128 rows for large launches whose grid allows it (below).
     int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     const Tuning tune = g_tuning;              // tuning/testing overrides (all unset in production)
-    if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4)) mb = tune.mb;
+    if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4 || tune.mb == 8)) mb = tune.mb;
     // Launches of 1024 rows on large weights: four 64-row tiles share the dequantised fragments of a tile
     // (gemm_wm_kernel).  Measured on MI355X it beats the private-fragment kernel by 13-20 % there and loses
     // below (m = 512: 102 vs 96 us on 8192 x 8192), where its 256-row workgroups leave CUs idle.
@@ -505,6 +504,18 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         return (int)(total - n6);
     };
     if (shared_frags) mb = 4;
+    // 128-row tiles (eight blocks per wave, accumulators in the accumulation registers, one wave per SIMD): every
+    // dequantised fragment feeds 16 MFMAs instead of 8, which measured 8-18 % faster than 64-row tiles wherever the
+    // grid still fills the chip (8192 x 8192: m = 384 72 -> 67 us, m = 512 88 -> 72; 4096 x 4096 at m = 1024 48 -> 43;
+    // 8192 x 28672 at m = 384 221 -> 206) and far slower where it does not (4096 x 4096 at m = 512: 128 workgroups,
+    // 27 -> 40 us).  One workgroup per CU is resident: taken when the workgroups fill their rounds to 85 %, or a
+    // single round to 70 %.
+    if (!shared_frags && !row_mix && tune.mb == kUnset && mb == 4 && prob_m > 256) {
+        const long long rows8 = prob_m < 128LL * max_par ? prob_m : 128LL * max_par;
+        const long long wgs8 = (long long)(prob_n / kTileN) * ((rows8 + 127) / 128);
+        const long long rounds = (wgs8 + cus - 1) / cus;
+        if (20 * wgs8 >= 17 * rounds * cus || (rounds == 1 && 10 * wgs8 >= 7 * cus)) mb = 8;
+    }
     const int rows_per_tile = 16 * mb;
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
     const int units = g128 ? prob_k / 128 : prob_k / 64;
@@ -833,6 +844,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
             int wk = base * ks <= cus && units / 16 >= ks ? 8 : kWaves;
             if (tune.wk != kUnset) wk = tune.wk == 8 ? 8 : kWaves;
+            if (mb == 8) wk = kWaves;                                  // (512 registers per wave: one wave per SIMD)
             // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
             // FP6 tiles' workgroups set the length of the launch (8192 x 8192 at m = 128: 33 us against 29 us with INT4
             // only).  Their k range is cut twice as finely where every slice still gets two units and the grid still
@@ -840,7 +852,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // a free CU loses far more than that).  A forced split applies to both kinds.
             a.ks4 = (int)ks;
             a.ks6 = (int)ks;
-            const long long resident = (long long)cus * (wk == 8 ? 1 : 2);
+            const long long resident = (long long)cus * (wk == 8 || mb == 8 ? 1 : 2);
             if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk &&
                 (base + (long long)a.tiles6 * mtiles) * ks <= resident)
                 a.ks6 = 2 * (int)ks;
@@ -862,8 +874,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // From two row tiles on, the requests A costs weigh more than the shorter look-ahead of the paired fetch
             // (measured: 64 rows 1-3 % slower with it, 128 rows 0-8 % faster, 256 and 512 rows 4-14 %).
             bool pair = a.m > 64;
-            if (tune.pair != kUnset) pair = mb == 4 && tune.pair != 0;
-            if (mb == 2) launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
+            if (tune.pair != kUnset) pair = mb >= 4 && tune.pair != 0;
+            if (mb == 8) {
+                void (*kernel)(const GemmArgs) = nullptr;
+                if (pair)
+                    kernel = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, true> : gemm_mb_kernel<false, 8, 3, 3, 4, true>;
+                else
+                    kernel = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, false> : gemm_mb_kernel<false, 8, 3, 3, 4, false>;
+                hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, a);
+            } else if (mb == 2) launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
             else if (pair) launch_mb<4, 3, 3, true>(a, g128, wk, grid, st);
             else launch_mb<4, 3, 3, false>(a, g128, wk, grid, st);
         }

@@ -50,6 +50,32 @@ __device__ __forceinline__ void mfma_acc(f4& acc, const h8& w, const h8& a)
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(w), "v"(a));
 }
 
+// Accumulators in the accumulation registers (eight 16-row blocks: 256 of them, next to the 256 ordinary registers
+// a wave that has a SIMD to itself may use).  The register class is all the asm statements ask for.  With all 256
+// taken the allocator still permutes some accumulators through ordinary registers at the loop's back edge (about a
+// hundred copies per trip of 256 MFMAs); naming each accumulator's quad in the constraints ("+{a[0:3]}") made that
+// worse: the copies in and out of the fixed registers around every statement no longer coalesced and spilled.
+template <bool FIRST>
+__device__ __forceinline__ void mfma_acc_a(f4& acc, const h8& w, const h8& a)
+{
+    if constexpr (FIRST)
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
+    else
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(a));
+}
+// Passes every accumulator through an empty asm: no read of it can be scheduled above this point.
+template <int MB, int I = 0>
+__device__ __forceinline__ void pin_all_acc(f4 (&acc)[MB][8])
+{
+    if constexpr (I < MB * 8) {
+        if constexpr (MB > 4)
+            asm volatile("" : "+a"(acc[I / 8][I % 8]));
+        else
+            asm volatile("" : "+v"(acc[I / 8][I % 8]));
+        pin_all_acc<MB, I + 1>(acc);
+    }
+}
+
 // Two of the four h2 a packed word expands to (half 0: fragment columns +0, half 1: columns +8).
 template <bool FP6>
 __device__ __forceinline__ void dequant_half(uint32_t q2, uint32_t q4, int half, const DequantConsts& k, h2& r0, h2& r1)
@@ -77,6 +103,20 @@ __device__ __forceinline__ void dequant_half(uint32_t q2, uint32_t q4, int half,
 // step's half-lines by all 16 rows is conflict-free.
 constexpr int kPairHalf = 1024 + 64;                      // from a block's first load to its second
 constexpr int kPairBlock = 2 * kPairHalf;                 // from block to block
+
+// The eight MFMAs of one 16-row block, `hook(block, t)` after each.
+template <int MB, int BLK, int T = 0, typename Hook>
+__device__ __forceinline__ void mfma_blocks_row(f4 (&acc)[MB][8], const h8 (&frag)[8], const h8& av, Hook&& hook)
+{
+    if constexpr (T < 8) {
+        if constexpr (MB > 4)
+            mfma_acc_a<T == 0>(acc[BLK][T], frag[T], av);
+        else
+            mfma_acc<T == 0>(acc[BLK][T], frag[T], av);
+        hook(Int<BLK>{}, Int<T>{});
+        mfma_blocks_row<MB, BLK, T + 1>(acc, frag, av, hook);
+    }
+}
 
 struct MbCtx {
     uint32_t abuf[4][4];
@@ -123,14 +163,7 @@ struct MbBlocks {
             uint32_t (&src)[4] = cx.abuf[(phase + BLK) & 3];
             asm volatile("" : "+v"(src[0]), "+v"(src[1]), "+v"(src[2]), "+v"(src[3]));
             const h8 av = __builtin_bit_cast(h8, u4{src[0], src[1], src[2], src[3]});
-            mfma_acc<true>(acc[BLK][0], frag[0], av); hook(Int<BLK>{}, Int<0>{});
-            mfma_acc<false>(acc[BLK][1], frag[1], av); hook(Int<BLK>{}, Int<1>{});
-            mfma_acc<false>(acc[BLK][2], frag[2], av); hook(Int<BLK>{}, Int<2>{});
-            mfma_acc<false>(acc[BLK][3], frag[3], av); hook(Int<BLK>{}, Int<3>{});
-            mfma_acc<false>(acc[BLK][4], frag[4], av); hook(Int<BLK>{}, Int<4>{});
-            mfma_acc<false>(acc[BLK][5], frag[5], av); hook(Int<BLK>{}, Int<5>{});
-            mfma_acc<false>(acc[BLK][6], frag[6], av); hook(Int<BLK>{}, Int<6>{});
-            mfma_acc<false>(acc[BLK][7], frag[7], av); hook(Int<BLK>{}, Int<7>{});
+            mfma_blocks_row<MB, BLK>(acc, frag, av, hook);
             MbBlocks<MB, kExtra, BLK + 1>::template run<phase, PAIRH, VMW>(cx, frag, acc, hook);
         }
     }
@@ -141,7 +174,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
                                                int step_begin, int step_end, f4 (&acc)[MB][8])
 {
     static_assert(DEPTH >= 3, "needs two steps of look-ahead");
-    static_assert(MB == 2 || MB == 4, "the A register ring assumes MB | 4; 128 accumulator VGPRs at most");
+    static_assert(MB == 2 || MB == 4 || MB == 8, "the A register ring assumes that MB divides or is a multiple of four");
     constexpr bool kGroup = G128 && !FP6;
     static_assert(!FP6 || DEPTH == 3, "the 2-bit plane alternates between two register sets");
     constexpr int kAOff = 2048;
@@ -368,12 +401,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     // MFMA results -> VALU reads: the wait states, then every accumulator is passed through an (empty)
     // asm so that no read of it can be scheduled above them.
     asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            asm volatile("" : "+v"(acc[mb][t]));
-        }
+    pin_all_acc<MB>(acc);
     if (FP6) {
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
@@ -414,7 +442,7 @@ template <bool FP6, bool G128, int MB>
 __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                                 int step_begin, int step_end, f4 (&acc)[MB][8])
 {
-    static_assert(MB == 4, "the A register ring runs with phase 0 in every step");
+    static_assert(MB == 4 || MB == 8, "the A register ring runs with phase 0 in every step");
     constexpr bool kGroup = G128 && !FP6;
     constexpr int kPair = MB * kPairBlock;                // one pair slot
     constexpr int kWOps = FP6 ? 4 : 2;                    // register loads per step
@@ -613,12 +641,7 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
     // MFMA results -> VALU reads: the wait states, then every accumulator is passed through an (empty)
     // asm so that no read of it can be scheduled above them.
     asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7");
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            asm volatile("" : "+v"(acc[mb][t]));
-        }
+    pin_all_acc<MB>(acc);
     // loads into the word registers may still have been in flight up to the wait above
 #pragma unroll
     for (int set = 0; set < 2; set++) {
@@ -814,11 +837,11 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 // would otherwise leave every SIMD a single wave.
 // PAIR: the INT4 tiles fetch A by pairs of steps and their words through registers (stream_tile_mbp).
 template <bool G128, int MB, int D4, int D6, int WK, bool PAIR>
-__global__ __launch_bounds__(64 * WK, WK == 4 ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
+__global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
 {
     // (FP6 tiles keep the ring: with the 2-bit plane's registers on top, the paired loop no longer fits 256 VGPRs.)
     constexpr bool kPaired = PAIR;
-    static_assert(!PAIR || MB == 4, "stream_tile_mbp is written for four blocks");
+    static_assert(!PAIR || MB == 4 || MB == 8, "stream_tile_mbp is written for whole rounds of the four A buffers");
     constexpr int kWaveLds = kPaired ? max3(mbp_wave_lds(MB), mb_wave_lds(MB, 0, D6), 0) : mb_wave_lds(MB, D4, D6);
     static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];

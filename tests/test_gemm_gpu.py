@@ -163,6 +163,26 @@ def test_shared_fragment_kernel(oracle):
     run(oracle, 1024, 768, 1024, qc=256, gs=128)                       # default dispatch stays on the other kernel
 
 
+def test_eight_row_blocks_per_wave(oracle):
+    """The m > 16 kernel with eight 16-row blocks per wave (128-row tiles, accumulators in the accumulation
+    registers), forced onto small problems: ragged row tiles, both regions, both scale modes, k splits through the
+    scratch, several launches, and one-hot rows bit for bit."""
+    for pair in (0, 1):                                                 # ring loop / paired activation fetch (INT4 tiles)
+        e = {"FP6M_MB": 8, "FP6M_WM": 0, "FP6M_PAIR": pair}
+        for m in (17, 100, 128, 129, 300):
+            run(oracle, m, 512, 1024, qc=256, gs=128, env=e)
+            run(oracle, m, 512, 1024, qc=256, env=e)
+        run(oracle, 200, 768, 512, qc=128, env=e)
+        run(oracle, 130, 256, 64, qc=-1, env=e)                         # one k unit: three idle slices
+        run(oracle, 260, 512, 2048, qc=256, gs=128, ksplit=3, env=e)
+        run(oracle, 520, 512, 512, qc=512, ksplit=2, env=e)             # all FP6
+        run(oracle, 2100, 256, 1024, qc=-1, gs=128, max_par=16, env=e)  # second launch of 52 rows
+        for n, k, qc in [(512, 256, 256), (768, 1024, 256)]:
+            for gs in (-1, 128):
+                one_hot_case(oracle, 200, n, k, qc, gs, {"mb": 8, "wm": 0, "pair": pair})
+                one_hot_case(oracle, 130, n, k, qc, gs, {"mb": 8, "wm": 0, "ksplit": 2, "pair": pair})
+
+
 def test_eight_k_slices_per_workgroup(oracle):
     """The m > 16 kernel with eight waves (k slices) per workgroup, which small grids on long k pick by themselves
     (here: 8192 x 512 at m = 40), forced on and off on ragged shapes."""

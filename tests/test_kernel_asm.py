@@ -85,15 +85,20 @@ def test_mfma_loops_keep_accumulators_in_place(asm):
             continue
         seen += 1
         meta = asm[asm.index(".name:           " + name) - 400:asm.index(".name:           " + name) + 800]
-        first, last = None, None
-        for n, l in enumerate(ins):
-            if l.startswith("v_mfma"):
-                first = n if first is None else first
-                last = n
-        moved = [l for l in ins[first:last] if l.startswith("v_accvgpr")]
+        # Between two MFMAs of one loop (fewer than 100 other instructions apart; what separates the FP6 loop from the
+        # INT4 loop of the same kernel is longer: with the accumulators in the accumulation registers the deferred
+        # FP6 re-bias reads and writes every one of them there) nothing may touch an accumulation register.
+        mfmas = [n for n, l in enumerate(ins) if l.startswith("v_mfma")]
+        moved = [l for a, b in zip(mfmas, mfmas[1:]) if b - a < 100 for l in ins[a:b] if l.startswith("v_accvgpr")]
+        if "gemm_mb_kernelILb1ELi8E" in name or "gemm_mb_kernelILb0ELi8E" in name:
+            # eight blocks: with all 256 accumulation registers taken the allocator permutes some accumulators through
+            # ordinary registers at the back edge of its two loops (four k steps = 256 MFMAs per trip): bounded, not none
+            assert len(moved) <= 300, f"{name}: {len(moved)} accumulator copies between MFMAs"
+            continue
         assert not moved, f"{name}: accumulator copies between MFMAs: {moved[:4]}"
-    # (group scales or not) x ((MB 2, MB 4, MB 4 with paired A fetches) x (4, 8 k slices) + (one, two tiles per workgroup))
-    assert seen == 16
+    # (group scales or not) x ((MB 2, MB 4, MB 4 with paired A fetches) x (4, 8 k slices) + MB 8 with and without them +
+    # (one, two tiles per workgroup))
+    assert seen == 20
     assert not re.findall(r"\.vgpr_spill_count:\s+[1-9]", asm), "a kernel spills VGPRs"
     # nothing may live in private memory either: a pointer that the compiler keeps on the stack costs the decode loop a
     # scratch load and a full `s_waitcnt vmcnt(0)` per step (seen once with pointers advanced under uniform branches)
@@ -120,4 +125,4 @@ def test_kernel_arguments_are_loaded_in_one_batch(asm):
         # the code of the epilogue may be laid out ahead of the loops: its loads (fused-epilogue pointers) do not count
         late = [(n, l) for n, l in late if not re.search(r"0x(a8|b0|b8)$", l)]
         assert not late, f"{name}: kernel-argument loads after the prologue: {late[:4]}"
-    assert seen == 30
+    assert seen == 34
