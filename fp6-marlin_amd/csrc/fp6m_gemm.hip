@@ -485,12 +485,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     const Tuning tune = g_tuning;              // tuning/testing overrides (all unset in production)
     if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4 || tune.mb == 8)) mb = tune.mb;
-    // Launches of 1024 rows on large weights: four 64-row tiles share the dequantised fragments of a tile
-    // (gemm_wm_kernel).  Measured on MI355X it beats the private-fragment kernel by 13-20 % there and loses
-    // below (m = 512: 102 vs 96 us on 8192 x 8192), where its 256-row workgroups leave CUs idle.
+    // Launches of 1024 rows on the largest weights: four 64-row tiles share the dequantised fragments of a tile
+    // (gemm_wm_kernel), two column tiles per workgroup.  Measured on MI355X it beats the 128-row tiles of the
+    // private-fragment kernel (below) by 5 % on 8192 x 16384 (262 vs 277 us at m = 1024), equals them on 8192 x 28672
+    // and loses on smaller weights (8192 x 8192: 146 vs 137 us) and below 1024 rows, where its 256-row workgroups
+    // leave CUs idle.
     const long long rows_per_launch = prob_m < 64LL * max_par ? prob_m : 64LL * max_par;
     const long long weights = (long long)prob_n * prob_k;
-    bool shared_frags = rows_per_launch >= 1024 && weights >= (64LL << 20);
+    bool shared_frags = rows_per_launch >= 1024 && weights >= (128LL << 20);
     if (tune.wm != kUnset) shared_frags = prob_m > 16 && tune.wm != 0;
     if (row_mix) shared_frags = false;                                // its waves run in lock step on one segment
     // Row mix: the kWaves * ks slices of a tile are dealt to the two segments in proportion to their cost (an FP6
@@ -506,8 +508,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     if (shared_frags) mb = 4;
     // 128-row tiles (eight blocks per wave, accumulators in the accumulation registers, one wave per SIMD): every
     // dequantised fragment feeds 16 MFMAs instead of 8, which measured 8-18 % faster than 64-row tiles wherever the
-    // grid still fills the chip (8192 x 8192: m = 384 72 -> 67 us, m = 512 88 -> 72; 4096 x 4096 at m = 1024 48 -> 43;
-    // 8192 x 28672 at m = 384 221 -> 206) and far slower where it does not (4096 x 4096 at m = 512: 128 workgroups,
+    // grid still fills the chip (8192 x 8192: m = 384 72 -> 65 us, m = 512 88 -> 69, m = 1024 175 -> 137; 4096 x 4096
+    // at m = 1024 48 -> 41; 8192 x 28672 at m = 384 221 -> 206) and far slower where it does not (4096 x 4096 at m = 512: 128 workgroups,
     // 27 -> 40 us).  One workgroup per CU is resident: taken when the workgroups fill their rounds to 85 %, or a
     // single round to 70 %.
     if (!shared_frags && !row_mix && tune.mb == kUnset && mb == 4 && prob_m > 256) {
@@ -547,7 +549,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         if (shared_frags) {
             gather_pass();
             // two tiles per workgroup also share the A slabs: pays once the weights are large enough that
-            // halving the grid still fills the chip (measured: 8192 x 16384 and up)
+            // halving the grid still fills the chip (measured: 8192 x 16384 and up; one tile per workgroup is
+            // what the tuning knob and the tests still reach)
             int wn = weights >= (128LL << 20) ? 2 : 1;
             if (tune.wn != kUnset) wn = tune.wn == 2 ? 2 : 1;
             const int wk = 2 / wn;

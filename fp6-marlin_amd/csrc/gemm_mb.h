@@ -866,9 +866,12 @@ __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb
     unsigned char* ring = smem + wave * kWaveLds;
     if (step_begin < step_end) {
         if constexpr (kPaired) {
-            if (ti.fp6)
-                stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
-            else
+            if (ti.fp6) {
+                if constexpr (MB > 4)                                    // (accumulators elsewhere: the registers are there)
+                    stream_tile_mbp<true, G128, MB>(p, ti, ring, step_begin, step_end, acc);
+                else
+                    stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+            } else
                 stream_tile_mbp<false, G128, MB>(p, ti, ring, step_begin, step_end, acc);
         } else {
             if (ti.fp6)
