@@ -183,6 +183,17 @@ def test_eight_row_blocks_per_wave(oracle):
                 one_hot_case(oracle, 130, n, k, qc, gs, {"mb": 8, "wm": 0, "ksplit": 2, "pair": pair})
 
 
+def test_dispatch_picks_128_row_tiles_where_they_fill_the_chip(oracle, capfd):
+    """The dispatcher's own choice: 128-row tiles for launches of more than 256 rows whose workgroups fill their rounds
+    of one per CU (here 32 column tiles x 8 row tiles = 256 workgroups, the last row tile ragged), 64-row tiles where
+    they do not (9 row tiles: 288 workgroups, two rounds at 56 %)."""
+    for m, want in ((1000, "MB=8"), (1024, "MB=8"), (1025, "MB=4"), (300, "MB=4")):
+        capfd.readouterr()
+        run(oracle, m, 4096, 512, qc=256, gs=128, env={"FP6M_VERBOSE": 1})
+        err = capfd.readouterr().err
+        assert want in err, (m, want, err[-400:])
+
+
 def test_eight_k_slices_per_workgroup(oracle):
     """The m > 16 kernel with eight waves (k slices) per workgroup, which small grids on long k pick by themselves
     (here: 8192 x 512 at m = 40), forced on and off on ragged shapes."""
