@@ -2,7 +2,7 @@
 """Benchmark of the mixed INT4/FP6 weight-only GEMM on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]          one JSON line (the driver's contract)
-    python bench.py --sweep sweep.json                           per-shape table for all BASELINE configs
+    python bench.py --sweep sweep.json                           per-shape table for all benchmark configurations
     python bench.py --shape 128,8192,8192                        one shape (m,k,n[,quant_cols,group_size])
 
 Workload of the JSON line: decode (M=1) through Llama-2-7B layer shapes (K x N) 4096x12288, 4096x4096,
@@ -241,7 +241,7 @@ def headline(args):
     }
     del model
     torch.cuda.empty_cache()
-    # the other regimes BASELINE's metric names (same protocol as --sweep): the 70B layer shapes at M = 1 and 16 and
+    # the other regimes the metric names (same protocol as --sweep): the 70B layer shapes at M = 1 and 16 and
     # the batch sweep on 8192 x 8192, each next to the fp16 GEMM of the same shape
     if not args.headline_only:
         regimes = [(f"70B M={mm}", mm, k, n) for mm in (1, 16) for (k, n) in LLAMA70B]
@@ -465,7 +465,7 @@ def pack_bench(args):
 
 
 def sweep(args):
-    """Per-shape numbers for every BASELINE configuration; written as JSON rows."""
+    """Per-shape numbers for every benchmark configuration; written as JSON rows."""
     import torch
     import fp6_marlin
     gen = torch.Generator().manual_seed(0)

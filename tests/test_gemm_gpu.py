@@ -4,7 +4,7 @@ GPU parity tests of the mixed INT4/FP6 GEMM, through the C ABI (fp6_marlin.mul -
 Oracle: dequantise-then-matmul (test.py:165-167) on operands quantised and packed by the CPU oracle;
 tolerance mean|C - C_ref| / mean|C_ref| <= 1e-3 (test.py:181).  The five groups of the reference's test.py
 are reproduced (tiles, k divisibility, very few k steps, errors, mixed), then group-128 scales, the
-BASELINE configurations, forced split-k reductions, and bit-exact one-hot probes that pin the layout at
+the benchmark's configurations (Llama-2 layer shapes, the M sweep), forced split-k reductions, and bit-exact one-hot probes that pin the layout at
 any size.
 """
 
@@ -370,7 +370,7 @@ MSWEEP = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024]
 
 
 def baseline_cases():
-    """(k, n) -> row counts: every shape x M that BASELINE configs 1-3 name, plus one shape of the two-tile
+    """(k, n) -> row counts: every shape x M of the benchmark's Llama-2-7B, Llama-2-70B and M-sweep configurations, plus one shape of the two-tile
     shared-fragment kernel."""
     cases = {}
     for k, n in LLAMA7B:
@@ -391,7 +391,7 @@ def tile_errors(c, ref, tile=128):
 
 @pytest.mark.parametrize("kn,ms", baseline_cases(), ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else None)
 def test_baseline_full_sizes_against_unpacked_words(oracle, kn, ms):
-    """BASELINE configs 1-3 at their real sizes, every shape x M.  The oracle cannot pack 8192 x 57344 in seconds, so
+    """The benchmark's Llama-2-7B, Llama-2-70B and M-sweep configurations at their real sizes, every shape x M.  The oracle cannot pack 8192 x 57344 in seconds, so
     the packed words are random bits (every FP6 code and INT4 nibble occurs) and the reference weight comes from the
     shipped unpacker, which tests/test_cpu_routines.py pins bit for bit against the oracle's dequantised weight; the
     reference product is an fp32 matmul of A with it.  The 1e-3 bar (test.py:181) is applied to every 128-column
