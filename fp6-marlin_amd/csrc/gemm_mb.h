@@ -54,7 +54,8 @@ __device__ __forceinline__ void mfma_acc(f4& acc, const h8& w, const h8& a)
 // a wave that has a SIMD to itself may use).  The register class is all the asm statements ask for.  With all 256
 // taken the allocator still permutes some accumulators through ordinary registers at the loop's back edge (about a
 // hundred copies per trip of 256 MFMAs); naming each accumulator's quad in the constraints ("+{a[0:3]}") made that
-// worse: the copies in and out of the fixed registers around every statement no longer coalesced and spilled.
+// worse: the copies in and out of the fixed registers around every statement no longer coalesced and spilled; the
+// MFMA builtin in place of the asm statements moved ten times as many.
 template <bool FIRST>
 __device__ __forceinline__ void mfma_acc_a(f4& acc, const h8& w, const h8& a)
 {
@@ -552,33 +553,73 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
             gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
         }
     };
-    // A quarter of one j group (4..8 VALU instructions): chunk = 4j + 2*half + word; see stream_tile_mb.
+    // Dequantisation of one step's words, cut into 48 stages of two or three VALU instructions: stage = 3 * chunk +
+    // phase, chunk = 4j + 2*half + word being a quarter of one j group (two h2 of one packed word).  The caller places
+    // the stages after consecutive MFMAs, so that no MFMA is followed by more VALU work than its own passes cover (a
+    // wave that has its SIMD to itself hides two independent VALU instructions per MFMA completely, each further one
+    // costs four cycles; a whole chunk in one place is six to eight, most of them dependent on their predecessor).
+    // Every stage ties its inputs and results to its place in the program (empty asm statements), so the scheduler
+    // leaves it between the two MFMAs it was placed between.
     h2 part[2];
-    auto chunk = [&](int ck, int set, h8 (&frag)[8]) {
+    uint32_t sx0 = 0, sx1 = 0;                             // the chunk in flight: between phase 0 and 1 ...
+    h2 sr0 = {(_Float16)0.f, (_Float16)0.f}, sr1 = sr0;    // ... and between phase 1 and 2
+    auto stage = [&](int st, int set, h8 (&frag)[8]) {
+        const int ck = st / 3, phase = st - 3 * ck;
         const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
-        uint32_t q4 = wq[set][word][j];
-        uint32_t q2 = 0;
-        asm volatile("" : "+v"(q4));
-        wq[set][word][j] = q4;
-        if (FP6) {
-            uint32_t t = tq[set][word][j >> 1];
-            asm volatile("" : "+v"(t));
-            tq[set][word][j >> 1] = t;
-            q2 = t << (4 * (j & 1));
-        }
-        h2 r0, r1;
-        dequant_half<FP6>(q2, q4, half, kc, r0, r1);
-        if (kGroup) {
-            r0 = r0 * gs_cur[2 * j + half];
-            r1 = r1 * gs_cur[2 * j + half];
-        }
-        if (word == 0) {
-            part[0] = r0;
-            part[1] = r1;
-            asm volatile("" : "+v"(part[0]), "+v"(part[1]));
+        if (phase == 0) {
+            uint32_t q4 = wq[set][word][j];
+            asm volatile("" : "+v"(q4));
+            wq[set][word][j] = q4;
+            if (FP6) {
+                uint32_t t = tq[set][word][j >> 1];
+                asm volatile("" : "+v"(t));
+                tq[set][word][j >> 1] = t;
+                const uint32_t q2 = t << (4 * (j & 1));
+                const uint32_t lo = half == 0 ? (q4 >> 2) : (q4 << 2);
+                const uint32_t hi = half == 0 ? q2 : (q2 << 2);
+                sx0 = (hi & kc.top2) | (lo & ~kc.top2);                  // s eeemm xx in every byte
+                asm volatile("" : "+v"(sx0));
+            } else {
+                const uint32_t q = half == 0 ? q4 : (q4 >> 8);
+                sx0 = (q & kc.lo) | kc.ex;
+                sx1 = (q & kc.hi) | kc.ex;
+                asm volatile("" : "+v"(sx0), "+v"(sx1));
+            }
+        } else if (phase == 1) {
+            asm volatile("" : "+v"(sx0), "+v"(sx1));
+            if (FP6) {
+                const s2 two = {2, 2};
+                sx1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, sx0 << 8) >> two);
+                sx0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, sx0) >> two);
+                asm volatile("" : "+v"(sx0), "+v"(sx1));
+            } else {
+                const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+                const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
+                const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+                sr0 = as_h2(sx0) - bias_lo;
+                sr1 = __builtin_elementwise_fma(as_h2(sx1), mul_hi, bias_hi);
+                asm volatile("" : "+v"(sr0), "+v"(sr1));
+            }
         } else {
-            frag[2 * j + half] = join(part[0], part[1], r0, r1);
-            asm volatile("" : "+v"(frag[2 * j + half]));
+            if (FP6) {
+                asm volatile("" : "+v"(sx0), "+v"(sx1));
+                sr0 = as_h2(sx0 & kc.exp_man);
+                sr1 = as_h2(sx1 & kc.exp_man);
+            } else {
+                asm volatile("" : "+v"(sr0), "+v"(sr1));
+                if (kGroup) {
+                    sr0 = sr0 * gs_cur[2 * j + half];
+                    sr1 = sr1 * gs_cur[2 * j + half];
+                }
+            }
+            if (word == 0) {
+                part[0] = sr0;
+                part[1] = sr1;
+                asm volatile("" : "+v"(part[0]), "+v"(part[1]));
+            } else {
+                frag[2 * j + half] = join(part[0], part[1], sr0, sr1);
+                asm volatile("" : "+v"(frag[2 * j + half]));
+            }
         }
     };
 
@@ -593,7 +634,7 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
     __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
     if (kGroup) settle_scales();
 #pragma unroll
-    for (int ck = 0; ck < 16; ck++) chunk(ck, 0, frag[0]);
+    for (int st = 0; st < 48; st++) stage(st, 0, frag[0]);
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
 #pragma unroll
@@ -612,14 +653,14 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
             h8 (&nxt)[8] = frag[(u + 1) & 1];
             auto hook = [&](auto blk, auto t) {
                 constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
-                constexpr int avail = 8 * MB - 8;                     // chunks go after the MFMAs of blocks >= 1
+                constexpr int avail = 8 * MB - 8;                     // stages go after the MFMAs of blocks >= 1
                 if constexpr (mslot == 8) {
                     if (next_group) settle_scales();
                 }
                 if constexpr (mslot >= 8) {
-                    constexpr int c0 = (mslot - 8) * 16 / avail, c1 = (mslot - 7) * 16 / avail;
+                    constexpr int s0 = (mslot - 8) * 48 / avail, s1 = (mslot - 7) * 48 / avail;
 #pragma unroll
-                    for (int ck = c0; ck < c1; ck++) chunk(ck, (u + 1) & 1, nxt);
+                    for (int st = s0; st < s1; st++) stage(st, (u + 1) & 1, nxt);
                 }
             };
             if ((u & 1) == 0) {
