@@ -23,6 +23,14 @@ template <int N>
 struct Int {
     static constexpr int value = N;
 };
+template <int I, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < END) {
+        f(Int<I>{});
+        static_for<I + 1, END>(f);
+    }
+}
 
 template <int OFF>
 __device__ __forceinline__ void lds_read_a4(uint32_t (&a)[4], const uint32_t (&addr)[4])
@@ -553,74 +561,91 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
             gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
         }
     };
-    // Dequantisation of one step's words, cut into 48 stages of two or three VALU instructions: stage = 3 * chunk +
-    // phase, chunk = 4j + 2*half + word being a quarter of one j group (two h2 of one packed word).  The caller places
-    // the stages after consecutive MFMAs, so that no MFMA is followed by more VALU work than its own passes cover (a
-    // wave that has its SIMD to itself hides two independent VALU instructions per MFMA completely, each further one
-    // costs four cycles; a whole chunk in one place is six to eight, most of them dependent on their predecessor).
-    // Every stage ties its inputs and results to its place in the program (empty asm statements), so the scheduler
-    // leaves it between the two MFMAs it was placed between.
-    h2 part[2];
-    uint32_t sx0 = 0, sx1 = 0;                             // the chunk in flight: between phase 0 and 1 ...
-    h2 sr0 = {(_Float16)0.f, (_Float16)0.f}, sr1 = sr0;    // ... and between phase 1 and 2
-    auto stage = [&](int st, int set, h8 (&frag)[8]) {
-        const int ck = st / 3, phase = st - 3 * ck;
-        const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
-        if (phase == 0) {
-            uint32_t q4 = wq[set][word][j];
-            asm volatile("" : "+v"(q4));
-            wq[set][word][j] = q4;
-            if (FP6) {
-                uint32_t t = tq[set][word][j >> 1];
-                asm volatile("" : "+v"(t));
-                tq[set][word][j >> 1] = t;
-                const uint32_t q2 = t << (4 * (j & 1));
-                const uint32_t lo = half == 0 ? (q4 >> 2) : (q4 << 2);
-                const uint32_t hi = half == 0 ? q2 : (q2 << 2);
-                sx0 = (hi & kc.top2) | (lo & ~kc.top2);                  // s eeemm xx in every byte
-                asm volatile("" : "+v"(sx0));
+    // Dequantisation of one step's words, written as asm statements of two instructions each and placed one by one
+    // after consecutive MFMAs.  Why asm: a wave issues one instruction of any kind every four cycles, so with a SIMD
+    // to itself it has three instruction slots per MFMA, and the empty asm statements that used to tie compiler-
+    // generated code to its place each cost an s_nop (the hazard recogniser assumes that an asm statement may have
+    // written its outputs with a sub-dword destination and separates it from the next reader): 2.2 s_nop per MFMA.
+    // A schedule entry works on a pair of chunks (the same (j, half) of the step's two k-blocks: words A and B) so
+    // that its two instructions are independent, and an entry's inputs come from the entry before the previous one.
+    //   INT4 entries: SHIFT (half 1 only)  ANDLO  ANDHI  SUB  FMA  [MUL0  MUL1 with group scales]
+    //   FP6 entries:  LO  HI (unless the shift is 0)  BFI  P8  ASHRA  ASHRB  ANDA  ANDB
+    constexpr int kEPP = FP6 ? 8 : (kGroup ? 7 : 5);      // entries per pair
+    constexpr int kEntries = 8 * kEPP;
+    uint32_t tA = 0, tB = 0, uA = 0, uB = 0, x0A = 0, x0B = 0, x1A = 0, x1B = 0, r0A = 0, r0B = 0, r1A = 0, r1B = 0;
+    const uint32_t b72 = vgpr_const(0xd480d480u);         // -72 (one scalar operand per instruction: the other constants)
+    auto entry = [&](auto e_tag, int set, h8 (&frag)[8]) {
+        constexpr int e = decltype(e_tag)::value;
+        constexpr int pr = e / kEPP, kind = e % kEPP, j = pr >> 1, half = pr & 1;
+        if constexpr (!FP6) {
+            if constexpr (kind == 0) {
+                if constexpr (half == 1)
+                    asm volatile("v_lshrrev_b32 %0, 8, %2\n\tv_lshrrev_b32 %1, 8, %3"
+                                 : "=&v"(tA), "=&v"(tB) : "v"(wq[set][0][j]), "v"(wq[set][1][j]));
+                else {
+                    tA = wq[set][0][j];
+                    tB = wq[set][1][j];
+                }
+            } else if constexpr (kind == 1) {
+                asm volatile("v_and_or_b32 %0, %2, %4, %5\n\tv_and_or_b32 %1, %3, %4, %5"
+                             : "=&v"(x0A), "=&v"(x0B) : "v"(tA), "v"(tB), "s"(0x000f000fu), "v"(kc.ex));
+            } else if constexpr (kind == 2) {
+                asm volatile("v_and_or_b32 %0, %2, %4, %5\n\tv_and_or_b32 %1, %3, %4, %5"
+                             : "=&v"(x1A), "=&v"(x1B) : "v"(tA), "v"(tB), "s"(0x00f000f0u), "v"(kc.ex));
+            } else if constexpr (kind == 3) {
+                asm volatile("v_pk_add_f16 %0, %2, %4\n\tv_pk_add_f16 %1, %3, %4"
+                             : "=&v"(r0A), "=&v"(r0B) : "v"(x0A), "v"(x0B), "s"(0xe408e408u));      // - 1032
+            } else if constexpr (kind == 4) {
+                asm volatile("v_pk_fma_f16 %0, %2, %4, %5\n\tv_pk_fma_f16 %1, %3, %4, %5"
+                             : "=&v"(r1A), "=&v"(r1B) : "v"(x1A), "v"(x1B), "s"(0x2c002c00u), "v"(b72));   // / 16 - 72
+            } else if constexpr (kind == 5) {
+                asm volatile("v_pk_mul_f16 %0, %0, %2\n\tv_pk_mul_f16 %1, %1, %2"
+                             : "+v"(r0A), "+v"(r0B) : "v"(gs_cur[2 * j + half]));
             } else {
-                const uint32_t q = half == 0 ? q4 : (q4 >> 8);
-                sx0 = (q & kc.lo) | kc.ex;
-                sx1 = (q & kc.hi) | kc.ex;
-                asm volatile("" : "+v"(sx0), "+v"(sx1));
-            }
-        } else if (phase == 1) {
-            asm volatile("" : "+v"(sx0), "+v"(sx1));
-            if (FP6) {
-                const s2 two = {2, 2};
-                sx1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, sx0 << 8) >> two);
-                sx0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s2, sx0) >> two);
-                asm volatile("" : "+v"(sx0), "+v"(sx1));
-            } else {
-                const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
-                const h2 mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};
-                const h2 bias_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-                sr0 = as_h2(sx0) - bias_lo;
-                sr1 = __builtin_elementwise_fma(as_h2(sx1), mul_hi, bias_hi);
-                asm volatile("" : "+v"(sr0), "+v"(sr1));
+                asm volatile("v_pk_mul_f16 %0, %0, %2\n\tv_pk_mul_f16 %1, %1, %2"
+                             : "+v"(r1A), "+v"(r1B) : "v"(gs_cur[2 * j + half]));
             }
         } else {
-            if (FP6) {
-                asm volatile("" : "+v"(sx0), "+v"(sx1));
-                sr0 = as_h2(sx0 & kc.exp_man);
-                sr1 = as_h2(sx1 & kc.exp_man);
-            } else {
-                asm volatile("" : "+v"(sr0), "+v"(sr1));
-                if (kGroup) {
-                    sr0 = sr0 * gs_cur[2 * j + half];
-                    sr1 = sr1 * gs_cur[2 * j + half];
+            constexpr int sh = 4 * (j & 1) + 2 * half;    // the 2-bit plane's field of this (j, half) to the top of every byte
+            if constexpr (kind == 0) {
+                if constexpr (half == 0)
+                    asm volatile("v_lshrrev_b32 %0, 2, %2\n\tv_lshrrev_b32 %1, 2, %3"
+                                 : "=&v"(tA), "=&v"(tB) : "v"(wq[set][0][j]), "v"(wq[set][1][j]));
+                else
+                    asm volatile("v_lshlrev_b32 %0, 2, %2\n\tv_lshlrev_b32 %1, 2, %3"
+                                 : "=&v"(tA), "=&v"(tB) : "v"(wq[set][0][j]), "v"(wq[set][1][j]));
+            } else if constexpr (kind == 1) {
+                if constexpr (sh != 0)
+                    asm volatile("v_lshlrev_b32 %0, %4, %2\n\tv_lshlrev_b32 %1, %4, %3"
+                                 : "=&v"(uA), "=&v"(uB) : "v"(tq[set][0][j >> 1]), "v"(tq[set][1][j >> 1]), "n"(sh));
+                else {
+                    uA = tq[set][0][j >> 1];
+                    uB = tq[set][1][j >> 1];
                 }
-            }
-            if (word == 0) {
-                part[0] = sr0;
-                part[1] = sr1;
-                asm volatile("" : "+v"(part[0]), "+v"(part[1]));
+            } else if constexpr (kind == 2) {             // s eeemm xx in every byte
+                asm volatile("v_bfi_b32 %0, %4, %2, %0\n\tv_bfi_b32 %1, %4, %3, %1"
+                             : "+v"(tA), "+v"(tB) : "v"(uA), "v"(uB), "s"(0xc0c0c0c0u));
+            } else if constexpr (kind == 3) {
+                asm volatile("v_lshlrev_b32 %0, 8, %2\n\tv_lshlrev_b32 %1, 8, %3" : "=&v"(x1A), "=&v"(x1B) : "v"(tA), "v"(tB));
+            } else if constexpr (kind == 4) {
+                asm volatile("v_pk_ashrrev_i16 %0, 2, %2 op_sel_hi:[0,1]\n\tv_pk_ashrrev_i16 %1, 2, %3 op_sel_hi:[0,1]"
+                             : "=&v"(x0A), "=&v"(x0B) : "v"(tA), "v"(tB));
+            } else if constexpr (kind == 5) {
+                asm volatile("v_pk_ashrrev_i16 %0, 2, %0 op_sel_hi:[0,1]\n\tv_pk_ashrrev_i16 %1, 2, %1 op_sel_hi:[0,1]"
+                             : "+v"(x1A), "+v"(x1B));
+            } else if constexpr (kind == 6) {
+                asm volatile("v_and_b32 %0, %4, %2\n\tv_and_b32 %1, %4, %3"
+                             : "=&v"(r0A), "=&v"(r0B) : "v"(x0A), "v"(x0B), "s"(0x9f009f00u));
             } else {
-                frag[2 * j + half] = join(part[0], part[1], sr0, sr1);
-                asm volatile("" : "+v"(frag[2 * j + half]));
+                asm volatile("v_and_b32 %0, %4, %2\n\tv_and_b32 %1, %4, %3"
+                             : "=&v"(r1A), "=&v"(r1B) : "v"(x1A), "v"(x1B), "s"(0x9f009f00u));
             }
         }
+        if constexpr (kind == kEPP - 1) frag[2 * j + half] = join(as_h2(r0A), as_h2(r1A), as_h2(r0B), as_h2(r1B));
+    };
+    auto entries = [&](auto first, auto last, int set, h8 (&frag)[8]) {
+        constexpr int e0 = decltype(first)::value, e1 = decltype(last)::value;
+        static_for<e0, e1>([&](auto e) { entry(e, set, frag); });
     };
 
     issue_a();                                            // pair 0
@@ -633,8 +658,7 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
     if (kGroup) fetch_scales(step_begin >> 2);
     __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
     if (kGroup) settle_scales();
-#pragma unroll
-    for (int st = 0; st < 48; st++) stage(st, 0, frag[0]);
+    entries(Int<0>{}, Int<kEntries>{}, 0, frag[0]);
 #pragma unroll 1
     for (int s = step_begin; s < step_end; s += kUnroll) {
 #pragma unroll
@@ -653,14 +677,13 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
             h8 (&nxt)[8] = frag[(u + 1) & 1];
             auto hook = [&](auto blk, auto t) {
                 constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
-                constexpr int avail = 8 * MB - 8;                     // stages go after the MFMAs of blocks >= 1
+                constexpr int avail = 8 * MB - 8;                     // the entries go after the MFMAs of blocks >= 1
                 if constexpr (mslot == 8) {
                     if (next_group) settle_scales();
                 }
                 if constexpr (mslot >= 8) {
-                    constexpr int s0 = (mslot - 8) * 48 / avail, s1 = (mslot - 7) * 48 / avail;
-#pragma unroll
-                    for (int st = s0; st < s1; st++) stage(st, (u + 1) & 1, nxt);
+                    constexpr int e0 = (mslot - 8) * kEntries / avail, e1 = (mslot - 7) * kEntries / avail;
+                    entries(Int<e0>{}, Int<e1>{}, (u + 1) & 1, nxt);
                 }
             };
             if ((u & 1) == 0) {
