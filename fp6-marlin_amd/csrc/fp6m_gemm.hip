@@ -879,11 +879,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             bool pair = a.m > 64;
             if (tune.pair != kUnset) pair = mb >= 4 && tune.pair != 0;
             if (mb == 8) {
-                void (*kernel)(const GemmArgs) = nullptr;
-                if (pair)
-                    kernel = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, true> : gemm_mb_kernel<false, 8, 3, 3, 4, true>;
-                else
-                    kernel = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, false> : gemm_mb_kernel<false, 8, 3, 3, 4, false>;
+                // (always the paired loop: the ring loop's 30 KiB per wave would fit, but it was slower at every size)
+                void (*kernel)(const GemmArgs) = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, true> : gemm_mb_kernel<false, 8, 3, 3, 4, true>;
                 hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, a);
             } else if (mb == 2) launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
             else if (pair) launch_mb<4, 3, 3, true>(a, g128, wk, grid, st);

@@ -107,6 +107,90 @@ __device__ __forceinline__ void dequant_half(uint32_t q2, uint32_t q4, int half,
     }
 }
 
+// Dequantisation of one step's words, written as asm statements of two instructions each that the loops place one by
+// one after consecutive MFMAs.  Why asm: a wave issues one instruction of any kind every four cycles, so with a SIMD
+// to itself it has three instruction slots per MFMA, and the empty asm statements that used to tie compiler-generated
+// code to its place each cost an s_nop (the hazard recogniser assumes that an asm statement may have written its
+// outputs with a sub-dword destination and separates it from the next reader): 2.2 s_nop per MFMA.  A schedule entry
+// works on a pair of chunks (the same (j, half) of the step's two k-blocks: words A and B) so that its two
+// instructions are independent, and an entry's inputs come from the entry before the previous one.
+//   INT4 entries: SHIFT (half 1 only)  ANDLO  ANDHI  SUB  FMA  [MUL0  MUL1 with group scales]
+//   FP6 entries:  LO  HI (unless the shift is 0)  BFI  P8  ASHRA  ASHRB  ANDA  ANDB
+// Entry E of a step: pair E / entries_per_pair (= 2j + half), kind E % entries_per_pair.  q4a / q4b: word j of the
+// 4-bit plane (INT4 words) of the two k-blocks; q2a / q2b: word j / 2 of the 2-bit plane; gs: the group scale of
+// columns (j, half) in both halves of a register.
+template <bool FP6, bool GROUP> constexpr int dequant_entries_per_pair() { return FP6 ? 8 : (GROUP ? 7 : 5); }
+struct DequantRegs {
+    uint32_t tA, tB, uA, uB, x0A, x0B, x1A, x1B, r0A, r0B, r1A, r1B;
+};
+template <bool FP6, bool GROUP, int E>
+__device__ __forceinline__ void dequant_entry(DequantRegs& d, uint32_t q4a, uint32_t q4b, uint32_t q2a, uint32_t q2b, h2 gs,
+                                              uint32_t ex, uint32_t b72, h8 (&frag)[8])
+{
+    constexpr int kEPP = dequant_entries_per_pair<FP6, GROUP>();
+    constexpr int pr = E / kEPP, kind = E % kEPP, j = pr >> 1, half = pr & 1;
+    if constexpr (!FP6) {
+        if constexpr (kind == 0) {
+            if constexpr (half == 1)
+                asm volatile("v_lshrrev_b32 %0, 8, %2\n\tv_lshrrev_b32 %1, 8, %3" : "=&v"(d.tA), "=&v"(d.tB) : "v"(q4a), "v"(q4b));
+            else {
+                d.tA = q4a;
+                d.tB = q4b;
+            }
+        } else if constexpr (kind == 1) {
+            asm volatile("v_and_or_b32 %0, %2, %4, %5\n\tv_and_or_b32 %1, %3, %4, %5"
+                         : "=&v"(d.x0A), "=&v"(d.x0B) : "v"(d.tA), "v"(d.tB), "s"(0x000f000fu), "v"(ex));
+        } else if constexpr (kind == 2) {
+            asm volatile("v_and_or_b32 %0, %2, %4, %5\n\tv_and_or_b32 %1, %3, %4, %5"
+                         : "=&v"(d.x1A), "=&v"(d.x1B) : "v"(d.tA), "v"(d.tB), "s"(0x00f000f0u), "v"(ex));
+        } else if constexpr (kind == 3) {
+            asm volatile("v_pk_add_f16 %0, %2, %4\n\tv_pk_add_f16 %1, %3, %4"
+                         : "=&v"(d.r0A), "=&v"(d.r0B) : "v"(d.x0A), "v"(d.x0B), "s"(0xe408e408u));            // - 1032
+        } else if constexpr (kind == 4) {
+            asm volatile("v_pk_fma_f16 %0, %2, %4, %5\n\tv_pk_fma_f16 %1, %3, %4, %5"
+                         : "=&v"(d.r1A), "=&v"(d.r1B) : "v"(d.x1A), "v"(d.x1B), "s"(0x2c002c00u), "v"(b72));   // / 16 - 72
+        } else if constexpr (kind == 5) {
+            asm volatile("v_pk_mul_f16 %0, %0, %2\n\tv_pk_mul_f16 %1, %1, %2" : "+v"(d.r0A), "+v"(d.r0B) : "v"(gs));
+        } else {
+            asm volatile("v_pk_mul_f16 %0, %0, %2\n\tv_pk_mul_f16 %1, %1, %2" : "+v"(d.r1A), "+v"(d.r1B) : "v"(gs));
+        }
+    } else {
+        constexpr int sh = 4 * (j & 1) + 2 * half;        // the 2-bit plane's field of this (j, half) to the top of every byte
+        if constexpr (kind == 0) {
+            if constexpr (half == 0)
+                asm volatile("v_lshrrev_b32 %0, 2, %2\n\tv_lshrrev_b32 %1, 2, %3" : "=&v"(d.tA), "=&v"(d.tB) : "v"(q4a), "v"(q4b));
+            else
+                asm volatile("v_lshlrev_b32 %0, 2, %2\n\tv_lshlrev_b32 %1, 2, %3" : "=&v"(d.tA), "=&v"(d.tB) : "v"(q4a), "v"(q4b));
+        } else if constexpr (kind == 1) {
+            if constexpr (sh != 0)
+                asm volatile("v_lshlrev_b32 %0, %4, %2\n\tv_lshlrev_b32 %1, %4, %3"
+                             : "=&v"(d.uA), "=&v"(d.uB) : "v"(q2a), "v"(q2b), "n"(sh));
+            else {
+                d.uA = q2a;
+                d.uB = q2b;
+            }
+        } else if constexpr (kind == 2) {                 // s eeemm xx in every byte
+            asm volatile("v_bfi_b32 %0, %4, %2, %0\n\tv_bfi_b32 %1, %4, %3, %1"
+                         : "+v"(d.tA), "+v"(d.tB) : "v"(d.uA), "v"(d.uB), "s"(0xc0c0c0c0u));
+        } else if constexpr (kind == 3) {
+            asm volatile("v_lshlrev_b32 %0, 8, %2\n\tv_lshlrev_b32 %1, 8, %3" : "=&v"(d.x1A), "=&v"(d.x1B) : "v"(d.tA), "v"(d.tB));
+        } else if constexpr (kind == 4) {
+            asm volatile("v_pk_ashrrev_i16 %0, 2, %2 op_sel_hi:[0,1]\n\tv_pk_ashrrev_i16 %1, 2, %3 op_sel_hi:[0,1]"
+                         : "=&v"(d.x0A), "=&v"(d.x0B) : "v"(d.tA), "v"(d.tB));
+        } else if constexpr (kind == 5) {
+            asm volatile("v_pk_ashrrev_i16 %0, 2, %0 op_sel_hi:[0,1]\n\tv_pk_ashrrev_i16 %1, 2, %1 op_sel_hi:[0,1]"
+                         : "+v"(d.x1A), "+v"(d.x1B));
+        } else if constexpr (kind == 6) {
+            asm volatile("v_and_b32 %0, %4, %2\n\tv_and_b32 %1, %4, %3"
+                         : "=&v"(d.r0A), "=&v"(d.r0B) : "v"(d.x0A), "v"(d.x0B), "s"(0x9f009f00u));
+        } else {
+            asm volatile("v_and_b32 %0, %4, %2\n\tv_and_b32 %1, %4, %3"
+                         : "=&v"(d.r1A), "=&v"(d.r1B) : "v"(d.x1A), "v"(d.x1B), "s"(0x9f009f00u));
+        }
+    }
+    if constexpr (kind == kEPP - 1) frag[2 * j + half] = join(as_h2(d.r0A), as_h2(d.r1A), as_h2(d.r0B), as_h2(d.r1B));
+}
+
 // A pair slot (two k steps of A): per 16-row block two loads of 8 rows x 128 bytes; the second lands 64 bytes
 // further than it would back to back, so that rows 8 .. 15 use the other half of the banks and a read of one
 // step's half-lines by all 16 rows is conflict-free.
@@ -302,36 +386,18 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
             gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
         }
     };
-    // A quarter of one j group (a "chunk": 4..8 VALU instructions): chunk = 4j + 2*half + word.  The
-    // word is tied to this point of the program first, the results after, so the instructions stay
-    // between the two MFMAs the chunk was placed between.
-    h2 part[2];
-    auto chunk = [&](int ck, int set, h8 (&frag)[8]) {
-        const int j = ck >> 2, half = (ck >> 1) & 1, word = ck & 1;
-        uint32_t q4 = word ? w.q1[j] : w.q0[j];
-        uint32_t q2 = 0;
-        asm volatile("" : "+v"(q4));
-        if (word) w.q1[j] = q4; else w.q0[j] = q4;
-        if (FP6) {
-            uint32_t t = tq[set][word][j >> 1];
-            asm volatile("" : "+v"(t));
-            tq[set][word][j >> 1] = t;
-            q2 = t << (4 * (j & 1));
-        }
-        h2 r0, r1;
-        dequant_half<FP6>(q2, q4, half, kc, r0, r1);
-        if (kGroup) {
-            r0 = r0 * gs_cur[2 * j + half];
-            r1 = r1 * gs_cur[2 * j + half];
-        }
-        if (word == 0) {
-            part[0] = r0;
-            part[1] = r1;
-            asm volatile("" : "+v"(part[0]), "+v"(part[1]));
-        } else {
-            frag[2 * j + half] = join(part[0], part[1], r0, r1);
-            asm volatile("" : "+v"(frag[2 * j + half]));
-        }
+    // Dequantisation: dequant_entry, one entry (or two) after each MFMA from the second block on.
+    constexpr int kEPP = dequant_entries_per_pair<FP6, kGroup>();
+    constexpr int kEntries = 8 * kEPP;
+    DequantRegs dq = {};
+    const uint32_t b72 = vgpr_const(0xd480d480u);         // -72
+    auto entries = [&](auto first, auto last, int set, h8 (&frag)[8]) {
+        constexpr int e0 = decltype(first)::value, e1 = decltype(last)::value;
+        static_for<e0, e1>([&](auto e) {
+            constexpr int E = decltype(e)::value, pr = E / kEPP, j = pr >> 1, half = pr & 1;
+            dequant_entry<FP6, kGroup, E>(dq, w.q0[j], w.q1[j], FP6 ? tq[set][0][j >> 1] : 0u, FP6 ? tq[set][1][j >> 1] : 0u,
+                                          kGroup ? gs_cur[2 * j + half] : h2{}, kc.ex, b72, frag);
+        });
     };
     auto slot_addrs = [&](uint32_t (&addr)[4], int slot) {
         const uint32_t so = slot * kSlot;
@@ -354,8 +420,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
     if (kGroup) fetch_scales(step_begin >> 2);
     __builtin_amdgcn_s_waitcnt(lgkmcnt_only(0));
     if (kGroup) settle_scales();
-#pragma unroll
-    for (int ck = 0; ck < 16; ck++) chunk(ck, 0, frag[0]);
+    entries(Int<0>{}, Int<kEntries>{}, 0, frag[0]);
     int slot_rd = 1;
     bool scales_in_flight = false;
 #pragma unroll 1
@@ -387,9 +452,8 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
                     if (next_group) settle_scales();
                 }
                 if constexpr (mslot >= 8) {
-                    constexpr int c0 = (mslot - 8) * 16 / avail, c1 = (mslot - 7) * 16 / avail;
-#pragma unroll
-                    for (int ck = c0; ck < c1; ck++) chunk(ck, (u + 1) & 1, nxt);
+                    constexpr int e0 = (mslot - 8) * kEntries / avail, e1 = (mslot - 7) * kEntries / avail;
+                    entries(Int<e0>{}, Int<e1>{}, (u + 1) & 1, nxt);
                 }
             };
             // (the LDS reads issued between A(1) and A(2): the words, and the group scales where a group starts)
@@ -561,91 +625,18 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
             gs_cur[t] = as_h2((gs_next[t] & 0xffffu) | (gs_next[t] << 16));
         }
     };
-    // Dequantisation of one step's words, written as asm statements of two instructions each and placed one by one
-    // after consecutive MFMAs.  Why asm: a wave issues one instruction of any kind every four cycles, so with a SIMD
-    // to itself it has three instruction slots per MFMA, and the empty asm statements that used to tie compiler-
-    // generated code to its place each cost an s_nop (the hazard recogniser assumes that an asm statement may have
-    // written its outputs with a sub-dword destination and separates it from the next reader): 2.2 s_nop per MFMA.
-    // A schedule entry works on a pair of chunks (the same (j, half) of the step's two k-blocks: words A and B) so
-    // that its two instructions are independent, and an entry's inputs come from the entry before the previous one.
-    //   INT4 entries: SHIFT (half 1 only)  ANDLO  ANDHI  SUB  FMA  [MUL0  MUL1 with group scales]
-    //   FP6 entries:  LO  HI (unless the shift is 0)  BFI  P8  ASHRA  ASHRB  ANDA  ANDB
-    constexpr int kEPP = FP6 ? 8 : (kGroup ? 7 : 5);      // entries per pair
+    // Dequantisation: dequant_entry, one entry after each MFMA from the second block on.
+    constexpr int kEPP = dequant_entries_per_pair<FP6, kGroup>();
     constexpr int kEntries = 8 * kEPP;
-    uint32_t tA = 0, tB = 0, uA = 0, uB = 0, x0A = 0, x0B = 0, x1A = 0, x1B = 0, r0A = 0, r0B = 0, r1A = 0, r1B = 0;
+    DequantRegs dq = {};
     const uint32_t b72 = vgpr_const(0xd480d480u);         // -72 (one scalar operand per instruction: the other constants)
-    auto entry = [&](auto e_tag, int set, h8 (&frag)[8]) {
-        constexpr int e = decltype(e_tag)::value;
-        constexpr int pr = e / kEPP, kind = e % kEPP, j = pr >> 1, half = pr & 1;
-        if constexpr (!FP6) {
-            if constexpr (kind == 0) {
-                if constexpr (half == 1)
-                    asm volatile("v_lshrrev_b32 %0, 8, %2\n\tv_lshrrev_b32 %1, 8, %3"
-                                 : "=&v"(tA), "=&v"(tB) : "v"(wq[set][0][j]), "v"(wq[set][1][j]));
-                else {
-                    tA = wq[set][0][j];
-                    tB = wq[set][1][j];
-                }
-            } else if constexpr (kind == 1) {
-                asm volatile("v_and_or_b32 %0, %2, %4, %5\n\tv_and_or_b32 %1, %3, %4, %5"
-                             : "=&v"(x0A), "=&v"(x0B) : "v"(tA), "v"(tB), "s"(0x000f000fu), "v"(kc.ex));
-            } else if constexpr (kind == 2) {
-                asm volatile("v_and_or_b32 %0, %2, %4, %5\n\tv_and_or_b32 %1, %3, %4, %5"
-                             : "=&v"(x1A), "=&v"(x1B) : "v"(tA), "v"(tB), "s"(0x00f000f0u), "v"(kc.ex));
-            } else if constexpr (kind == 3) {
-                asm volatile("v_pk_add_f16 %0, %2, %4\n\tv_pk_add_f16 %1, %3, %4"
-                             : "=&v"(r0A), "=&v"(r0B) : "v"(x0A), "v"(x0B), "s"(0xe408e408u));      // - 1032
-            } else if constexpr (kind == 4) {
-                asm volatile("v_pk_fma_f16 %0, %2, %4, %5\n\tv_pk_fma_f16 %1, %3, %4, %5"
-                             : "=&v"(r1A), "=&v"(r1B) : "v"(x1A), "v"(x1B), "s"(0x2c002c00u), "v"(b72));   // / 16 - 72
-            } else if constexpr (kind == 5) {
-                asm volatile("v_pk_mul_f16 %0, %0, %2\n\tv_pk_mul_f16 %1, %1, %2"
-                             : "+v"(r0A), "+v"(r0B) : "v"(gs_cur[2 * j + half]));
-            } else {
-                asm volatile("v_pk_mul_f16 %0, %0, %2\n\tv_pk_mul_f16 %1, %1, %2"
-                             : "+v"(r1A), "+v"(r1B) : "v"(gs_cur[2 * j + half]));
-            }
-        } else {
-            constexpr int sh = 4 * (j & 1) + 2 * half;    // the 2-bit plane's field of this (j, half) to the top of every byte
-            if constexpr (kind == 0) {
-                if constexpr (half == 0)
-                    asm volatile("v_lshrrev_b32 %0, 2, %2\n\tv_lshrrev_b32 %1, 2, %3"
-                                 : "=&v"(tA), "=&v"(tB) : "v"(wq[set][0][j]), "v"(wq[set][1][j]));
-                else
-                    asm volatile("v_lshlrev_b32 %0, 2, %2\n\tv_lshlrev_b32 %1, 2, %3"
-                                 : "=&v"(tA), "=&v"(tB) : "v"(wq[set][0][j]), "v"(wq[set][1][j]));
-            } else if constexpr (kind == 1) {
-                if constexpr (sh != 0)
-                    asm volatile("v_lshlrev_b32 %0, %4, %2\n\tv_lshlrev_b32 %1, %4, %3"
-                                 : "=&v"(uA), "=&v"(uB) : "v"(tq[set][0][j >> 1]), "v"(tq[set][1][j >> 1]), "n"(sh));
-                else {
-                    uA = tq[set][0][j >> 1];
-                    uB = tq[set][1][j >> 1];
-                }
-            } else if constexpr (kind == 2) {             // s eeemm xx in every byte
-                asm volatile("v_bfi_b32 %0, %4, %2, %0\n\tv_bfi_b32 %1, %4, %3, %1"
-                             : "+v"(tA), "+v"(tB) : "v"(uA), "v"(uB), "s"(0xc0c0c0c0u));
-            } else if constexpr (kind == 3) {
-                asm volatile("v_lshlrev_b32 %0, 8, %2\n\tv_lshlrev_b32 %1, 8, %3" : "=&v"(x1A), "=&v"(x1B) : "v"(tA), "v"(tB));
-            } else if constexpr (kind == 4) {
-                asm volatile("v_pk_ashrrev_i16 %0, 2, %2 op_sel_hi:[0,1]\n\tv_pk_ashrrev_i16 %1, 2, %3 op_sel_hi:[0,1]"
-                             : "=&v"(x0A), "=&v"(x0B) : "v"(tA), "v"(tB));
-            } else if constexpr (kind == 5) {
-                asm volatile("v_pk_ashrrev_i16 %0, 2, %0 op_sel_hi:[0,1]\n\tv_pk_ashrrev_i16 %1, 2, %1 op_sel_hi:[0,1]"
-                             : "+v"(x1A), "+v"(x1B));
-            } else if constexpr (kind == 6) {
-                asm volatile("v_and_b32 %0, %4, %2\n\tv_and_b32 %1, %4, %3"
-                             : "=&v"(r0A), "=&v"(r0B) : "v"(x0A), "v"(x0B), "s"(0x9f009f00u));
-            } else {
-                asm volatile("v_and_b32 %0, %4, %2\n\tv_and_b32 %1, %4, %3"
-                             : "=&v"(r1A), "=&v"(r1B) : "v"(x1A), "v"(x1B), "s"(0x9f009f00u));
-            }
-        }
-        if constexpr (kind == kEPP - 1) frag[2 * j + half] = join(as_h2(r0A), as_h2(r1A), as_h2(r0B), as_h2(r1B));
-    };
     auto entries = [&](auto first, auto last, int set, h8 (&frag)[8]) {
         constexpr int e0 = decltype(first)::value, e1 = decltype(last)::value;
-        static_for<e0, e1>([&](auto e) { entry(e, set, frag); });
+        static_for<e0, e1>([&](auto e) {
+            constexpr int E = decltype(e)::value, pr = E / kEPP, j = pr >> 1, half = pr & 1;
+            dequant_entry<FP6, kGroup, E>(dq, wq[set][0][j], wq[set][1][j], FP6 ? tq[set][0][j >> 1] : 0u,
+                                          FP6 ? tq[set][1][j >> 1] : 0u, kGroup ? gs_cur[2 * j + half] : h2{}, kc.ex, b72, frag);
+        });
     };
 
     issue_a();                                            // pair 0

@@ -167,7 +167,7 @@ def test_eight_row_blocks_per_wave(oracle):
     """The m > 16 kernel with eight 16-row blocks per wave (128-row tiles, accumulators in the accumulation
     registers), forced onto small problems: ragged row tiles, both regions, both scale modes, k splits through the
     scratch, several launches, and one-hot rows bit for bit."""
-    for pair in (0, 1):                                                 # ring loop / paired activation fetch (INT4 tiles)
+    for pair in (1,):                                                   # (eight blocks always fetch A by pairs of steps)
         e = {"FP6M_MB": 8, "FP6M_WM": 0, "FP6M_PAIR": pair}
         for m in (17, 100, 128, 129, 300):
             run(oracle, m, 512, 1024, qc=256, gs=128, env=e)
