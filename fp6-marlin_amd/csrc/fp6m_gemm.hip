@@ -485,14 +485,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     const Tuning tune = g_tuning;              // tuning/testing overrides (all unset in production)
     if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4 || tune.mb == 8)) mb = tune.mb;
-    // Launches of 1024 rows on the largest weights: four 64-row tiles share the dequantised fragments of a tile
-    // (gemm_wm_kernel), two column tiles per workgroup.  Measured on MI355X it beats the 128-row tiles of the
-    // private-fragment kernel (below) by 5 % on 8192 x 16384 (262 vs 277 us at m = 1024), equals them on 8192 x 28672
-    // and loses on smaller weights (8192 x 8192: 146 vs 137 us) and below 1024 rows, where its 256-row workgroups
-    // leave CUs idle.
-    const long long rows_per_launch = prob_m < 64LL * max_par ? prob_m : 64LL * max_par;
+    // gemm_wm_kernel (four 64-row tiles share the dequantised fragments of a tile through LDS) was the kernel of launches
+    // of 1024 rows and more until the 128-row tiles of the private-fragment kernel (below) got their dequantisation as
+    // asm: those now measure 1-5 % faster on every large shape (m = 1024: 8192 x 16384 268 vs 272 us, 8192 x 28672
+    // 483 vs 507, 16384 x 16384 504 vs 527, 8192 x 57344 957 vs 1006).  It stays reachable through the tuning hook.
     const long long weights = (long long)prob_n * prob_k;
-    bool shared_frags = rows_per_launch >= 1024 && weights >= (128LL << 20);
+    bool shared_frags = false;
     if (tune.wm != kUnset) shared_frags = prob_m > 16 && tune.wm != 0;
     if (row_mix) shared_frags = false;                                // its waves run in lock step on one segment
     // Row mix: the kWaves * ks slices of a tile are dealt to the two segments in proportion to their cost (an FP6
