@@ -22,9 +22,10 @@
 //    (a rule plus a small cost model fitted to per-workgroup timelines on MI355X).
 //
 // gemm_common.h  argument block, tile bookkeeping, load / wait / dequantisation helpers
+// gemm_sk.h      gemm_sk_kernel (one row: the decode kernel)
 // gemm_m16.h     gemm_m16_kernel (m <= 16)
 // gemm_mb.h      gemm_mb_kernel (16 < m)
-// gemm_wm.h      gemm_wm_kernel (launches of >= 1024 rows on large weights)
+// gemm_wm.h      gemm_wm_kernel (fragments shared by four row tiles; superseded, reachable through the tuning hook)
 // this file      activation gather, per-device scratch, dispatch and the extern "C" entry points
 #include <hip/hip_runtime.h>
 

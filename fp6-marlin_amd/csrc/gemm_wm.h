@@ -1,4 +1,5 @@
-// gemm_wm_kernel: the large-m kernel of fp6m_gemm.hip (four row tiles share a tile's dequantised fragments).
+// gemm_wm_kernel: a large-m kernel of fp6m_gemm.hip (four row tiles share a tile's dequantised fragments); the
+// dispatcher prefers the 128-row tiles of gemm_mb.h, this one is reached through the tuning hook.
 // Uses the MFMA, A-ring and epilogue pieces of gemm_mb.h.
 #pragma once
 #include "gemm_mb.h"
