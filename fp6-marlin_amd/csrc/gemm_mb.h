@@ -7,10 +7,12 @@ namespace fp6m {
 // ------------------------------------------------------------------------------------------------ 16 < m: ring kernel with MB row blocks
 //
 // Same lane routing and k-sliced workgroup as the m <= 16 kernel, but a wave multiplies MB blocks of 16 rows of A and
-// every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per 16*MB rows.  Two
-// loops: stream_tile_mb keeps the words and one step of A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (INT4
-// tiles of launches with more than 64 rows) fetches A a pair of steps at a time and the words through registers.
-// A workgroup is one tile x four or eight k slices; blockIdx.y walks the row tiles.  Group scales are
+// every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per 16*MB rows.  MB = 2 or
+// 4 (accumulators in ordinary registers, two waves per SIMD) or 8 (accumulators in the accumulation registers, one
+// wave per SIMD; launches whose 128-row tiles fill the chip).  Two loops: stream_tile_mb keeps the words and one step of
+// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 64 rows: the INT4 tiles, with MB = 8 the
+// FP6 tiles too) fetches A a pair of steps at a time and the words through registers.  Both dequantise through
+// dequant_entry.  A workgroup is one tile x four or eight k slices; blockIdx.y walks the row tiles.  Group scales are
 // applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more
 // registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
 // the number of direct-to-LDS loads per step is constant) and never stored.
@@ -447,7 +449,7 @@ __device__ __forceinline__ void stream_tile_mb(const GemmArgs& p, const TileInfo
             h8 (&nxt)[8] = frag[(u + 1) & 1];
             auto hook = [&](auto blk, auto t) {
                 constexpr int mslot = decltype(blk)::value * 8 + decltype(t)::value;   // MFMA just issued
-                constexpr int avail = 8 * MB - 8;                     // chunks go after the MFMAs of blocks >= 1
+                constexpr int avail = 8 * MB - 8;                     // the entries go after the MFMAs of blocks >= 1
                 if constexpr (mslot == 8) {
                     if (next_group) settle_scales();
                 }
