@@ -938,7 +938,9 @@ __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb
         }
     }
     FP6M_MARK(p, 2);
-    constexpr int BPR = kWaveLds >= 2 * 16 * kRedStride * 4 ? 2 : 1;  // the drained rings hold two blocks per wave
+    // the drained rings hold two blocks per wave; four in the eight-block kernel, which has the registers for a round
+    // of that size (half the barriers: 139 -> 135 us at m = 1024 on 8192 x 8192)
+    constexpr int BPR = (MB > 4 && kWaveLds >= 4 * 16 * kRedStride * 4) ? 4 : (kWaveLds >= 2 * 16 * kRedStride * 4 ? 2 : 1);
     wg_finish_mb<MB, WK, BPR>(p, ti, wave, ks, slot_base, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
                          reinterpret_cast<int*>(smem + WK * kWaveLds), true, p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
