@@ -184,14 +184,17 @@ def test_eight_row_blocks_per_wave(oracle):
 
 
 def test_dispatch_picks_128_row_tiles_where_they_fill_the_chip(oracle, capfd):
-    """The dispatcher's own choice: 128-row tiles for launches of more than 256 rows whose workgroups fill their rounds
-    of one per CU (here 32 column tiles x 8 row tiles = 256 workgroups, the last row tile ragged), 64-row tiles where
-    they do not (9 row tiles: 288 workgroups, two rounds at 56 %)."""
-    for m, want in ((1000, "MB=8"), (1024, "MB=8"), (1025, "MB=4"), (300, "MB=4")):
+    """The dispatcher's own choice between 128-row tiles (one workgroup per CU, whole rounds) and 64-row tiles (a third
+    slower per row, finer grain): with 32 column tiles, 8 row tiles of 128 fill one round of 256 CUs exactly (the last
+    tile ragged at m = 1000) and 5 of them beat 10 half-size workgroups that no longer fit one per CU; 9 row tiles
+    would take two rounds for 1.1 rounds of work, and at m = 300 the 64-row tiles still fit one per CU.  With 256
+    column tiles even a single, ragged row tile of 128 wins (one round instead of 512 half-size workgroups)."""
+    for m, n, want in ((1000, 4096, "MB=8"), (1024, 4096, "MB=8"), (640, 4096, "MB=8"), (1025, 4096, "MB=4"),
+                       (300, 4096, "MB=4"), (96, 32768, "MB=8"), (96, 4096, "MB=4"), (64, 32768, "MB=4")):
         capfd.readouterr()
-        run(oracle, m, 4096, 512, qc=256, gs=128, env={"FP6M_VERBOSE": 1})
+        run(oracle, m, n, 512, qc=256, gs=128, env={"FP6M_VERBOSE": 1})
         err = capfd.readouterr().err
-        assert want in err, (m, want, err[-400:])
+        assert want in err, (m, n, want, err[-400:])
 
 
 def test_eight_k_slices_per_workgroup(oracle):
