@@ -515,3 +515,53 @@ def test_dispatcher_choices_over_many_shapes(oracle):
             assert int(ws.abs().sum().item()) == 0
         del w, Bd, sd
         torch.cuda.empty_cache()
+
+
+def test_random_shapes_rows_and_limits_against_unpacked_words(oracle):
+    """A seeded random walk over what the dispatcher can be asked: k and n in multiples of 256 (up to 8192 x 8192
+    weights), any multiple of 128 FP6 columns including none and all, both scale modes, 1 .. 1500 rows, `max_par`
+    16 .. 1 (several launches), `sms` limits.  Random packed words against the pinned unpacker and an fp32 matmul:
+    the relative-error bar on each region, an element-wise bound so that nothing hides in a mean, C fully written,
+    two calls bit-identical, the workspace left zero."""
+    import random
+    import fp6_marlin
+    rnd = random.Random(11)
+    g = torch.Generator().manual_seed(11)
+    for ci in range(120):
+        k = 256 * rnd.choice([1, 2, 3, 4, 6, 8, 11, 16, 20, 32])
+        n = 256 * rnd.choice([1, 2, 3, 5, 8, 13, 16, 24, 32, 43, 64, 112])
+        if k * n > 8192 * 8192:
+            n = 2048
+        qc = min(n, rnd.choice([0, 256, 256, 256, 512, n, 128, 384]))
+        gs = rnd.choice([-1, 128])
+        m = rnd.choice([rnd.randint(1, 16), rnd.randint(17, 64), rnd.randint(65, 300), rnd.randint(300, 1500), 64, 128, 129, 256, 1024])
+        max_par = rnd.choice([16, 16, 16, 8, 2, 1])
+        sms = rnd.choice([-1, -1, -1, 1, 2, 7, 64])
+        n4 = n - qc
+        B = torch.randint(-2 ** 31, 2 ** 31 - 1, (k * n4 // 8 + k * qc * 3 // 16,), generator=g, dtype=torch.int64).to(torch.int32)
+        s = (torch.rand(((k // gs) * n4 if gs > 0 else n4) + qc, generator=g) * 0.01 + 0.001).half()
+        qarg = qc if qc else -1
+        print(f"case random {ci} m={m} k={k} n={n} qc={qc} gs={gs} max_par={max_par} sms={sms}", flush=True)
+        w = fp6_marlin.unpack_to_fp16(B, s, k, n, qarg, gs).to(dev())
+        Bd, sd = B.to(dev()), s.to(dev())
+        ws = torch.zeros(n // 128 * max_par, dtype=torch.int32, device=dev())
+        a = torch.randn((m, k), generator=g).half().to(dev())
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        C2 = torch.full_like(C, float("nan"))
+        for out in (C, C2):
+            fp6_marlin.mul(a, Bd, out, sd, ws, qarg, -1, -1, sms, max_par, gs)
+            torch.cuda.synchronize()
+        case = (ci, m, k, n, qc, gs, max_par, sms)
+        assert torch.isfinite(C).all(), case
+        assert torch.equal(C, C2), case
+        assert int(ws.abs().sum().item()) == 0, case
+        ref = a.float() @ w.float()
+        for sl in (slice(0, n4), slice(n4, n)):
+            if sl.stop > sl.start:
+                r = ref[:, sl]
+                d = (C[:, sl].float() - r).abs()
+                assert (d.mean() / r.abs().mean()).item() <= TOL, case
+                # fp16 rounding of the result plus the accumulation order: far below a wrong or missing k step
+                assert bool((d <= 4e-3 * r.abs() + 0.13 * r.abs().mean()).all()), case
+        del w, Bd, sd, a, C, C2, ref
+        torch.cuda.empty_cache()
