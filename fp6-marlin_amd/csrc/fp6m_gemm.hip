@@ -68,7 +68,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -322,7 +322,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -455,6 +455,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.s_fp6 = a.s_int4 + (g128 ? (size_t)(prob_k / 128) * n4 : (size_t)n4);
     a.scratch = fixed_scratch ? device->static_scratch : region->partials;
     a.counters = static_cast<int*>(workspace);
+    a.cells = nullptr;
     a.n = prob_n;
     a.k = prob_k;
     a.n4 = n4;
@@ -813,6 +814,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.ks6 = (int)ks6_of(ks, cfg.wk);
             if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
             a.ksplit = a.ks4;
+            // Up to four rows, shared tiles meet in cells (one returning atomic per element and workgroup) instead of
+            // being published, counted and gathered: one round trip after the loop instead of three (4096 x 4096 at two
+            // rows 8.1 -> 7.0 us, 11008 x 4096 11.1 -> 10.1, 8192 x 8192 12.2 -> 11.6; even at four rows; the atomics of
+            // eight and sixteen rows cost more than the round trips: 4096 x 4096 at sixteen rows 9.3 -> 10.3 us).
+            const bool want_cells = tune.cells != kUnset ? tune.cells != 0 : a.m <= 4;
+            if (want_cells && (size_t)prob_n * 16 * sizeof(unsigned long long) <= kCellBytes && a.ks4 <= kMaxParts &&
+                a.ks6 <= kMaxParts)
+                a.cells = reinterpret_cast<unsigned long long*>(reinterpret_cast<unsigned char*>(a.scratch) + scratch_bytes);
             if (row_mix) {
                 a.ks6 = 0;                                            // no FP6 column region: groups6 is 0
                 a.slices4 = deal_slices(a.ks4 * cfg.wk);

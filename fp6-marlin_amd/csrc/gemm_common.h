@@ -78,6 +78,7 @@ struct GemmArgs {
     const uint16_t* bias;     // fp16 [n], indexed by C column
     const uint16_t* residual; // fp16 [m, n], same rows as C
     int fused;
+    unsigned long long* cells;   // m <= 16: the shared tiles' parts meet here instead of in `scratch` (null: they do not)
 #ifdef FP6M_TIMELINE
     unsigned long long* timeline;   // 8 realtime-clock stamps per workgroup (performance debugging builds only)
 #endif
@@ -119,7 +120,7 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int total)
 __device__ __forceinline__ void preload_args(const GemmArgs& p)
 {
     asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
-                        "s"(p.scratch), "s"(p.counters));
+                        "s"(p.scratch), "s"(p.counters), "s"(p.cells));
     asm volatile("" : : "s"(p.m), "s"(p.n), "s"(p.k), "s"(p.n4), "s"(p.qc), "s"(p.tiles6), "s"(p.tiles), "s"(p.ksplit),
                         "s"(p.ks6), "s"(p.ks4), "s"(p.groups6), "s"(p.groups4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
     asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
@@ -177,6 +178,35 @@ __device__ __forceinline__ void store_fused_one(const Args& p, const FusedCols& 
     if (p.residual) v += (float)__builtin_bit_cast(_Float16, p.residual[at]);
     p.C[at] = __builtin_bit_cast(uint16_t, (_Float16)v);
 }
+
+// ------------------------------------------------------------------------------------------------ cells
+// One 64-bit cell per output element of a tile that several waves or workgroups share: every part adds
+//         2^56  +  2^47  +  round(value * 2^29)            (count | biased fixed-point value, |value| < 2^17)
+// with one returning agent-scope atomic; whoever reads back count == parts - 1 holds the complete sum.
+constexpr int kCellFracBits = 29;
+constexpr unsigned long long kCellBias = 1ull << 47;        // makes every part's contribution positive
+constexpr unsigned long long kCellOne = 1ull << 56;         // the arrival count sits above the sum
+constexpr unsigned long long kCellSumMask = kCellOne - 1;
+constexpr int kMaxParts = 255;                              // 255 * (2^47 + 2^46) < 2^56
+constexpr size_t kCellBytes = size_t(8) << 20;              // cells of one workspace: n * m * 8 bytes at most
+
+
+__device__ __forceinline__ unsigned long long cell_contribution(float x)
+{
+    const float lim = 131071.0f;
+    float y = x < lim ? x : lim;                            // (NaN compares false: it saturates high)
+    y = y > -lim ? y : -lim;
+    const long long f = (long long)(y * (float)(1ll << kCellFracBits));
+    return kCellOne + kCellBias + (unsigned long long)f;
+}
+
+// The complete sum as a float: `old` is what the atomic returned, `mine` what this wave added.
+__device__ __forceinline__ float cell_total(unsigned long long old, unsigned long long mine, int parts)
+{
+    const unsigned long long sum = ((old + mine) & kCellSumMask) - (unsigned long long)parts * kCellBias;
+    return (float)(long long)sum * (1.0f / (float)(1ll << kCellFracBits));
+}
+
 
 // ------------------------------------------------------------------------------------------------ tile bookkeeping
 

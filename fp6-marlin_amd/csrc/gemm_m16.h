@@ -375,6 +375,41 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
         return;
     }
 
+    if (p.cells) {
+        // The parts of the tile meet in its cells (see gemm_common.h): one returning atomic per element, values in output
+        // units; whoever arrives last at an element stores it and writes its cell back to zero.  Nothing is published,
+        // counted or gathered, and no barrier follows the sum through LDS.
+        unsigned long long* cell = p.cells + (size_t)ti.tile * (16 * kTileN) + lane;   // [row][64 even | 64 odd columns]
+        unsigned long long old[RMAX][2];
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            const int m = wk + r * WK;
+            v0[r] *= s0;
+            v1[r] *= s1;
+            if (tile_valid && m < nrows) {
+                old[r][0] = __hip_atomic_fetch_add(cell + m * kTileN, cell_contribution(v0[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                old[r][1] = __hip_atomic_fetch_add(cell + m * kTileN + 64, cell_contribution(v1[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) {
+            const int m = wk + r * WK;
+            if (!(tile_valid && m < nrows)) continue;
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                if ((int)(old[r][e] >> 56) != ks - 1) continue;              // somebody else arrives last at this element
+                const float v = cell_total(old[r][e], cell_contribution(e ? v1[r] : v0[r]), ks);
+                __hip_atomic_store(cell + m * kTileN + 64 * e, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (p.fused)
+                    store_fused_one(p, fcols, (size_t)m, e, v);
+                else
+                    c_out[(size_t)m * p.n + e] = __builtin_bit_cast(uint16_t, (_Float16)v);
+            }
+        }
+        FP6M_MARK(p, 6);
+        return;
+    }
+
     // Publish.  A slot holds [WN tiles][16 rows][128 columns] fp32; 8-byte agent-scope accesses.
     constexpr size_t kSlotU64 = (size_t)WN * 16 * kTileN / 2;
     unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) + (size_t)slot_base * kSlotU64 +

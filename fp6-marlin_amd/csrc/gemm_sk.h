@@ -36,13 +36,6 @@ namespace fp6m {
 // fp16's; a part that is not finite or is out of range saturates, which makes the element infinite.  The cells
 // live in the scratch region that belongs to the call's workspace, are zero when no call is in flight, and are left
 // zero.
-constexpr int kCellFracBits = 29;
-constexpr unsigned long long kCellBias = 1ull << 47;        // makes every part's contribution positive
-constexpr unsigned long long kCellOne = 1ull << 56;         // the arrival count sits above the sum
-constexpr unsigned long long kCellSumMask = kCellOne - 1;
-constexpr int kMaxParts = 255;                              // 255 * (2^47 + 2^46) < 2^56
-constexpr size_t kCellBytes = size_t(8) << 20;              // cells of one workspace: n * m * 8 bytes at most
-
 // Kernel arguments, laid out as three 64-byte blocks and a 16-byte one that the kernel fetches itself with four
 // scalar loads behind one wait (left to the compiler, the loads of the fields come in several dependent batches, each a
 // round trip to a cold line before the wave's first weight load).
@@ -118,22 +111,6 @@ __device__ __forceinline__ SkArgs load_sk_args()
 __device__ __forceinline__ uint32_t mul_shift40(unsigned long long magic, uint32_t n)
 {
     return (uint32_t)(((unsigned long long)n * magic) >> 40);
-}
-
-__device__ __forceinline__ unsigned long long cell_contribution(float x)
-{
-    const float lim = 131071.0f;
-    float y = x < lim ? x : lim;                            // (NaN compares false: it saturates high)
-    y = y > -lim ? y : -lim;
-    const long long f = (long long)(y * (float)(1ll << kCellFracBits));
-    return kCellOne + kCellBias + (unsigned long long)f;
-}
-
-// The complete sum as a float: `old` is what the atomic returned, `mine` what this wave added.
-__device__ __forceinline__ float cell_total(unsigned long long old, unsigned long long mine, int parts)
-{
-    const unsigned long long sum = ((old + mine) & kCellSumMask) - (unsigned long long)parts * kCellBias;
-    return (float)(long long)sum * (1.0f / (float)(1ll << kCellFracBits));
 }
 
 // A shared tile's elements this wave has added to and not yet looked at: the atomics' results come back while the
