@@ -730,8 +730,13 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     // barriers each, so fewer rounds help; the gather below keeps the loads of up to 32 rows in flight per lane.
     static_assert(MB % BPR == 0, "whole rounds");
     constexpr int RMAX = 16 / WK;                                    // rows of a block one wave finishes
-    constexpr int MBC = MB < (32 / RMAX > 0 ? 32 / RMAX : 1) ? MB : (32 / RMAX > 0 ? 32 / RMAX : 1);   // blocks per gather round
-    constexpr int PCH = 32 / (MBC * RMAX) > 0 ? 32 / (MBC * RMAX) : 1;                                 // parts per gather round
+    // The gather keeps up to 32 8-byte loads per lane in flight.
+    constexpr int kInFlight = 32;
+    // (shared tiles) this workgroup's own sums stay in registers where there are few enough of them: if it turns out to
+    // arrive last it takes them from there, in their place in the part order, instead of loading them back
+    constexpr bool kKeep = MB * RMAX <= 32;
+    constexpr int MBC = MB < kInFlight / RMAX ? MB : kInFlight / RMAX;                                 // blocks per gather round
+    constexpr int PCH = kInFlight / (MBC * RMAX) > 0 ? kInFlight / (MBC * RMAX) : 1;                   // parts per gather round
     typedef float f2 __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x & 63;
     const bool leader = lane == 0 && wk == 0;
@@ -767,6 +772,7 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) + (size_t)slot_base * kSlotU64 + lane;
     unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
 
+    float keep0[kKeep ? MB : 1][RMAX], keep1[kKeep ? MB : 1][RMAX];
 #pragma unroll
     for (int mb0 = 0; mb0 < MB; mb0 += BPR) {
         __syncthreads();
@@ -807,6 +813,10 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
                         v1 += j >= first_fp6 ? tv[b][r][j][1] * x1 : tv[b][r][j][1];
                     }
                 }
+                if constexpr (kKeep) {
+                    keep0[mb0 + b][r] = v0;
+                    keep1[mb0 + b][r] = v1;
+                }
                 if (row < nrows) {
                     if (ks == 1) {
                         store_row(row, v0, v1);
@@ -838,7 +848,7 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
     FP6M_MARK(p, 5);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     // The last arrival sums all parts in part order: MBC blocks at a time, PCH parts' loads in flight together.
-#pragma unroll 1
+#pragma unroll
     for (int mb0 = 0; mb0 < MB; mb0 += MBC) {
         float v0[MBC][RMAX], v1[MBC][RMAX];
 #pragma unroll
@@ -858,7 +868,7 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
                     for (int r = 0; r < RMAX; r++) {
                         const int row = 16 * (mb0 + b) + wk + r * WK;
                         t[u][b][r] = 0;
-                        if (row < nrows && pp + u < ks)
+                        if (row < nrows && pp + u < ks && !(kKeep && pp + u == ti.part))
                             t[u][b][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + (size_t)row * (kTileN / 2),
                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
@@ -869,8 +879,9 @@ __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& 
 #pragma unroll
                     for (int r = 0; r < RMAX; r++) {
                         const f2 v = __builtin_bit_cast(f2, t[u][b][r]);
-                        v0[b][r] += v[0];
-                        v1[b][r] += v[1];
+                        const bool own = kKeep && pp + u == ti.part;   // (uniform) the bits that were stored, from registers
+                        v0[b][r] += own ? keep0[kKeep ? mb0 + b : 0][r] : v[0];
+                        v1[b][r] += own ? keep1[kKeep ? mb0 + b : 0][r] : v[1];
                     }
         }
 #pragma unroll
