@@ -869,7 +869,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.ks4 = (int)ks;
             a.ks6 = (int)ks;
             const long long resident = (long long)cus * (wk == 8 || mb == 8 ? 1 : 2);
-            if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk &&
+            // (Not for 128-row tiles, whose FP6 workgroups are only a few per cent behind: there the second partner's
+            // partial tiles cost more than the shorter loop gains, 8192 x 8192 at m = 384 61.8 vs 58.4 us.)
+            if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk && mb != 8 &&
                 (base + (long long)a.tiles6 * mtiles) * ks <= resident)
                 a.ks6 = 2 * (int)ks;
             if (row_mix) {
@@ -887,9 +889,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (tune.verbose)
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks4=%d ks6=%d k slices %d grid=%ux%u\n", a.m, prob_n,
                         prob_k, mb, mtiles, a.ks4, a.ks6, wk, grid.x, grid.y);
-            // From two row tiles on, the requests A costs weigh more than the shorter look-ahead of the paired fetch
-            // (measured: 64 rows 1-3 % slower with it, 128 rows 0-8 % faster, 256 and 512 rows 4-14 %).
-            bool pair = a.m > 64;
+            // Every launch of 64-row tiles takes the paired loop (33 rows: -5 % .. +5 % over five shapes, 40 rows 0-9 % faster,
+            // 64 rows 9-16 %, from 65 rows on 12-20 %; before the FP6 tiles had it too, whose workgroups set a resident
+            // grid's length, it paid from 65 rows on only).  The ring loop stays for 32-row tiles and the tuning hook.
+            bool pair = true;
             if (tune.pair != kUnset) pair = mb >= 4 && tune.pair != 0;
             if (mb == 8) {
                 // (always the paired loop: the ring loop's 30 KiB per wave would fit, but it was slower at every size)

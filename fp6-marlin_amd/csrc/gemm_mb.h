@@ -10,8 +10,8 @@ namespace fp6m {
 // every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per 16*MB rows.  MB = 2 or
 // 4 (accumulators in ordinary registers, two waves per SIMD) or 8 (accumulators in the accumulation registers, one
 // wave per SIMD; launches whose 128-row tiles fill the chip).  Two loops: stream_tile_mb keeps the words and one step of
-// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 64 rows: the INT4 tiles, with MB = 8 the
-// FP6 tiles too) fetches A a pair of steps at a time and the words through registers.  Both dequantise through
+// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 64 rows) fetches A a pair of steps at a
+// time and the words through registers.  Both dequantise through
 // dequant_entry.  A workgroup is one tile x four or eight k slices; blockIdx.y walks the row tiles.  Group scales are
 // applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more
 // registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
@@ -903,11 +903,13 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 
 // WK = k slices (waves) per workgroup: four, or eight (one workgroup per CU, two waves per SIMD) for grids that
 // would otherwise leave every SIMD a single wave.
-// PAIR: the INT4 tiles fetch A by pairs of steps and their words through registers (stream_tile_mbp).
+// PAIR: A is fetched by pairs of steps and the words through registers (stream_tile_mbp).
 template <bool G128, int MB, int D4, int D6, int WK, bool PAIR>
 __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
 {
-    // (FP6 tiles keep the ring: with the 2-bit plane's registers on top, the paired loop no longer fits 256 VGPRs.)
+    // FP6 tiles take the paired loop too: with the dequantisation as asm statements it fits 256 VGPRs with the 2-bit
+    // plane's registers on top, and in a grid that is resident all at once the few FP6 workgroups set the length of
+    // the launch (8192 x 8192 with 256 FP6 columns: m = 128 31.8 -> 27.1 us, m = 256 47.0 -> 40.3).
     constexpr bool kPaired = PAIR;
     static_assert(!PAIR || MB == 4 || MB == 8, "stream_tile_mbp is written for whole rounds of the four A buffers");
     constexpr int kWaveLds = kPaired ? max3(mbp_wave_lds(MB), mb_wave_lds(MB, 0, D6), 0) : mb_wave_lds(MB, D4, D6);
@@ -935,10 +937,7 @@ __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb
     if (step_begin < step_end) {
         if constexpr (kPaired) {
             if (ti.fp6) {
-                if constexpr (MB > 4)                                    // (accumulators elsewhere: the registers are there)
-                    stream_tile_mbp<true, G128, MB>(p, ti, ring, step_begin, step_end, acc);
-                else
-                    stream_tile_mb<true, G128, D6, MB>(p, ti, ring, step_begin, step_end, acc);
+                stream_tile_mbp<true, G128, MB>(p, ti, ring, step_begin, step_end, acc);
             } else
                 stream_tile_mbp<false, G128, MB>(p, ti, ring, step_begin, step_end, acc);
         } else {
