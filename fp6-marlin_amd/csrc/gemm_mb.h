@@ -10,7 +10,7 @@ namespace fp6m {
 // every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per 16*MB rows.  MB = 2 or
 // 4 (accumulators in ordinary registers, two waves per SIMD) or 8 (accumulators in the accumulation registers, one
 // wave per SIMD; launches whose 128-row tiles fill the chip).  Two loops: stream_tile_mb keeps the words and one step of
-// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 64 rows) fetches A a pair of steps at a
+// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 32 rows) fetches A a pair of steps at a
 // time and the words through registers.  Both dequantise through
 // dequant_entry.  A workgroup is one tile x four or eight k slices; blockIdx.y walks the row tiles.  Group scales are
 // applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more

@@ -237,7 +237,7 @@ def test_eight_k_slices_per_workgroup(oracle):
 
 def test_paired_activation_fetch_of_the_four_block_kernel(oracle):
     """The m > 32 kernel with the activations fetched a pair of k steps at a time and the INT4 words through
-    registers (picked from 65 rows on), forced on and off: ragged row counts (row groups of eight that are partly
+    registers (picked from 33 rows on), forced on and off: ragged row counts (row groups of eight that are partly
     or wholly past m), one k unit per slice, group scales or not, FP6-only and INT4-only problems, eight or four
     slices per workgroup, several launches."""
     for pair in (1, 0):
