@@ -764,7 +764,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // k step when its four-wave workgroup has the CU to itself, 0.56 us when the CU hosts eight waves (two such
             // workgroups, or one of eight waves), 0.72 us when every CU does, 1.1 us beyond; the kernel lasts as long as
             // the longest slice on the busiest CU, plus 2.5 us and 0.15 us per partner when tiles are split across
-            // workgroups.  Grids of exactly one or two workgroups per CU with equal slices, and eight-wave workgroups
+            // workgroups, plus the partial sums' traffic.  Grids of exactly one or two workgroups per CU with equal slices, and eight-wave workgroups
             // that need no split at all, beat the rule by 4-15 % where the shape allows them; the rule's choice is kept
             // unless the model sees 8 % or more.
             {
@@ -779,14 +779,17 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         // eight waves per workgroup paid off only with one workgroup on (nearly) every CU: measured
                         // slower both when CUs hosted two of them and when a quarter or more of the CUs stayed idle
                         // (without a k split of the INT4 tiles there is no tail to lose, so fewer busy CUs still pay)
-                        if (load > 1.0 || load < (c == 1 ? 0.5 : 0.75)) return 1e9;
+                        if (load > 1.0 || load < (c == 1 ? 0.5 : 0.65)) return 1e9;
                         t = 0.56;
                     }
                     auto longest = [&](long long slices) { return (double)((units + slices - 1) / slices) * unit_steps; };
                     auto tail = [](long long partners) { return partners > 1 ? 2.5 + 0.15 * partners : 0.0; };
                     const double int4_us = a.groups4 ? longest(c * wk) * t + tail(c) : 0.0;
                     const double fp6_us = a.groups6 ? 1.5 * longest(c6 * wk) * t + tail(c6) : 0.0;   // an FP6 step moves 1.5x the bytes
-                    return int4_us > fp6_us ? int4_us : fp6_us;
+                    // every workgroup of a split tile writes its m x 128 partial sums and the last arrival reads them
+                    // back, at about 2 TB/s all told (5120 x 13824 at 16 rows: 440 workgroups 15.4 us, 220 13.6)
+                    const double partial_us = (c > 1 ? a.groups4 * c : 0) * a.m * 0.0005 + (c6 > 1 ? a.groups6 * c6 : 0) * a.m * 0.0005;
+                    return (int4_us > fp6_us ? int4_us : fp6_us) + partial_us;
                 };
                 int best_wk = cfg.wk;
                 long long best = ks;
