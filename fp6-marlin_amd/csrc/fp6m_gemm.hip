@@ -861,7 +861,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.ksplit = (int)ks;
             // A grid of at most one workgroup per CU would leave every SIMD a single wave: give the workgroup eight
             // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
-            int wk = base * ks <= cus && units / 16 >= ks ? 8 : kWaves;
+            // (Two waves on a SIMD take turns at its one VALU/MFMA port: eight half-length slices last as long as four
+            // whole ones, so eight (which hide latency better: 13824 x 5120 at 256 rows 60.6 vs 67.8 us) only pay while
+            // their longest slice, in whole k units, is no more than 0.55 of the longest of four: 5120 x 13824 at 64
+            // rows, 40 units over 16 slices 24.1 us, over 8 slices 21.7.)
+            const long long longest8 = (units + 8 * ks - 1) / (8 * ks), longest4 = (units + 4 * ks - 1) / (4 * ks);
+            int wk = base * ks <= cus && units / 16 >= ks && 20 * longest8 <= 11 * longest4 ? 8 : kWaves;
             if (tune.wk != kUnset) wk = tune.wk == 8 ? 8 : kWaves;
             if (mb == 8) wk = kWaves;                                  // (512 registers per wave: one wave per SIMD)
             // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
@@ -871,10 +876,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // a free CU loses far more than that).  A forced split applies to both kinds.
             a.ks4 = (int)ks;
             a.ks6 = (int)ks;
-            const long long resident = (long long)cus * (wk == 8 || mb == 8 ? 1 : 2);
+            // (a grid that fits one workgroup per CU must still do so afterwards: a CU with two runs both at little
+            // more than half speed, 11008 x 4096 at 256 rows 34 -> 52 us with 272 workgroups)
+            const long long resident = (long long)cus * (wk == 8 || mb == 8 || base * ks <= cus ? 1 : 2);
             // (Not for 128-row tiles, whose FP6 workgroups are only a few per cent behind: there the second partner's
             // partial tiles cost more than the shorter loop gains, 8192 x 8192 at m = 384 61.8 vs 58.4 us.)
-            if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk && mb != 8 &&
+            // Re-measured with every tile on the paired loop (ten shapes x 32 .. 256 rows, alternating): still 5-13 % on
+            // wide weights up to two row tiles (4096 x 11008 at 128 rows 25.3 -> 22.2 us, 8192 x 28672 at 32 rows
+            // 38.2 -> 34.5), but 3-8 % slower from three row tiles on (5120 x 5120 at 256 rows 27.4 -> 29.7): up to two.
+            if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk && mb != 8 && mtiles <= 2 &&
                 (base + (long long)a.tiles6 * mtiles) * ks <= resident)
                 a.ks6 = 2 * (int)ks;
             if (row_mix) {
