@@ -508,10 +508,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     if (shared_frags) mb = 4;
     // 128-row tiles (eight blocks per wave, accumulators in the accumulation registers, one wave per SIMD): every
     // dequantised fragment feeds 16 MFMAs instead of 8.  One workgroup per CU is resident, so the launch takes whole
-    // rounds of 128 rows per CU; 64-row tiles (two workgroups per CU, or one of eight waves) take a third longer for
-    // the same rows (measured 1.28-1.5 x over six shapes, m = 320 .. 2048) but come in finer grain, and below one
+    // rounds of 128 rows per CU; 64-row tiles (two workgroups per CU, or one of eight waves) take 1.13-1.32 x as long for
+    // the same rows (eight shapes, m = 320 .. 2048) but come in finer grain, and below one
     // workgroup per CU they spread their k slices over the idle CUs.  Hence: 128-row tiles when the 64-row tiles
-    // would not fit one per CU and  rounds of 128-row workgroups <= 1.33 x max(1, the same work in rounds).
+    // would not fit one per CU and  rounds of 128-row workgroups <= 1.25 x max(1, the same work in rounds).
     // (8192 x 8192: m = 384 74 -> 62 us, m = 512 88 -> 69, m = 768 136 -> 121, m = 1024 177 -> 137; 4096 x 4096 at
     // m = 640 40 -> 36, at m = 512 the rule keeps 64-row tiles: 28 vs 36; 8192 x 5120 at m = 512 69 -> 60, at m = 2048
     // 233 -> 188, at m = 896 it keeps them: 109 vs 117.)
@@ -520,8 +520,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         const long long tiles_n = prob_n / kTileN;
         const long long wgs8 = tiles_n * ((rows8 + 127) / 128), wgs4 = tiles_n * ((rows8 + 63) / 64);
         const long long rounds8 = (wgs8 + cus - 1) / cus;
-        // rounds8 <= 1.33 * max(1, wgs4 / (2 cus))   <=>   3 * rounds8 * 2 cus <= 4 * max(2 cus, wgs4)
-        if (wgs4 > cus && 6 * rounds8 * cus <= 4 * (wgs4 > 2LL * cus ? wgs4 : 2LL * cus)) mb = 8;
+        // rounds8 <= 1.25 * max(1, wgs4 / (2 cus))   <=>   4 * rounds8 * 2 cus <= 5 * max(2 cus, wgs4)
+        if (wgs4 > cus && 8 * rounds8 * cus <= 5 * (wgs4 > 2LL * cus ? wgs4 : 2LL * cus)) mb = 8;
     }
     const int rows_per_tile = 16 * mb;
     const int mtiles_total = (prob_m + rows_per_tile - 1) / rows_per_tile;
