@@ -904,14 +904,27 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         prob_k, mb, mtiles, a.ks4, a.ks6, wk, grid.x, grid.y);
             // Every launch of 64-row tiles takes the paired loop (33 rows: -5 % .. +5 % over five shapes, 40 rows 0-9 % faster,
             // 64 rows 9-16 %, from 65 rows on 12-20 %; before the FP6 tiles had it too, whose workgroups set a resident
-            // grid's length, it paid from 65 rows on only).  The ring loop stays for 32-row tiles and the tuning hook.
+            // grid's length, it paid from 65 rows on only).  The ring loop stays for the tuning hook and for 32-row tiles in
+            // four-wave workgroups (below).
             bool pair = true;
             if (tune.pair != kUnset) pair = mb >= 4 && tune.pair != 0;
             if (mb == 8) {
                 // (always the paired loop: the ring loop's 30 KiB per wave would fit, but it was slower at every size)
                 void (*kernel)(const GemmArgs) = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, true> : gemm_mb_kernel<false, 8, 3, 3, 4, true>;
                 hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, a);
-            } else if (mb == 2) launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
+            } else if (mb == 2) {
+                // 32-row tiles: the paired loop where two waves share a SIMD (4096 x 11008 at 32 rows 15.4 -> 14.0 us,
+                // per-column scales 14.9 -> 12.8; 8192 x 8192 16.6 -> 15.8), the ring loop, with its longer look-ahead,
+                // where a wave has the SIMD to itself (5120 x 13824 with group scales: 16.7 vs 17.4 paired)
+                bool pair2 = wk == 8;
+                if (tune.pair != kUnset) pair2 = wk == 8 && tune.pair != 0;
+                if (pair2) {
+                    void (*kernel)(const GemmArgs) = g128 ? gemm_mb_kernel<true, 2, 4, 3, 8, true> : gemm_mb_kernel<false, 2, 4, 3, 8, true>;
+                    hipLaunchKernelGGL(kernel, grid, dim3(512), 0, st, a);
+                } else {
+                    launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
+                }
+            }
             else if (pair) launch_mb<4, 3, 3, true>(a, g128, wk, grid, st);
             else launch_mb<4, 3, 3, false>(a, g128, wk, grid, st);
         }

@@ -10,8 +10,8 @@ namespace fp6m {
 // every dequantised weight fragment feeds 2*MB MFMAs, so the packed words are read once per 16*MB rows.  MB = 2 or
 // 4 (accumulators in ordinary registers, two waves per SIMD) or 8 (accumulators in the accumulation registers, one
 // wave per SIMD; launches whose 128-row tiles fill the chip).  Two loops: stream_tile_mb keeps the words and one step of
-// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 32 rows) fetches A a pair of steps at a
-// time and the words through registers.  Both dequantise through
+// A (MB x 1 KiB) per slot of a ring; stream_tile_mbp (launches with more than 32 rows, and 32-row tiles in eight-wave
+// workgroups) fetches A a pair of steps at a time and the words through registers.  Both dequantise through
 // dequant_entry.  A workgroup is one tile x four or eight k slices; blockIdx.y walks the row tiles.  Group scales are
 // applied to the dequantised weights (fp16) because per-group fp32 accumulators would need MB*32 more
 // registers.  Rows beyond m are clamped to the last row on the fetch side (every lane always loads, so
@@ -517,7 +517,8 @@ template <bool FP6, bool G128, int MB>
 __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInfo& ti, unsigned char* ring,
                                                 int step_begin, int step_end, f4 (&acc)[MB][8])
 {
-    static_assert(MB == 4 || MB == 8, "the A register ring runs with phase 0 in every step");
+    static_assert(MB == 2 || MB == 4 || MB == 8, "the A register ring");
+    constexpr int kOddPhase = MB == 2 ? 2 : 0;            // (two blocks per step walk the four register buffers in two steps)
     constexpr bool kGroup = G128 && !FP6;
     constexpr int kPair = MB * kPairBlock;                // one pair slot
     constexpr int kWOps = FP6 ? 4 : 2;                    // register loads per step
@@ -685,9 +686,9 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
 #pragma unroll
                 for (int d = 0; d < 4; d++) cx.addr_next[d] = cx.addr_cur[d] + to_next;
                 if (next_group)                                        // (the reads of the group scales sit between A(1) and A(2))
-                    MbBlocks<MB, 8>::template run<0, 1, kWOps>(cx, cur, acc, hook);
+                    MbBlocks<MB, 8>::template run<kOddPhase, 1, kWOps>(cx, cur, acc, hook);
                 else
-                    MbBlocks<MB, 0>::template run<0, 1, kWOps>(cx, cur, acc, hook);
+                    MbBlocks<MB, 0>::template run<kOddPhase, 1, kWOps>(cx, cur, acc, hook);
 #pragma unroll
                 for (int d = 0; d < 4; d++) cx.addr_cur[d] = cx.addr_next[d];   // on to the next pair's slot
                 to_next = 0u - to_next;
@@ -911,7 +912,6 @@ __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb
     // plane's registers on top, and in a grid that is resident all at once the few FP6 workgroups set the length of
     // the launch (8192 x 8192 with 256 FP6 columns: m = 128 31.8 -> 27.1 us, m = 256 47.0 -> 40.3).
     constexpr bool kPaired = PAIR;
-    static_assert(!PAIR || MB == 4 || MB == 8, "stream_tile_mbp is written for whole rounds of the four A buffers");
     constexpr int kWaveLds = kPaired ? max3(mbp_wave_lds(MB), mb_wave_lds(MB, 0, D6), 0) : mb_wave_lds(MB, D4, D6);
     static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];

@@ -236,8 +236,8 @@ def test_eight_k_slices_per_workgroup(oracle):
 
 
 def test_paired_activation_fetch_of_the_four_block_kernel(oracle):
-    """The m > 32 kernel with the activations fetched a pair of k steps at a time and the INT4 words through
-    registers (picked from 33 rows on), forced on and off: ragged row counts (row groups of eight that are partly
+    """The m > 16 kernel with the activations fetched a pair of k steps at a time and the packed words through
+    registers (picked from 33 rows on, and for 32-row tiles in eight-wave workgroups), forced on and off: ragged row counts (row groups of eight that are partly
     or wholly past m), one k unit per slice, group scales or not, FP6-only and INT4-only problems, eight or four
     slices per workgroup, several launches."""
     for pair in (1, 0):
@@ -248,9 +248,21 @@ def test_paired_activation_fetch_of_the_four_block_kernel(oracle):
             run(oracle, 48, 768, 512, qc=128, env=e)
             run(oracle, 70, 256, 64, qc=-1, env=e)                      # one k unit: idle slices
             run(oracle, 130, 512, 2048, qc=256, ksplit=3, env=e)
-            run(oracle, 77, 512, 512, qc=512, ksplit=2, env=e)          # all FP6: every tile on the ring path
+            run(oracle, 77, 512, 512, qc=512, ksplit=2, env=e)          # all FP6
             run(oracle, 300, 256, 1024, qc=-1, gs=128, max_par=2, env=e)   # three launches, the last of 44 rows
     run(oracle, 256, 2048, 2048, qc=256, gs=128)                        # the dispatcher's own choice of it
+    # 32-row tiles take the paired loop in eight-wave workgroups (two blocks per step walk the four activation
+    # register buffers in two steps): ragged rows, both scale modes, all FP6, a forced split, one-hot rows bit for
+    # bit, and bit-identical to the ring loop
+    for m in (17, 24, 25, 32):
+        outs = [run(oracle, m, 512, 1024, qc=256, gs=128, env={"FP6M_WK": 8, "FP6M_PAIR": pair}) for pair in (1, 0)]
+        assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+        run(oracle, m, 768, 512, qc=128, env={"FP6M_WK": 8, "FP6M_PAIR": 1})
+    run(oracle, 30, 512, 512, qc=512, ksplit=2, env={"FP6M_WK": 8, "FP6M_PAIR": 1})
+    run(oracle, 20, 256, 64, qc=-1, env={"FP6M_WK": 8, "FP6M_PAIR": 1})       # one k unit: idle slices
+    run(oracle, 29, 1024, 8192, qc=256, gs=128)                           # the dispatcher's own choice of it
+    for gs in (-1, 128):
+        one_hot_case(oracle, 27, 768, 1024, 256, gs, {"wk": 8, "pair": 1})
 
 
 def test_fp6_tiles_with_a_finer_k_split_than_int4_tiles(oracle):
