@@ -243,10 +243,11 @@ inline FastDiv make_div(long long d, long long max_n)
 template <int AROWS, int WN, int WK, int D4, int D6>
 void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
-    if (g128)
-        hipLaunchKernelGGL((gemm_m16_kernel<true, AROWS, WN, WK, D4, D6>), grid, dim3(64 * WN * WK), 0, stream, a);
-    else
-        hipLaunchKernelGGL((gemm_m16_kernel<false, AROWS, WN, WK, D4, D6>), grid, dim3(64 * WN * WK), 0, stream, a);
+    void (*kernel)(const GemmArgs) = g128 ? gemm_m16_kernel<true, AROWS, WN, WK, D4, D6, false> : gemm_m16_kernel<false, AROWS, WN, WK, D4, D6, false>;
+    if constexpr (AROWS == 4) {                                       // (the cells serve up to four rows)
+        if (a.cells) kernel = g128 ? gemm_m16_kernel<true, AROWS, WN, WK, D4, D6, true> : gemm_m16_kernel<false, AROWS, WN, WK, D4, D6, true>;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * WN * WK), 0, stream, a);
 }
 
 // n / d as (n * magic) >> 40: exact for n < 2^24 and d < 2^16.
@@ -821,7 +822,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // being published, counted and gathered: one round trip after the loop instead of three (4096 x 4096 at two
             // rows 8.1 -> 7.0 us, 11008 x 4096 11.1 -> 10.1, 8192 x 8192 12.2 -> 11.6; even at four rows; the atomics of
             // eight and sixteen rows cost more than the round trips: 4096 x 4096 at sixteen rows 9.3 -> 10.3 us).
-            const bool want_cells = tune.cells != kUnset ? tune.cells != 0 : a.m <= 4;
+            const bool want_cells = a.m <= 4 && !(tune.cells != kUnset && tune.cells == 0);
             if (want_cells && (size_t)prob_n * 16 * sizeof(unsigned long long) <= kCellBytes && a.ks4 <= kMaxParts &&
                 a.ks6 <= kMaxParts)
                 a.cells = reinterpret_cast<unsigned long long*>(reinterpret_cast<unsigned char*>(a.scratch) + scratch_bytes);

@@ -290,7 +290,7 @@ constexpr int wave_lds_bytes(int d4, int d6, int arows)
 // tile wn over the WK slices (fixed order) with lane L owning columns 2L, 2L+1.  With one k part per
 // tile group it scales and writes C; otherwise it publishes the rows with agent-scope stores, the
 // workgroup bumps the group's counter, and the workgroup that arrives last sums all parts in part order.
-template <int WN, int WK>
+template <int WN, int WK, bool CELLS>
 __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti, bool tile_valid, int wn, int wk,
                                           int ks, int slot_base, int* counter, f4 (&acc)[1][8],
                                           bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
@@ -375,7 +375,7 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
         return;
     }
 
-    if (p.cells) {
+    if constexpr (CELLS) {
         // The parts of the tile meet in its cells (see gemm_common.h): one returning atomic per element, values in output
         // units; whoever arrives last at an element stores it and writes its cell back to zero.  Nothing is published,
         // counted or gathered, and no barrier follows the sum through LDS.
@@ -472,7 +472,10 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
     if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <bool G128, int AROWS, int WN, int WK, int D4, int D6>
+// CELLS: tiles shared by several workgroups are summed in the accumulate-and-count cells (up to four rows) instead of
+// through published partial tiles; a compile-time choice, because the mere presence of the other path behind a
+// run-time branch cost the partial-tile path 0.3-0.6 us (4096 x 4096 at 16 rows: 8.9 -> 9.4 us).
+template <bool G128, int AROWS, int WN, int WK, int D4, int D6, bool CELLS>
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
 __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void gemm_m16_kernel(const GemmArgs p)
 {
@@ -526,7 +529,7 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
     // scratch slots: FP6 groups first (groups6 * ks6 slots), then INT4 groups; counters likewise
     const int slot_base = region6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
     int* counter = p.counters + (region6 ? group : p.groups6 + group);
-    wg_finish<WN, WK>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
+    wg_finish<WN, WK, CELLS>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
                       reinterpret_cast<int*>(smem + NW * kWaveLds), p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
 }

@@ -159,8 +159,8 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * "wm" / "wn" (shared-fragment kernel on/off, its column tiles per workgroup), "pair" (paired activation fetch on/off),
  * "sk" (the one-wave decode kernel on for m <= 4 / off), "share" / "share6" (k units per chunk of its work list: both
  * regions / the FP6 region only), "cap" (the waves it aims at), "wgs" (exactly that many waves, one-unit chunks drawn
- * from the counters), "gather" (its own activation gather on / off), "cells" (the m <= 16 kernel's shared tiles summed
- * in the accumulate-and-count cells on / off; by default up to four rows),
+ * from the counters), "gather" (its own activation gather on / off), "cells" (0: the m <= 16 kernel sums the shared
+ * tiles of up to four rows through partial tiles, like those of more rows, instead of in the accumulate-and-count cells),
  * "verbose" (print every launch's configuration to stderr); knob = NULL clears all overrides.  Unknown knob ->
  * FP6M_ERR_ARG.  Not synchronised with GEMM calls running on other threads.  The library reads no environment
  * variables on a call (FP6M_VERBOSE is looked up once at load time).

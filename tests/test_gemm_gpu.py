@@ -145,26 +145,26 @@ def test_forced_split_k_and_determinism(oracle):
 
 
 def test_cells_and_partial_tiles_up_to_sixteen_rows(oracle):
-    """The m <= 16 kernel sums a tile shared by several workgroups either in the accumulate-and-count cells (its
-    choice up to four rows) or through published partial tiles gathered by the last arrival (beyond): both forced
-    for every row count class, with 1 .. 16 partners, both scale modes, a fused epilogue, one-hot rows bit for
-    bit, and each against itself on a second call."""
-    import fp6_marlin
+    """The m <= 16 kernel sums a tile shared by several workgroups in the accumulate-and-count cells up to four rows
+    and through published partial tiles gathered by the last arrival beyond (the `cells` knob sends the small row
+    counts there too): every row count class, 1 .. 16 partners, both scale modes, all FP6, one-hot rows bit for
+    bit, each against itself on a second call, and the two paths against each other."""
     for cells in (1, 0):
         e = {"FP6M_CELLS": cells}
         for m in (2, 3, 4, 5, 9, 16):
             run(oracle, m, 512, 2048, qc=256, gs=128, env=e)
             run(oracle, m, 1024, 1024, qc=256, ksplit=3, env=e)
         for ks in (2, 8, 16):
+            run(oracle, 4, 512, 2048, qc=256, ksplit=ks, env=e)
             run(oracle, 16, 512, 2048, qc=256, ksplit=ks, env=e)
-        run(oracle, 7, 256, 4096, qc=-1, env=e)
-        run(oracle, 12, 512, 1024, qc=512, ksplit=4, env=e)                # all FP6
+        run(oracle, 3, 256, 4096, qc=-1, env=e)
+        run(oracle, 4, 512, 1024, qc=512, ksplit=4, env=e)                 # all FP6
         for gs in (-1, 128):
-            one_hot_case(oracle, 9, 768, 1024, 256, gs, {"cells": cells, "ksplit": 4})
+            one_hot_case(oracle, 4, 768, 1024, 256, gs, {"cells": cells, "ksplit": 4})
             one_hot_case(oracle, 3, 512, 2048, 256, gs, {"cells": cells})
     # the same sums either way, up to the cells' fixed-point grid of 2^-29 in output units: at most one fp16 ulp apart
-    a = run(oracle, 16, 512, 2048, qc=256, gs=128, ksplit=8, env={"FP6M_CELLS": 1})
-    b = run(oracle, 16, 512, 2048, qc=256, gs=128, ksplit=8, env={"FP6M_CELLS": 0})
+    a = run(oracle, 4, 512, 2048, qc=256, gs=128, ksplit=8, env={"FP6M_CELLS": 1})
+    b = run(oracle, 4, 512, 2048, qc=256, gs=128, ksplit=8, env={"FP6M_CELLS": 0})
     ulps = np.abs(a.view(np.int16).astype(np.int32) - b.view(np.int16).astype(np.int32))
     assert ulps.max() <= 1 and (ulps != 0).mean() < 0.01, (ulps.max(), (ulps != 0).mean())
 
