@@ -277,19 +277,35 @@ inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, d
         launch_m16<16, 1, 4, 4, 3>(a, g128, grid, stream);
 }
 
-template <int MB, int D4, int D6, bool PAIR>
+// Whether a call needs the kernel build with the row mix, the fused epilogue and the gfx950 word order in it.
+inline bool needs_extras(const GemmArgs& a) { return a.k4 != 0 || a.fused != 0 || a.native != 0; }
+
+template <bool G128, int MB, int D4, int D6, int WK, bool PAIR, bool LEAN>
+void launch_mb_one(const GemmArgs& a, dim3 grid, hipStream_t stream)
+{
+    void (*kernel)(const GemmArgs) = gemm_mb_kernel<G128, MB, D4, D6, WK, PAIR, true>;
+    // (One of them does not: without the extras the allocator of the four-wave 64-row kernel with per-column scales
+    // ends up one register short of its 256 and spills.)
+    if constexpr (LEAN && !(MB == 4 && WK == 4 && !G128)) {
+        if (!needs_extras(a)) kernel = gemm_mb_kernel<G128, MB, D4, D6, WK, PAIR, false>;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * WK), 0, stream, a);
+}
+
+// LEAN: the kernels the dispatcher picks by itself also exist without the extras (those only the tuning hook reaches do not).
+template <int MB, int D4, int D6, bool PAIR, bool LEAN = true>
 void launch_mb(const GemmArgs& a, bool g128, int wk, dim3 grid, hipStream_t stream)
 {
     if (wk == 8) {
         if (g128)
-            hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6, 8, PAIR>), grid, dim3(512), 0, stream, a);
+            launch_mb_one<true, MB, D4, D6, 8, PAIR, LEAN>(a, grid, stream);
         else
-            hipLaunchKernelGGL((gemm_mb_kernel<false, MB, D4, D6, 8, PAIR>), grid, dim3(512), 0, stream, a);
+            launch_mb_one<false, MB, D4, D6, 8, PAIR, LEAN>(a, grid, stream);
     } else {
         if (g128)
-            hipLaunchKernelGGL((gemm_mb_kernel<true, MB, D4, D6, 4, PAIR>), grid, dim3(256), 0, stream, a);
+            launch_mb_one<true, MB, D4, D6, 4, PAIR, LEAN>(a, grid, stream);
         else
-            hipLaunchKernelGGL((gemm_mb_kernel<false, MB, D4, D6, 4, PAIR>), grid, dim3(256), 0, stream, a);
+            launch_mb_one<false, MB, D4, D6, 4, PAIR, LEAN>(a, grid, stream);
     }
 }
 
@@ -911,8 +927,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (tune.pair != kUnset) pair = mb >= 4 && tune.pair != 0;
             if (mb == 8) {
                 // (always the paired loop: the ring loop's 30 KiB per wave would fit, but it was slower at every size)
-                void (*kernel)(const GemmArgs) = g128 ? gemm_mb_kernel<true, 8, 3, 3, 4, true> : gemm_mb_kernel<false, 8, 3, 3, 4, true>;
-                hipLaunchKernelGGL(kernel, grid, dim3(256), 0, st, a);
+                if (g128)
+                    launch_mb_one<true, 8, 3, 3, 4, true, true>(a, grid, st);
+                else
+                    launch_mb_one<false, 8, 3, 3, 4, true, true>(a, grid, st);
             } else if (mb == 2) {
                 // 32-row tiles: the paired loop where two waves share a SIMD (4096 x 11008 at 32 rows 15.4 -> 14.0 us,
                 // per-column scales 14.9 -> 12.8; 8192 x 8192 16.6 -> 15.8), the ring loop, with its longer look-ahead,
@@ -920,14 +938,16 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 bool pair2 = wk == 8;
                 if (tune.pair != kUnset) pair2 = wk == 8 && tune.pair != 0;
                 if (pair2) {
-                    void (*kernel)(const GemmArgs) = g128 ? gemm_mb_kernel<true, 2, 4, 3, 8, true> : gemm_mb_kernel<false, 2, 4, 3, 8, true>;
-                    hipLaunchKernelGGL(kernel, grid, dim3(512), 0, st, a);
+                    if (g128)
+                        launch_mb_one<true, 2, 4, 3, 8, true, true>(a, grid, st);
+                    else
+                        launch_mb_one<false, 2, 4, 3, 8, true, true>(a, grid, st);
                 } else {
                     launch_mb<2, 4, 3, false>(a, g128, wk, grid, st);
                 }
             }
             else if (pair) launch_mb<4, 3, 3, true>(a, g128, wk, grid, st);
-            else launch_mb<4, 3, 3, false>(a, g128, wk, grid, st);
+            else launch_mb<4, 3, 3, false, false>(a, g128, wk, grid, st);
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return hip_fail(e);

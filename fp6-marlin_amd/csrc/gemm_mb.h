@@ -905,9 +905,23 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 // WK = k slices (waves) per workgroup: four, or eight (one workgroup per CU, two waves per SIMD) for grids that
 // would otherwise leave every SIMD a single wave.
 // PAIR: A is fetched by pairs of steps and the words through registers (stream_tile_mbp).
-template <bool G128, int MB, int D4, int D6, int WK, bool PAIR>
-__global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb_kernel(const GemmArgs p)
+// EXTRAS = false: a build of the same kernel without the row mix, the fused epilogue and the gfx950 word order, for
+// calls that use none of them (plain fp6m_mul on reference-order words).  Their run-time branches cost the plain path
+// 2-6 % (4096 x 4096 at 64 rows 15.8 -> 14.8 us, 8192 x 8192 at 512 rows 68.4 -> 67.3): the arguments are overwritten
+// with constants and the compiler removes what hangs on them.
+template <bool G128, int MB, int D4, int D6, int WK, bool PAIR, bool EXTRAS = true>
+__global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb_kernel(const GemmArgs args)
 {
+    GemmArgs p = args;
+    if constexpr (!EXTRAS) {
+        p.k4 = 0;
+        p.slices4 = 0;
+        p.native = 0;
+        p.fused = 0;
+        p.c_cols = nullptr;
+        p.bias = nullptr;
+        p.residual = nullptr;
+    }
     // FP6 tiles take the paired loop too: with the dequantisation as asm statements it fits 256 VGPRs with the 2-bit
     // plane's registers on top, and in a grid that is resident all at once the few FP6 workgroups set the length of
     // the launch (8192 x 8192 with 256 FP6 columns: m = 128 31.8 -> 27.1 us, m = 256 47.0 -> 40.3).
@@ -916,7 +930,7 @@ __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb
     static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];
 
-    preload_args(p);
+    preload_args(args);
     FP6M_MARK(p, 0);
     TileInfo ti = locate_tile(p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
