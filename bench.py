@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline workload (mean of its four GEMMs): FETCH_SIZE + WRITE_SIZE from two
 # `rocprofv3 --pmc` runs of `bench.py --traffic-probe`, each scaled by what the same counter reads for a
 # 256 MiB device copy (x2.000 and x1.000); figures in profiles/gemm_sk_kernel_decode7b_hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28944107
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28882764
 TRAFFIC_PROFILE = "profiles/gemm_sk_kernel_decode7b_hbm_traffic.txt"
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLAMA7B = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
@@ -232,7 +232,7 @@ def headline(args):
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in " + TRAFFIC_PROFILE +
                                        ", not measured in this run",
-                     "kernel": "fp6m::gemm_sk_kernel<true, 0, false>", "us_per_launch": round(per_launch * 1e6, 3),
+                     "kernel": "fp6m::gemm_sk_kernel<true, 0, false, false>", "us_per_launch": round(per_launch * 1e6, 3),
                      "bytes_per_launch": step_bytes // launches_per_step},
         "cpu_baseline": cpu_baseline(torch),
         "fp16_hipblaslt": {"ms_per_step": round(wall16 / args.steps * 1e3, 5),

@@ -240,14 +240,33 @@ inline FastDiv make_div(long long d, long long max_n)
 //   1: rows <= 16, same shape, 1 KiB of A per slot
 // Workgroups of several adjacent tiles (WN > 1) were measured and were never faster on MI355X; the
 // kernel keeps the template parameter, only WN = 1 is instantiated.
+// Whether a call needs the kernel build with the row mix, the fused epilogue and the gfx950 word order in it.
+inline bool needs_extras(const GemmArgs& a) { return a.k4 != 0 || a.fused != 0 || a.native != 0; }
+
+template <bool G128, int AROWS, int WN, int WK, int D4, int D6, bool EXTRAS>
+void launch_m16_one(const GemmArgs& a, dim3 grid, hipStream_t stream)
+{
+    void (*kernel)(const GemmArgs) = gemm_m16_kernel<G128, AROWS, WN, WK, D4, D6, false, EXTRAS>;
+    if constexpr (AROWS == 4) {                                       // (the cells serve up to four rows)
+        if (a.cells) kernel = gemm_m16_kernel<G128, AROWS, WN, WK, D4, D6, true, EXTRAS>;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * WN * WK), 0, stream, a);
+}
+
 template <int AROWS, int WN, int WK, int D4, int D6>
 void launch_m16(const GemmArgs& a, bool g128, dim3 grid, hipStream_t stream)
 {
-    void (*kernel)(const GemmArgs) = g128 ? gemm_m16_kernel<true, AROWS, WN, WK, D4, D6, false> : gemm_m16_kernel<false, AROWS, WN, WK, D4, D6, false>;
-    if constexpr (AROWS == 4) {                                       // (the cells serve up to four rows)
-        if (a.cells) kernel = g128 ? gemm_m16_kernel<true, AROWS, WN, WK, D4, D6, true> : gemm_m16_kernel<false, AROWS, WN, WK, D4, D6, true>;
+    if (needs_extras(a)) {
+        if (g128)
+            launch_m16_one<true, AROWS, WN, WK, D4, D6, true>(a, grid, stream);
+        else
+            launch_m16_one<false, AROWS, WN, WK, D4, D6, true>(a, grid, stream);
+    } else {
+        if (g128)
+            launch_m16_one<true, AROWS, WN, WK, D4, D6, false>(a, grid, stream);
+        else
+            launch_m16_one<false, AROWS, WN, WK, D4, D6, false>(a, grid, stream);
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(64 * WN * WK), 0, stream, a);
 }
 
 // n / d as (n * magic) >> 40: exact for n < 2^24 and d < 2^16.
@@ -276,9 +295,6 @@ inline void launch_m16_any(const M16Config& cfg, const GemmArgs& a, bool g128, d
     else
         launch_m16<16, 1, 4, 4, 3>(a, g128, grid, stream);
 }
-
-// Whether a call needs the kernel build with the row mix, the fused epilogue and the gfx950 word order in it.
-inline bool needs_extras(const GemmArgs& a) { return a.k4 != 0 || a.fused != 0 || a.native != 0; }
 
 template <bool G128, int MB, int D4, int D6, int WK, bool PAIR, bool LEAN>
 void launch_mb_one(const GemmArgs& a, dim3 grid, hipStream_t stream)
@@ -738,10 +754,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // variants: group scales or not; one chunk per wave with or without the gather, or chunks drawn from counters
             void (*kernel)(const SkArgs) = nullptr;
             const bool draw = sk.total4 || sk.total6;
+            const bool lean = sk.flags == 0;                          // (no fused epilogue, reference-order words)
             if (gather_inside)
                 kernel = g128 ? gemm_sk_kernel<true, 1, false> : gemm_sk_kernel<false, 1, false>;
+            else if (draw && lean)
+                kernel = g128 ? gemm_sk_kernel<true, 0, true, false> : gemm_sk_kernel<false, 0, true, false>;
             else if (draw)
                 kernel = g128 ? gemm_sk_kernel<true, 0, true> : gemm_sk_kernel<false, 0, true>;
+            else if (lean)
+                kernel = g128 ? gemm_sk_kernel<true, 0, false, false> : gemm_sk_kernel<false, 0, false, false>;
             else
                 kernel = g128 ? gemm_sk_kernel<true, 0, false> : gemm_sk_kernel<false, 0, false>;
             hipLaunchKernelGGL(kernel, grid, dim3(64), 0, st, sk);

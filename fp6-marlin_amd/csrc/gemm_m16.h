@@ -475,15 +475,27 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
 // CELLS: tiles shared by several workgroups are summed in the accumulate-and-count cells (up to four rows) instead of
 // through published partial tiles; a compile-time choice, because the mere presence of the other path behind a
 // run-time branch cost the partial-tile path 0.3-0.6 us (4096 x 4096 at 16 rows: 8.9 -> 9.4 us).
-template <bool G128, int AROWS, int WN, int WK, int D4, int D6, bool CELLS>
+// EXTRAS = false: the build for calls without row mix, fused epilogue or gfx950 word order (their arguments are
+// overwritten with constants; their presence cost the plain call 2-3 %).
+template <bool G128, int AROWS, int WN, int WK, int D4, int D6, bool CELLS, bool EXTRAS = true>
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
-__global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void gemm_m16_kernel(const GemmArgs p)
+__global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void gemm_m16_kernel(const GemmArgs args)
 {
     constexpr int NW = WN * WK;
     constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);
     __shared__ __attribute__((aligned(16))) unsigned char smem[NW * kWaveLds + 16];
 
-    preload_args(p);
+    GemmArgs p = args;
+    if constexpr (!EXTRAS) {
+        p.k4 = 0;
+        p.slices4 = 0;
+        p.native = 0;
+        p.fused = 0;
+        p.c_cols = nullptr;
+        p.bias = nullptr;
+        p.residual = nullptr;
+    }
+    preload_args(args);
     FP6M_MARK(p, 0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
     const int wn = wave % WN, wk = wave / WN;

@@ -610,11 +610,19 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
 constexpr int kSkWaveLds = wave_lds_bytes(4, 3, 4) + 4 * kRedStride * 4;   // ring, then the four-row slab
 
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
-template <bool G128, int GR, bool DRAW>
+// EXTRAS = false: the build for calls without a fused epilogue on reference-order words (the arguments that select
+// those paths are overwritten with constants; their presence cost the plain call 1-3 %).
+template <bool G128, int GR, bool DRAW, bool EXTRAS = true>
 __global__ __launch_bounds__(64, 3) void gemm_sk_kernel(const SkArgs in_kernarg_segment)
 {
     __shared__ __attribute__((aligned(16))) unsigned char smem[kSkWaveLds];
-    const SkArgs p = load_sk_args();
+    SkArgs p = load_sk_args();
+    if constexpr (!EXTRAS) {
+        p.flags = 0;
+        p.c_cols = nullptr;
+        p.bias = nullptr;
+        p.residual = nullptr;
+    }
     FP6M_MARK(p, 0);
 #ifdef FP6M_TIMELINE
     if (p.timeline) {                                                    // where the wave runs: HW_ID and XCC_ID registers
