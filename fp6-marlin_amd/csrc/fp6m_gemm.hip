@@ -754,7 +754,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // variants: group scales or not; one chunk per wave with or without the gather, or chunks drawn from counters
             void (*kernel)(const SkArgs) = nullptr;
             const bool draw = sk.total4 || sk.total6;
-            const bool lean = sk.flags == 0;                          // (no fused epilogue, reference-order words)
+            const bool lean = sk.flags == 0 && sk.m == 1;             // (one row, no fused epilogue, reference-order words)
             if (gather_inside)
                 kernel = g128 ? gemm_sk_kernel<true, 1, false> : gemm_sk_kernel<false, 1, false>;
             else if (draw && lean)
