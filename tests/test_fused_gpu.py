@@ -240,3 +240,56 @@ def test_graph_replays_of_fused_and_row_mix_calls(oracle):
         assert int(ws.abs().sum()) == 0
         fp6_marlin.mul(A, B, outs[0], s, ws, qc, -1, -1, -1, 16, gs)     # eager work between replays
         torch.cuda.synchronize()
+
+
+def test_random_shapes_maps_and_additions_against_unpacked_words():
+    """A seeded random walk over the fused entry point: shapes, FP6 column counts, scale modes, 1 .. 1100 rows (every
+    kernel), any subset of activation gather (from a wider matrix), output permutation, bias and residual; random
+    packed words against the pinned unpacker and an fp32 matmul with the same reorders and additions."""
+    import random
+    import fp6_marlin
+    from fp6_marlin import cabi
+    rnd = random.Random(7)
+    g = torch.Generator().manual_seed(7)
+    for ci in range(60):
+        k = 256 * rnd.choice([1, 2, 3, 4, 8, 11, 16])
+        n = 256 * rnd.choice([1, 2, 3, 5, 8, 16, 24, 43])
+        qc = min(n, rnd.choice([0, 256, 256, 512, n, 128]))
+        gs = rnd.choice([-1, 128])
+        m = rnd.choice([1, 1, rnd.randint(2, 16), rnd.randint(17, 64), rnd.randint(65, 300), rnd.randint(300, 1100)])
+        max_par = rnd.choice([16, 16, 2])
+        n4 = n - qc
+        B = torch.randint(-2 ** 31, 2 ** 31 - 1, (k * n4 // 8 + k * qc * 3 // 16,), generator=g, dtype=torch.int64).to(torch.int32)
+        s = (torch.rand(((k // gs) * n4 if gs > 0 else n4) + qc, generator=g) * 0.01 + 0.001).half()
+        qarg = qc if qc else -1
+        use_a, use_c, use_b, use_r = [rnd.random() < 0.6 for _ in range(4)]
+        lda = k + (rnd.choice([0, 64, 1000]) if use_a else 0)
+        case = (ci, m, k, n, qc, gs, max_par, use_a, use_c, use_b, use_r, lda)
+        print("case random fused", case, flush=True)
+        w = fp6_marlin.unpack_to_fp16(B, s, k, n, qarg, gs).to(dev())
+        ws = torch.zeros(n // 128 * max_par, dtype=torch.int32, device=dev())
+        A = torch.randn((m, lda), generator=g).half().to(dev())
+        a_cols = torch.randperm(lda, generator=g)[:k].to(torch.int32).to(dev()) if use_a else None
+        c_cols = torch.randperm(n, generator=g).to(torch.int32).to(dev()) if use_c else None
+        bias = (torch.randn(n, generator=g) * 0.5).half().to(dev()) if use_b else None
+        resid = (torch.randn((m, n), generator=g) * 0.5).half().to(dev()) if use_r else None
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        cabi.mul_fused(A, B.to(dev()), C, s.to(dev()), ws, qarg, gs, a_cols=a_cols, c_cols=c_cols, bias=bias, residual=resid,
+                       max_par=max_par)
+        torch.cuda.synchronize()
+        ref = (A[:, a_cols.long()] if use_a else A[:, :k]).float() @ w.float()
+        if use_c:
+            out = torch.empty_like(ref)
+            out[:, c_cols.long()] = ref
+            ref = out
+        if use_b:
+            ref = ref + bias.float()
+        if use_r:
+            ref = ref + resid.float()
+        assert torch.isfinite(C).all(), case
+        assert int(ws.abs().sum().item()) == 0, case
+        d = (C.float() - ref).abs()
+        assert (d.mean() / ref.abs().mean()).item() <= TOL, case
+        assert bool((d <= 4e-3 * ref.abs() + 0.13 * ref.abs().mean()).all()), case
+        del w, A, C, ref
+        torch.cuda.empty_cache()
