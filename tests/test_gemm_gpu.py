@@ -602,3 +602,32 @@ def test_random_shapes_rows_and_limits_against_unpacked_words(oracle):
                 assert bool((d <= 4e-3 * r.abs() + 0.13 * r.abs().mean()).all()), case
         del w, Bd, sd, a, C, C2, ref
         torch.cuda.empty_cache()
+
+
+def test_long_k_with_a_poorly_filled_grid_takes_128_row_tiles_with_a_k_split(capfd):
+    """13824 x 5120 at 256 rows: 160 workgroups of 64 rows would occupy 160 of 256 CUs with nothing left to split; the
+    dispatcher takes 128-row tiles with three k parts instead (read back from its verbose output) and the result is
+    checked per region against the pinned unpacker; on k = 8192 the rule does not apply."""
+    import fp6_marlin
+    g = torch.Generator().manual_seed(9)
+    for k, n, want in ((13824, 5120, "MB=8 row tiles 2 ks4=3"), (8192, 5120, "MB=4")):
+        qc, gs, m = 256, 128, 256
+        n4 = n - qc
+        B = torch.randint(-2 ** 31, 2 ** 31 - 1, (k * n4 // 8 + k * qc * 3 // 16,), generator=g, dtype=torch.int64).to(torch.int32)
+        s = (torch.rand((k // gs) * n4 + qc, generator=g) * 0.01 + 0.001).half()
+        w = fp6_marlin.unpack_to_fp16(B, s, k, n, qc, gs).to(dev())
+        a = torch.randn((m, k), generator=g).half().to(dev())
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+        capfd.readouterr()
+        with fp6_marlin.cabi.tuning(verbose=1):
+            fp6_marlin.mul(a, B.to(dev()), C, s.to(dev()), ws, qc, -1, -1, -1, 16, gs)
+            torch.cuda.synchronize()
+        err = capfd.readouterr().err
+        assert want in err, (k, n, err[-300:])
+        ref = a.float() @ w.float()
+        for sl in (slice(0, n4), slice(n4, n)):
+            d = (C[:, sl].float() - ref[:, sl]).abs()
+            assert (d.mean() / ref[:, sl].abs().mean()).item() <= TOL
+            assert bool((d <= 4e-3 * ref[:, sl].abs() + 0.13 * ref[:, sl].abs().mean()).all())
+        assert int(ws.abs().sum().item()) == 0
