@@ -555,13 +555,13 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         const long long rounds8 = (wgs8 + cus - 1) / cus;
         // rounds8 <= 1.25 * max(1, wgs4 / (2 cus))   <=>   4 * rounds8 * 2 cus <= 5 * max(2 cus, wgs4)
         if (wgs4 > cus && 8 * rounds8 * cus <= 5 * (wgs4 > 2LL * cus ? wgs4 : 2LL * cus)) mb = 8;
-        // One more case: 64-row workgroups that fit one per CU but fill under 70 % of them without a k split (more than
-        // half the CUs: no split possible), on a long k.  128-row tiles with the k split that fills the chip then win
-        // although their partial tiles are twice the size (13824 x 5120 at 256 rows: 160 of 256 CUs, 58 -> 49 us; on
-        // k = 8192 the same trade loses, 8192 x 5120 at 256 rows 37.3 vs 39.0).
+        // One more case: 64-row workgroups that occupy more than half of the CUs, so that they cannot be split, on a
+        // long k.  128-row tiles with a k split that fills at least as many CUs (and three quarters of them) then win
+        // although their partial tiles are twice the size (13824 x 5120 at 256 rows: 160 of 256 CUs, 58 -> 49 us;
+        // 11008 x 5120 48.1 -> 42.5; on k = 8192 the trade is even, below it loses: 5120 x 5120 27.0 vs 30.4).
         const long long ks8 = wgs8 > 0 ? cus / wgs8 : 0;
-        if (mb == 4 && wgs4 <= cus && 2 * wgs4 > cus && 10 * wgs4 < 7 * cus && prob_k >= 12288 && ks8 >= 2 &&
-            20 * wgs8 * ks8 >= 17 * cus && ks8 <= prob_k / (16LL * 128) &&
+        if (mb == 4 && wgs4 <= cus && 2 * wgs4 > cus && prob_k >= 10240 && ks8 >= 2 && 4 * wgs8 * ks8 >= 3 * cus &&
+            wgs8 * ks8 >= wgs4 && ks8 <= prob_k / (16LL * 128) &&
             (size_t)(tiles_n + qc / kTileN) * ((rows8 + 127) / 128) * ks8 * (8 * 16 * kTileN * sizeof(float)) <= kScratchBytes)
             mb = 8;
     }
