@@ -657,7 +657,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // Chunks and waves (measured on MI355X over 17 shapes).  Shorter chunks are faster as long as every chunk
             // has a wave of its own resident at once (twelve waves per CU fit by registers; eleven are used) and a
             // tile is not cut into more than 32 chunks (more made the adds to one cell queue up; the few FP6 tiles, whose
-            // steps take twice as long, may have up to 64 as k grows, so that their waves do not finish last: 43 took
+            // steps take twice as long, may have up to 64 as k grows (24 + a chunk per 512 of k), so that their waves do not finish last: 43 took
             // 11008 x 4096 from 9.9 to 8.8 us and 56 took 28672 x 8192 from 25.2 to 24.7, while 64 chunks of one or two
             // units cost 4096 x 4096 and 8192 x 8192 half a microsecond: short chunks all finish at the same time).  Chunks beyond the
             // waves are drawn from the counters and processed correctly, but every draw and every further chunk's
@@ -699,7 +699,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if (sms == 1 || !cells_fit || q > units_r) q = units_r;
                 return q;
             };
-            const long long max_chunks6 = 32 + u6 / 16 < 64 ? 32 + u6 / 16 : 64;
+            const long long max_chunks6 = 24 + u6 / 8 < 64 ? 24 + u6 / 8 : 64;
             long long q4, q6, cpt4, cpt6, chunks4, chunks6;
             for (;; want4++) {                                         // (a last, shorter chunk per tile may push the count over)
                 want6 = g128 ? want4 : (want4 + 1) / 2;
