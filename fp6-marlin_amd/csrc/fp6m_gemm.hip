@@ -68,7 +68,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -97,6 +97,7 @@ static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBy
 
 struct DeviceState {
     int cus = 0;
+    int xcd_placement = -1;            // 1: workgroup b of a grid runs on XCD b % 8 (verified by verify_placement), 0: not so, -1: not looked at yet
     float* static_scratch = nullptr;   // device address of this GPU's copy of g_static_scratch
     int nregions = 0;
     void* pack_temp = nullptr;      // kPackTempBytes for the on-GPU packer's flag and column maxima
@@ -219,6 +220,55 @@ int pack_temp(int dev, void** ptr)
     return FP6M_OK;
 }
 
+// Every workgroup notes the XCD it runs on in the mask of its group of eight consecutive workgroups.
+constexpr int kProbeGroups = 512;
+__global__ __launch_bounds__(64) void placement_probe_kernel(unsigned* masks)
+{
+    if (threadIdx.x != 0) return;
+    const unsigned linear = blockIdx.y * gridDim.x + blockIdx.x;
+    if ((linear >> 3) < kProbeGroups) atomicOr(masks + (linear >> 3), 1u << (xcc_id() & 31));
+}
+
+// The XCD-local reduction (gemm_m16.h, wg_finish<LOCAL>) identifies a workgroup by the XCD it finds itself on and its
+// index / 8, which covers the work exactly once if eight consecutive workgroups of a dispatch always run on eight
+// different XCDs.  That is how these GPUs deal out workgroups (the XCD of the first one varies with the queue), but it
+// is a property of the machine and of its partition mode, so it is looked at once per device before the dispatcher
+// relies on it: a few grids of a probe kernel on the given stream.  This waits for the device (once), so it is
+// skipped while `stream` is being captured; until it has run, launches use the agent-scope protocol.  Callers hold
+// g_scratch_mutex.
+void verify_placement(int dev, DeviceState& d, hipStream_t stream)
+{
+    if (d.xcd_placement >= 0 || !d.static_scratch) return;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return;
+    }
+    bool ok = true;
+    const hipError_t e = on_device(dev, [&] {
+        unsigned* masks = reinterpret_cast<unsigned*>(d.static_scratch);   // (partial-tile part of the scratch: no contents to keep)
+        static unsigned host[kProbeGroups];
+        const dim3 grids[] = {dim3(8), dim3(264), dim3(8 * kProbeGroups), dim3(40, 5), dim3(272, 2)};
+        hipError_t e2 = hipDeviceSynchronize();                       // nothing in flight may be using the scratch
+        for (const dim3& g : grids) {
+            const unsigned groups = g.x * g.y / 8;
+            if (e2 == hipSuccess) e2 = hipMemsetAsync(masks, 0, sizeof(host), stream);
+            if (e2 != hipSuccess) break;
+            hipLaunchKernelGGL(placement_probe_kernel, g, dim3(64), 0, stream, masks);
+            e2 = hipGetLastError();
+            if (e2 == hipSuccess) e2 = hipStreamSynchronize(stream);
+            if (e2 == hipSuccess) e2 = hipMemcpy(host, masks, sizeof(host), hipMemcpyDeviceToHost);
+            for (unsigned i = 0; i < groups && e2 == hipSuccess; i++) ok = ok && host[i] == 0xffu;
+        }
+        return e2;
+    });
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        ok = false;
+    }
+    d.xcd_placement = ok ? 1 : 0;
+}
+
 inline SliceRule make_rule(int units, int nslices)
 {
     SliceRule r;
@@ -249,6 +299,8 @@ void launch_m16_one(const GemmArgs& a, dim3 grid, hipStream_t stream)
     void (*kernel)(const GemmArgs) = gemm_m16_kernel<G128, AROWS, WN, WK, D4, D6, false, EXTRAS>;
     if constexpr (AROWS == 4) {                                       // (the cells serve up to four rows)
         if (a.cells) kernel = gemm_m16_kernel<G128, AROWS, WN, WK, D4, D6, true, EXTRAS>;
+    } else {                                                          // (beyond, partial tiles: through one XCD's L2 where placed so)
+        if (a.xcd_local) kernel = gemm_m16_kernel<G128, AROWS, WN, WK, D4, D6, false, EXTRAS, true>;
     }
     hipLaunchKernelGGL(kernel, grid, dim3(64 * WN * WK), 0, stream, a);
 }
@@ -355,7 +407,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -369,7 +421,9 @@ int fp6m_init(int dev)
 {
     std::lock_guard<std::mutex> lock(fp6m::g_scratch_mutex);
     fp6m::DeviceState* d = nullptr;
-    return fp6m::device_state(dev, &d);
+    if (int rc = fp6m::device_state(dev, &d)) return rc;
+    fp6m::verify_placement(dev, *d, nullptr);
+    return FP6M_OK;
 }
 
 int fp6m_init_workspace(int dev, const void* workspace, int with_gather)
@@ -479,6 +533,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         return rc;
     }
     const int cus = device->cus;
+    int xcd_placement;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        verify_placement(dev, *device, st);
+        xcd_placement = device->xcd_placement;
+    }
 
     GemmArgs a;
     a.b_int4 = static_cast<const uint32_t*>(B);
@@ -497,6 +557,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.tiles = prob_n / kTileN;
     a.k4 = 0;
     a.slices4 = 0;
+    a.xcd_local = 0;
+    a.xm4_lo = a.xm4_hi = a.xm6_lo = a.xm6_hi = 0;
     if (row_mix) {
         // every tile spans all n columns of both segments: INT4 words of rows [0, k4), then the FP6 planes of the rest
         a.b_fp6_2 = a.b_int4 + (size_t)k4 * prob_n / 8;
@@ -881,13 +943,44 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 a.rule[0] = make_rule(units, a.ks4 * cfg.wk);
                 a.rule[1] = make_rule(units, (a.ks6 > 0 ? a.ks6 : 1) * cfg.wk);
             }
-            const long long wgs = (long long)a.groups6 * a.ks6 + (long long)a.groups4 * a.ks4;
+            long long wgs = (long long)a.groups6 * a.ks6 + (long long)a.groups4 * a.ks4;
             a.div[0] = make_div(a.groups4, wgs);
             a.div[1] = make_div(a.groups6, wgs);
+            // Tiles shared by several workgroups, more than four rows: the workgroups of a tile may be placed on one XCD
+            // (xcd_place in gemm_common.h) and exchange their partial tiles through its L2 instead of through memory:
+            // the publishing stores are acknowledged 0.2-0.3 us earlier and the gather is 0.1-0.2 us shorter.  The grid
+            // is eight times the largest number of workgroups any XCD gets, so a few workgroups have nothing to do,
+            // and the tiles are dealt to the XCDs whole, which leaves the XCDs with an FP6 tile more to do than the others.
+            // Measured (alternating, us): four-wave workgroups gain 2-4 % (4096 x 4096 at 16 rows 8.54 -> 8.35, at 5
+            // rows 8.42 -> 8.11, 11008 x 4096 11.65 -> 11.41, 28672 x 8192 28.25 -> 27.45); eight-wave workgroups,
+            // one per CU, gain nothing where the XCDs' shares stay below their 32 CUs (8192 x 8192 13.1 both) and
+            // lose a whole round where they do not (8192 x 10240 14.1 -> 19.4), so those keep the agent-scope exchange.
+            a.xcd_local = 0;
+            bool want_local = cfg.wk == 4 && a.ks4 > 1;
+            if (tune.xcd != kUnset) want_local = tune.xcd != 0;
+            if (want_local && cfg.id == 1 && cfg.wn == 1 && !a.cells && xcd_placement == 1 && (a.ks4 > 1 || a.ks6 > 1) &&
+                a.ks4 <= kMaxLocalParts && a.ks6 <= kMaxLocalParts) {
+                long long most = 0;
+                for (int x = 0; x < 8; x++) {
+                    const long long c6 = (a.groups6 + 7 - x) >> 3, g0 = (x - a.groups6) & 7, c4 = (a.groups4 + 7 - g0) >> 3;
+                    const long long w = c6 * a.ks6 + c4 * a.ks4;
+                    most = w > most ? w : most;
+                }
+                // (no XCD may get more workgroups than its CUs hold at once: two of four waves each)
+                if (most < 8192 && (tune.xcd != kUnset || 8 * most <= 2LL * cus)) {
+                    a.xcd_local = 1;
+                    wgs = 8 * most;
+                    auto magic32 = [](int d) { return d >= 2 ? (uint32_t)((0x100000000ULL + d - 1) / (unsigned long long)d) : 0u; };
+                    a.xm4_lo = magic32(a.groups4 >> 3);
+                    a.xm4_hi = magic32((a.groups4 >> 3) + 1);
+                    a.xm6_lo = magic32(a.groups6 >> 3);
+                    a.xm6_hi = magic32((a.groups6 >> 3) + 1);
+                }
+            }
             dim3 grid((unsigned)wgs, 1);
             if (tune.verbose)
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u\n", a.m, prob_n,
-                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x);
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u%s\n", a.m, prob_n,
+                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x, a.xcd_local ? " (tiles placed per XCD)" : "");
             launch_m16_any(cfg, a, g128, grid, st);
         } else {
             gather_pass();

@@ -79,6 +79,11 @@ struct GemmArgs {
     const uint16_t* residual; // fp16 [m, n], same rows as C
     int fused;
     unsigned long long* cells;   // m <= 16: the shared tiles' parts meet here instead of in `scratch` (null: they do not)
+    // Workgroups that share a tile placed on one XCD (xcd_tile_of): their partial tiles then meet in that XCD's L2.
+    // xm4_lo / xm4_hi: 2^32 / (INT4 tiles per XCD, rounded down / up); xm6_*: the same for the FP6 tiles.  (Separate
+    // fields, selected by value: an indexed table makes the compiler copy the argument block to scratch memory.)
+    int xcd_local;
+    uint32_t xm4_lo, xm4_hi, xm6_lo, xm6_hi;
 #ifdef FP6M_TIMELINE
     unsigned long long* timeline;   // 8 realtime-clock stamps per workgroup (performance debugging builds only)
 #endif
@@ -125,6 +130,48 @@ __device__ __forceinline__ void preload_args(const GemmArgs& p)
                         "s"(p.ks6), "s"(p.ks4), "s"(p.groups6), "s"(p.groups4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
     asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
                         "s"(p.div[0].d), "s"(p.div[0].magic), "s"(p.div[1].d), "s"(p.div[1].magic), "s"(p.fused));
+    asm volatile("" : : "s"(p.xcd_local), "s"(p.xm4_lo), "s"(p.xm4_hi), "s"(p.xm6_lo), "s"(p.xm6_hi));
+}
+
+// The XCD (accelerator die: 32 CUs with an L2 of their own) this wave runs on.
+__device__ __forceinline__ int xcc_id()
+{
+    int v;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+    return v & 15;
+}
+
+// Placement of a 1-D grid's workgroups so that all k parts of a tile run on one XCD.  The hardware deals the workgroups
+// of a dispatch to the XCDs round robin, starting at an XCD that depends on the queue: workgroups 8i .. 8i + 7 run on
+// eight different XCDs, but which of them runs where is only known to the workgroup itself (XCC_ID).  So a workgroup is
+// identified by (x = the XCD it finds itself on, i = index / 8).  The tile list [FP6 tiles | INT4 tiles] is dealt to
+// the XCDs round robin; XCD x's workgroups, in the order of i, walk its FP6 tiles part-major (ks6 parts each), then
+// its INT4 tiles part-major (ks4 parts each).  The grid is 8 x the largest per-XCD count, so some workgroups are idle.
+// (fp6m_init checks the eight-different-XCDs property on the device before the dispatcher uses this; the reduction
+// itself notices a (tile, part) that arrives twice, see wg_finish.)
+struct XcdPlace {
+    bool valid, fp6;
+    int group, part;         // tile index inside its region, k part
+};
+__device__ __forceinline__ XcdPlace xcd_place(const GemmArgs& p, int b, int tiles6, int tiles4)
+{
+    XcdPlace r;
+    const int x = xcc_id() & 7, i = b >> 3;
+    const int c6 = (tiles6 + 7 - x) >> 3;                   // FP6 tiles f with f % 8 == x
+    const int g0 = (x - tiles6) & 7;                        // first INT4 tile of this XCD
+    const int c4 = (tiles4 + 7 - g0) >> 3;
+    const int w6 = c6 * p.ks6;
+    r.fp6 = i < w6;
+    const int li = r.fp6 ? i : i - w6;
+    const int c = r.fp6 ? c6 : c4;
+    const int lo = (r.fp6 ? tiles6 : tiles4) >> 3;
+    const uint32_t magic_lo = r.fp6 ? p.xm6_lo : p.xm4_lo, magic_hi = r.fp6 ? p.xm6_hi : p.xm4_hi;
+    const uint32_t magic = c == lo ? magic_lo : magic_hi;
+    r.part = c <= 1 ? li : (int)__umulhi((uint32_t)li, magic);
+    const int j = li - r.part * c;
+    r.group = (r.fp6 ? x : g0) + 8 * j;
+    r.valid = c > 0 && r.part < (r.fp6 ? p.ks6 : p.ks4);
+    return r;
 }
 // Epilogue of fp6m_mul_fused for the two adjacent packed columns a lane owns: C[row, c_cols[col]] =
 // fp16(v + bias[c_cols[col]] + residual[row, c_cols[col]]), everything added in fp32 and rounded once.
@@ -366,6 +413,55 @@ __device__ __forceinline__ void dma_a_blocks(uint32_t slot_lds, const void* sbas
         if constexpr (lds_off % 4096 == 0) set_m0(slot_lds + lds_off);
         dma16_m0<lds_off % 4096, false>(sbase_a, voff[I]);
         dma_a_blocks<MB, A_OFF, I + 1>(slot_lds, sbase_a, voff);
+    }
+}
+
+// 8-byte accesses of the partial tiles in scalar-base form: address = sbase + voff + OFF, so a tile's rows and parts
+// cost no vector address arithmetic (the compiler's own code for them was ten instructions and a branch per access,
+// and a last-arriving workgroup spent a microsecond issuing them).  AGENT: the access goes through to memory (visible
+// to every XCD); otherwise it stops at this XCD's L2 and only bypasses the CU's own cache.  The loads are invisible to
+// the compiler's wait insertion: callers wait (vmcnt) and pass the results through settle64 before using them.
+template <int OFF, bool AGENT>
+__device__ __forceinline__ void st8_sbase(const void* sbase, uint32_t voff, unsigned long long v)
+{
+    static_assert(OFF >= 0 && OFF < 4096, "13-bit signed immediate");
+    if constexpr (AGENT)
+        asm volatile("global_store_dwordx2 %0, %1, %2 offset:%3 sc1" : : "v"(voff), "v"(v), "s"(sbase), "n"(OFF) : "memory");
+    else
+        asm volatile("global_store_dwordx2 %0, %1, %2 offset:%3 sc0" : : "v"(voff), "v"(v), "s"(sbase), "n"(OFF) : "memory");
+}
+template <int OFF, bool AGENT>
+__device__ __forceinline__ unsigned long long ld8_sbase(const void* sbase, uint32_t voff)
+{
+    static_assert(OFF >= 0 && OFF < 4096, "13-bit signed immediate");
+    unsigned long long v;
+    if constexpr (AGENT)
+        asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3 sc1" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+    else
+        asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3 sc0" : "=v"(v) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+    return v;
+}
+__device__ __forceinline__ void settle64(unsigned long long& v) { asm volatile("" : "+v"(v)); }
+// The same for byte offset `row_bytes` (a multiple of 2 KiB below 8 KiB, constant once the caller's loop is unrolled)
+// from lane offsets `lo` and `hi` = lo + 4096.
+template <bool AGENT>
+__device__ __forceinline__ void st8_row(const void* sbase, uint32_t lo, uint32_t hi, int row_bytes, unsigned long long v)
+{
+    switch (row_bytes) {
+    case 0: st8_sbase<0, AGENT>(sbase, lo, v); break;
+    case 2048: st8_sbase<2048, AGENT>(sbase, lo, v); break;
+    case 4096: st8_sbase<0, AGENT>(sbase, hi, v); break;
+    default: st8_sbase<2048, AGENT>(sbase, hi, v); break;
+    }
+}
+template <bool AGENT>
+__device__ __forceinline__ unsigned long long ld8_row(const void* sbase, uint32_t lo, uint32_t hi, int row_bytes)
+{
+    switch (row_bytes) {
+    case 0: return ld8_sbase<0, AGENT>(sbase, lo);
+    case 2048: return ld8_sbase<2048, AGENT>(sbase, lo);
+    case 4096: return ld8_sbase<0, AGENT>(sbase, hi);
+    default: return ld8_sbase<2048, AGENT>(sbase, hi);
     }
 }
 

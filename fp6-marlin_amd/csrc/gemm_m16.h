@@ -290,7 +290,15 @@ constexpr int wave_lds_bytes(int d4, int d6, int arows)
 // tile wn over the WK slices (fixed order) with lane L owning columns 2L, 2L+1.  With one k part per
 // tile group it scales and writes C; otherwise it publishes the rows with agent-scope stores, the
 // workgroup bumps the group's counter, and the workgroup that arrives last sums all parts in part order.
-template <int WN, int WK, bool CELLS>
+// LOCAL: every workgroup that shares the tile runs on this XCD (xcd_place), so the partial tiles travel through its
+// L2: stores acknowledged by the L2 and loads that bypass only the CU's own cache, instead of agent-scope accesses that
+// go through to memory and back.  The counter stays an agent-scope atomic (atomics have no narrower scope); here it
+// is a mask of the parts that have arrived rather than their number, so that a part arriving twice -- which would
+// mean that two workgroups of one group of eight ran on the same XCD, against what the placement relies on -- is
+// noticed: the tile is then stored as NaN instead of a sum with a part missing.
+constexpr int kMaxLocalParts = 30;
+constexpr unsigned kPoisoned = 1u << 31;
+template <int WN, int WK, bool CELLS, bool LOCAL = false>
 __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti, bool tile_valid, int wn, int wk,
                                           int ks, int slot_base, int* counter, f4 (&acc)[1][8],
                                           bool per_column_scale, unsigned char* smem, int wave_lds, int* flag,
@@ -410,60 +418,86 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
         return;
     }
 
-    // Publish.  A slot holds [WN tiles][16 rows][128 columns] fp32; 8-byte agent-scope accesses.
-    constexpr size_t kSlotU64 = (size_t)WN * 16 * kTileN / 2;
-    unsigned long long* slot0 = reinterpret_cast<unsigned long long*>(p.scratch) + (size_t)slot_base * kSlotU64 +
-                                (size_t)wn * (16 * kTileN / 2) + lane;
-    unsigned long long* my = slot0 + (size_t)ti.part * kSlotU64;
+    // Publish.  A slot holds [WN tiles][16 rows][128 columns] fp32: row m of a tile is 512 bytes, lane L's column
+    // pair 8 bytes of it.  Rows wk + r * WK of this wave sit WK * 512 bytes apart: immediates below 4 KiB on one of two
+    // lane offsets.
+    constexpr int kSlotBytes = WN * 16 * kTileN * 4;
+    const unsigned char* slot0 = reinterpret_cast<const unsigned char*>(p.scratch) + (size_t)slot_base * kSlotBytes +
+                                 (size_t)wn * (16 * kTileN * 4);
+    const unsigned char* my = uniform_ptr(slot0 + (size_t)ti.part * kSlotBytes);
+    const uint32_t voff_lo = 8 * lane + 512 * wk, voff_hi = voff_lo + 4096;
+    static_assert(WK == 4 || WK == 8, "row offsets of 2 or 4 KiB");
+    if (tile_valid) {
 #pragma unroll
-    for (int r = 0; r < RMAX; r++) {
-        const int m = wk + r * WK;
-        if (tile_valid && m < nrows) {
-            const f2 v = {v0[r], v1[r]};
-            __hip_atomic_store(my + m * (kTileN / 2), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-        }
+        for (int r = 0; r < RMAX; r++)
+            if (wk + r * WK < nrows) {                                   // (uniform)
+                const f2 v = {v0[r], v1[r]};
+                st8_row<!LOCAL>(my, voff_lo, voff_hi, r * WK * 512, __builtin_bit_cast(unsigned long long, v));
+            }
     }
-    // Every wave waits until its own partial-sum stores are acknowledged (they are agent-scope write-through stores:
-    // the acknowledgement means they are visible to every other CU), and only then joins the barrier in front of
-    // the counter increment.  A workgroup-scope fence alone would not wait for them, and neither does s_barrier.
+    // Every wave waits until its own partial-sum stores are acknowledged (agent scope: written through to memory and
+    // so visible to every other CU; XCD-local: by this XCD's L2, which every reader of the tile shares), and only then
+    // joins the barrier in front of the counter increment.  A workgroup-scope fence alone would not wait for them, and
+    // neither does s_barrier.
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");               // (keeps the compiler from moving accesses across)
     __syncthreads();
     FP6M_MARK(p, 4);
     if (threadIdx.x == 0) {
-        const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *flag = (seen == ks - 1);
+        if constexpr (LOCAL) {
+            const unsigned mine = 1u << ti.part, all = (1u << ks) - 1;
+            const unsigned seen = __hip_atomic_fetch_or(reinterpret_cast<unsigned*>(counter), mine, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+            if (seen & mine) {                                           // this part has been here before
+                __hip_atomic_fetch_or(reinterpret_cast<unsigned*>(counter), kPoisoned, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *flag = 2;
+            } else {
+                *flag = ((seen | mine) & all) == all ? ((seen & kPoisoned) ? 2 : 1) : 0;
+            }
+        } else {
+            const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = seen == ks - 1;
+        }
     }
     __syncthreads();
     FP6M_MARK(p, 5);
-    if (!*flag) return;
+    const int finish = *flag;
+    if (!finish) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll
     for (int r = 0; r < RMAX; r++) {
         v0[r] = 0.f;
         v1[r] = 0.f;
     }
+    // Gather: the loads of up to PCHUNK parts in flight together (rows past m are read too, they lie inside the slot,
+    // and never stored), then the sums in part order.
+    const unsigned char* part0 = uniform_ptr(slot0);
     for (int pp = 0; pp < ks; pp += PCHUNK) {
         unsigned long long t[PCHUNK][RMAX];
 #pragma unroll
         for (int u = 0; u < PCHUNK; u++)
+            if (tile_valid && pp + u < ks) {                             // (uniform)
+                const unsigned char* src = part0 + (size_t)(pp + u) * kSlotBytes;
 #pragma unroll
-            for (int r = 0; r < RMAX; r++) {
-                const int m = wk + r * WK;
-                t[u][r] = 0;
-                if (tile_valid && m < nrows && pp + u < ks)
-                    t[u][r] = __hip_atomic_load(slot0 + (size_t)(pp + u) * kSlotU64 + m * (kTileN / 2), __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
+                for (int r = 0; r < RMAX; r++) t[u][r] = ld8_row<!LOCAL>(src, voff_lo, voff_hi, r * WK * 512);
             }
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
 #pragma unroll
         for (int u = 0; u < PCHUNK; u++)
+            if (tile_valid && pp + u < ks) {
 #pragma unroll
-            for (int r = 0; r < RMAX; r++) {
-                const f2 v = __builtin_bit_cast(f2, t[u][r]);
-                v0[r] += v[0];
-                v1[r] += v[1];
+                for (int r = 0; r < RMAX; r++) {
+                    settle64(t[u][r]);
+                    const f2 v = __builtin_bit_cast(f2, t[u][r]);
+                    v0[r] += v[0];
+                    v1[r] += v[1];
+                }
             }
+    }
+    if (LOCAL && finish == 2) {                                          // (see above: never on a device that fp6m_init has looked at)
+        const float nan = __builtin_nanf("");
+#pragma unroll
+        for (int r = 0; r < RMAX; r++) v0[r] = v1[r] = nan;
     }
 #pragma unroll
     for (int r = 0; r < RMAX; r++)
@@ -477,10 +511,12 @@ __device__ __forceinline__ void wg_finish(const GemmArgs& p, const TileInfo& ti,
 // run-time branch cost the partial-tile path 0.3-0.6 us (4096 x 4096 at 16 rows: 8.9 -> 9.4 us).
 // EXTRAS = false: the build for calls without row mix, fused epilogue or gfx950 word order (their arguments are
 // overwritten with constants; their presence cost the plain call 2-3 %).
-template <bool G128, int AROWS, int WN, int WK, int D4, int D6, bool CELLS, bool EXTRAS = true>
+// LOCAL: the workgroups of a tile are placed on one XCD and exchange their partial tiles through its L2.
+template <bool G128, int AROWS, int WN, int WK, int D4, int D6, bool CELLS, bool EXTRAS = true, bool LOCAL = false>
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
 __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void gemm_m16_kernel(const GemmArgs args)
 {
+    static_assert(!LOCAL || (WN == 1 && !CELLS), "the cells are atomics, which have no XCD-local form");
     constexpr int NW = WN * WK;
     constexpr int kWaveLds = wave_lds_bytes(D4, D6, AROWS);
     __shared__ __attribute__((aligned(16))) unsigned char smem[NW * kWaveLds + 16];
@@ -499,19 +535,28 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
     FP6M_MARK(p, 0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
     const int wn = wave % WN, wk = wave / WN;
-    const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    const int wgs6 = p.groups6 * p.ks6;                                  // the FP6 region's workgroups come first
     TileInfo ti;
-    ti.fp6 = logical < wgs6;
-    const int local = ti.fp6 ? logical : logical - wgs6;
-    const int groups = ti.fp6 ? p.groups6 : p.groups4;
+    int group;
+    if constexpr (LOCAL) {
+        const XcdPlace pl = xcd_place(p, blockIdx.x, p.groups6, p.groups4);
+        if (!pl.valid) return;                                           // (the grid is padded to a multiple of eight)
+        ti.fp6 = pl.fp6;
+        ti.part = pl.part;
+        group = pl.group;
+    } else {
+        const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+        const int wgs6 = p.groups6 * p.ks6;                              // the FP6 region's workgroups come first
+        ti.fp6 = logical < wgs6;
+        const int local = ti.fp6 ? logical : logical - wgs6;
+        const int groups = ti.fp6 ? p.groups6 : p.groups4;
+        // (both entries are read at fixed kernarg offsets and selected by value: an index computed here would turn
+        // into a second, dependent scalar load, which measured 0.4 us before the first weight load)
+        const FastDiv gdiv = {ti.fp6 ? p.div[1].d : p.div[0].d, ti.fp6 ? p.div[1].magic : p.div[0].magic};
+        ti.part = fast_div(gdiv, local);                                 // part-major: neighbours share k, adjoin in n
+        group = local - ti.part * groups;
+    }
     const int ks = ti.fp6 ? p.ks6 : p.ks4;
-    // (both entries are read at fixed kernarg offsets and selected by value: an index computed here would turn
-    // into a second, dependent scalar load, which measured 0.4 us before the first weight load)
-    const FastDiv gdiv = {ti.fp6 ? p.div[1].d : p.div[0].d, ti.fp6 ? p.div[1].magic : p.div[0].magic};
     const SliceRule srule = {ti.fp6 ? p.rule[1].q : p.rule[0].q, ti.fp6 ? p.rule[1].first_long : p.rule[0].first_long};
-    ti.part = fast_div(gdiv, local);                                     // part-major: neighbours share k, adjoin in n
-    const int group = local - ti.part * groups;
     ti.tcol = group * WN + wn;
     ti.region_n = ti.fp6 ? p.qc : p.n4;
     const bool tile_valid = ti.tcol * kTileN < ti.region_n;
@@ -541,8 +586,9 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
     // scratch slots: FP6 groups first (groups6 * ks6 slots), then INT4 groups; counters likewise
     const int slot_base = region6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
     int* counter = p.counters + (region6 ? group : p.groups6 + group);
-    wg_finish<WN, WK, CELLS>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem, kWaveLds,
-                      reinterpret_cast<int*>(smem + NW * kWaveLds), p.k4 ? p.slices4 - ti.part * WK : WK);
+    wg_finish<WN, WK, CELLS, LOCAL>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem,
+                                    kWaveLds, reinterpret_cast<int*>(smem + NW * kWaveLds),
+                                    p.k4 ? p.slices4 - ti.part * WK : WK);
     FP6M_MARK(p, 7);
 }
 

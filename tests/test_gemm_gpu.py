@@ -169,6 +169,57 @@ def test_cells_and_partial_tiles_up_to_sixteen_rows(oracle):
     assert ulps.max() <= 1 and (ulps != 0).mean() < 0.01, (ulps.max(), (ulps != 0).mean())
 
 
+def test_partial_tiles_exchanged_through_one_xcd(oracle):
+    """5 .. 16 rows: the workgroups that share a tile may be placed on one XCD and exchange their partial tiles through its
+    L2 (`xcd` knob: 1 forces the placement, 0 the agent-scope exchange).  Same sums in the same order: the results
+    must agree bit for bit -- for tile counts that do and do not divide by the eight XCDs, several split factors
+    (forced and the dispatcher's own), both scale modes, all FP6; on the default stream, on a side stream and from a
+    replayed HIP graph (the XCD that a dispatch's first workgroup runs on differs between them)."""
+    import fp6_marlin
+    for (m, n, k, qc, gs, ks) in [(16, 512, 2048, 256, 128, None), (16, 1024, 2048, 256, -1, 4), (5, 1280, 1024, 256, 128, 3),
+                                  (9, 2304, 1024, 512, 128, 2), (16, 4096, 1024, 256, 128, None), (8, 512, 2048, 512, -1, 6),
+                                  (16, 1152, 4096, 128, 128, 16), (12, 3072, 512, 256, -1, 2)]:
+        a = run(oracle, m, n, k, qc=qc, gs=gs, ksplit=ks, env={"FP6M_XCD": 0})
+        b = run(oracle, m, n, k, qc=qc, gs=gs, ksplit=ks, env={"FP6M_XCD": 1})
+        assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), (m, n, k, qc, gs, ks)
+    one_hot_case(oracle, 16, 1024, 2048, 256, 128, {"xcd": 1, "ksplit": 4})
+    one_hot_case(oracle, 7, 768, 1024, 256, -1, {"xcd": 1, "ksplit": 2})
+    # other streams, and a captured graph replayed several times with eager work in between
+    m, n, k, qc, gs = 16, 2048, 2048, 256, 128
+    ref, B, s = problem(oracle, n, k, qc, gs)
+    A = torch.randn((m, k), generator=torch.Generator().manual_seed(5), dtype=torch.float32).half().to(dev())
+    ws = fp6_marlin.init_workspace(torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev()))
+    outs = {}
+    for xcd in (0, 1):
+        with fp6_marlin.cabi.tuning(xcd=xcd, ksplit=4):
+            C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+            fp6_marlin.mul(A, B, C, s, ws, qc, -1, -1, -1, 16, gs)
+            torch.cuda.synchronize()
+            outs[xcd] = C.clone()
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                C.fill_(float("nan"))
+                fp6_marlin.mul(A, B, C, s, ws, qc, -1, -1, -1, 16, gs)
+            side.synchronize()
+            assert torch.equal(C, outs[xcd]), f"side stream, xcd={xcd}"
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fp6_marlin.mul(A, B, C, s, ws, qc, -1, -1, -1, 16, gs)
+            for _ in range(3):
+                C.fill_(float("nan"))
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(C, outs[xcd]), f"graph replay, xcd={xcd}"
+                C.fill_(float("nan"))
+                fp6_marlin.mul(A, B, C, s, ws, qc, -1, -1, -1, 16, gs)   # eager, after a capture
+                torch.cuda.synchronize()
+                assert torch.equal(C, outs[xcd]), f"eager after capture, xcd={xcd}"
+    assert torch.equal(outs[0], outs[1])
+    assert int(ws.abs().sum().item()) == 0
+    c_ref = oracle.matmul_ref(A.cpu().numpy(), ref)
+    assert oracle.rel_err(outs[1].cpu().numpy(), c_ref) <= TOL
+
+
 def test_shared_fragment_kernel(oracle):
     """The kernel that large launches use (four row tiles share a tile's dequantised fragments; one or two
     column tiles per workgroup), forced onto small problems: ragged row tiles, odd tile counts in both regions,

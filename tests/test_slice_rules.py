@@ -105,3 +105,62 @@ def test_forty_bit_reciprocal_division_is_exact_in_its_range():
         assert magic < (1 << 41)
         got = (ns * np.uint64(magic)) >> np.uint64(40)              # n < 2^24, magic < 2^41: no overflow of 64 bits
         assert (got == ns // np.uint64(d)).all(), d
+
+
+# ---- placement of the workgroups that share a tile on one XCD (gemm_common.h: xcd_place; fp6m_gemm.hip: the grid and
+# the multiply-high constants of the m <= 16 launch).  A workgroup knows the XCD it runs on from the hardware; the only
+# thing assumed about the dispatch is that workgroups 8i .. 8i+7 run on eight different XCDs, in any order.
+
+def xcd_grid(tiles6, tiles4, ks6, ks4):
+    most = 0
+    for x in range(8):
+        c6 = (tiles6 + 7 - x) >> 3
+        g0 = (x - tiles6) & 7
+        c4 = (tiles4 + 7 - g0) >> 3
+        most = max(most, c6 * ks6 + c4 * ks4)
+    per = (tiles4 >> 3, tiles6 >> 3)
+    xmagic = [[((2 ** 32 + (per[r] + h) - 1) // (per[r] + h)) if per[r] + h >= 2 else 0 for h in range(2)] for r in range(2)]
+    return 8 * most, xmagic
+
+
+def xcd_place(b, x, tiles6, tiles4, ks6, ks4, xmagic):
+    i = b >> 3
+    c6 = (tiles6 + 7 - x) >> 3
+    g0 = (x - tiles6) & 7
+    c4 = (tiles4 + 7 - g0) >> 3
+    w6 = c6 * ks6
+    fp6 = i < w6
+    li = i if fp6 else i - w6
+    c = c6 if fp6 else c4
+    lo = (tiles6 if fp6 else tiles4) >> 3
+    magic = xmagic[1 if fp6 else 0][0 if c == lo else 1]
+    part = li if c <= 1 else (li * magic) >> 32
+    j = li - part * c
+    group = (x if fp6 else g0) + 8 * j
+    valid = c > 0 and part < (ks6 if fp6 else ks4)
+    return valid, fp6, group, part, x
+
+
+def test_xcd_placement_covers_every_tile_part_once_on_one_xcd():
+    cases = [(t6, t4, k6, k4) for t6 in (0, 1, 2, 3, 4, 7, 8, 9, 17) for t4 in (0, 1, 5, 8, 30, 62, 78, 94, 170, 447)
+             for (k6, k4) in ((1, 1), (2, 1), (4, 2), (16, 8), (6, 3), (5, 7), (1, 4))]
+    for tiles6, tiles4, ks6, ks4 in cases:
+        if tiles6 + tiles4 == 0:
+            continue
+        grid, xmagic = xcd_grid(tiles6, tiles4, ks6, ks4)
+        seen = {}
+        rng = np.random.default_rng(tiles6 * 1000 + tiles4)
+        # XCD of every workgroup: a rotation per dispatch (what the hardware does) or any permutation per group of eight
+        xcd_of = np.concatenate([rng.permutation(8) if tiles4 % 2 else (np.arange(8) + tiles6) % 8 for _ in range(grid // 8)])
+        for b in range(grid):
+            valid, fp6, group, part, x = xcd_place(b, int(xcd_of[b]), tiles6, tiles4, ks6, ks4, xmagic)
+            if not valid:
+                continue
+            assert 0 <= group < (tiles6 if fp6 else tiles4) and 0 <= part < (ks6 if fp6 else ks4)
+            key = (fp6, group, part)
+            assert key not in seen, (tiles6, tiles4, ks6, ks4, b)
+            seen[key] = x
+        assert len(seen) == tiles6 * ks6 + tiles4 * ks4, (tiles6, tiles4, ks6, ks4)
+        for (fp6, group, part), x in seen.items():                                   # all parts of a tile on one XCD
+            assert x == seen[(fp6, group, 0)]
+        assert grid <= 8 * (-(-(tiles6 * ks6 + tiles4 * ks4) // 8) + max(ks6, ks4) * 2)   # little padding
