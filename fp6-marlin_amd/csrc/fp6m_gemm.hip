@@ -74,20 +74,29 @@ struct Tuning {
 Tuning g_tuning;
 
 // Device memory the GEMM needs beyond its operands: fp32 partial tiles of column tiles whose k range is shared by
-// several workgroups, and the buffer that gathered activations pass through.  The reference keeps its partial sums
-// in C under the locks in the caller's `workspace`, so its rule is one call at a time per workspace, and two calls
-// with two workspaces may overlap.  Here the rule is the same because the scratch belongs to the workspace: every
-// workspace address that has been seen on a device owns a region, allocated on its first call (or by
-// fp6m_init_workspace) and kept until fp6m_release_workspace.  The table is bounded; when it is full the library
-// waits for the device and frees every region, which is safe because nothing is in flight then.
+// several workgroups, the accumulate-and-count cells, and the buffer that gathered activations pass through.  The
+// reference keeps its partial sums in C under the locks in the caller's `workspace`, so its rule is one call at a
+// time per workspace, and two calls with two workspaces may overlap.  Here the rule is the same because the scratch
+// belongs to the workspace: every workspace address that is in use on a device owns a region.  A device has
+// kMaxRegions of them.  The first kStaticSlots are slots of a file-scope device array, so an ordinary call allocates
+// nothing and never waits for the device; the others get their memory from hipMalloc (synchronous) when a fifth,
+// sixth .. workspace turns up, and keep it: memory that a captured graph may hold the address of is never freed
+// behind the caller's back.  When every region is taken, the one whose workspace has gone unused longest is handed
+// to the newcomer after a hipDeviceSynchronize (callers that make a new workspace per call, as the reference's own
+// test.py:168 and bench.py:44 do, never run out); a call that is being captured cannot wait and is refused instead.
 struct Region {
-    const void* workspace = nullptr;
+    const void* workspace = nullptr;   // null: nobody's
     float* partials = nullptr;      // kScratchBytes of partial tiles (m > 16, row mix), then kCellBytes of cells (m <= 16)
-    uint16_t* gathered = nullptr;   // kGatherBytes, allocated by the first gathering call with this workspace
+    uint16_t* gathered = nullptr;   // kGatherBytes, allocated by the first gathering call that gets this region
+    unsigned long long last_use = 0;
+    int pins = 0;                   // host threads between looking the region up and having launched with it
 };
 constexpr size_t kGatherBytes = size_t(64) << 20;
 constexpr int kMaxDevices = 64;
-constexpr int kMaxRegions = 128;    // per device
+constexpr int kMaxRegions = 16;     // per device
+constexpr int kStaticSlots = 4;     // of them in the code object's own memory
+constexpr size_t kRegionBytes = kScratchBytes + kCellBytes;
+static __device__ __align__(256) unsigned char g_slot_scratch[kStaticSlots * kRegionBytes];   // (zero when loaded, like a fresh region)
 // Partial-tile scratch of fp6m_mul_static, the entry point for callers that must not allocate: part of the loaded
 // code object, so every GPU the library runs on holds its own copy until the process ends.  In host code the
 // array's name is only a handle; its device address is looked up once per device (device_state) and kept there.
@@ -99,7 +108,8 @@ struct DeviceState {
     int cus = 0;
     int xcd_placement = -1;            // 1: workgroup b of a grid runs on XCD b % 8 (verified by verify_placement), 0: not so, -1: not looked at yet
     float* static_scratch = nullptr;   // device address of this GPU's copy of g_static_scratch
-    int nregions = 0;
+    unsigned char* slot_scratch = nullptr;   // ... and of g_slot_scratch
+    unsigned long long tick = 0;
     void* pack_temp = nullptr;      // kPackTempBytes for the on-GPU packer's flag and column maxima
     Region regions[kMaxRegions];
 };
@@ -133,90 +143,20 @@ int device_state(int dev, DeviceState** out)
     DeviceState& d = g_devices[dev];
     if (!d.cus) {
         int cus = 0;
-        void* sym = nullptr;
+        void *sym = nullptr, *slots = nullptr;
         const hipError_t e = on_device(dev, [&] {
             hipError_t e2 = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
             if (e2 == hipSuccess) e2 = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_static_scratch));
+            if (e2 == hipSuccess) e2 = hipGetSymbolAddress(&slots, HIP_SYMBOL(g_slot_scratch));
             return e2;
         });
         if (e != hipSuccess) return hip_fail(e);
-        if (!sym) return hip_fail(hipErrorInvalidSymbol);
+        if (!sym || !slots) return hip_fail(hipErrorInvalidSymbol);
         d.static_scratch = static_cast<float*>(sym);
+        d.slot_scratch = static_cast<unsigned char*>(slots);
         d.cus = cus > 0 ? cus : 256;
     }
     *out = &d;
-    return FP6M_OK;
-}
-
-// Frees every region of the device after waiting for it.  Callers hold g_scratch_mutex.
-hipError_t free_regions(int dev, DeviceState& d)
-{
-    return on_device(dev, [&] {
-        hipError_t e = hipDeviceSynchronize();
-        for (int i = 0; i < d.nregions && e == hipSuccess; i++) {
-            e = hipFree(d.regions[i].partials);
-            if (e == hipSuccess && d.regions[i].gathered) e = hipFree(d.regions[i].gathered);
-            d.regions[i] = Region{};
-        }
-        if (e == hipSuccess) d.nregions = 0;
-        return e;
-    });
-}
-
-// The region of `workspace` on `dev`; the first call for an address allocates it (zeroed: the reduction protocols
-// leave what they use zeroed and rely on finding it so).
-int workspace_region(int dev, const void* workspace, bool want_gather, DeviceState** dev_out, Region** out)
-{
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    DeviceState* d = nullptr;
-    if (int rc = device_state(dev, &d)) return rc;
-    Region* r = nullptr;
-    for (int i = 0; i < d->nregions; i++)
-        if (d->regions[i].workspace == workspace) r = &d->regions[i];
-    if (!r) {
-        if (d->nregions == kMaxRegions) {
-            const hipError_t e = free_regions(dev, *d);
-            if (e != hipSuccess) return hip_fail(e);
-        }
-        void* mem = nullptr;
-        const hipError_t e = on_device(dev, [&] {
-            hipError_t e2 = hipMalloc(&mem, kScratchBytes + kCellBytes);
-            if (e2 == hipSuccess) e2 = hipMemset(mem, 0, kScratchBytes + kCellBytes);
-            return e2;
-        });
-        if (e != hipSuccess) {
-            if (mem) (void)hipFree(mem);
-            return hip_fail(e);
-        }
-        r = &d->regions[d->nregions++];
-        r->workspace = workspace;
-        r->partials = static_cast<float*>(mem);
-        r->gathered = nullptr;
-    }
-    if (want_gather && !r->gathered) {
-        void* mem = nullptr;
-        const hipError_t e = on_device(dev, [&] { return hipMalloc(&mem, kGatherBytes); });
-        if (e != hipSuccess) return hip_fail(e);
-        r->gathered = static_cast<uint16_t*>(mem);
-    }
-    *dev_out = d;
-    *out = r;
-    return FP6M_OK;
-}
-
-// Scratch of the on-GPU packer (fp6m_pack.hip): one buffer per device (a pack call waits for its kernels).
-int pack_temp(int dev, void** ptr)
-{
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    DeviceState* d = nullptr;
-    if (int rc = device_state(dev, &d)) return rc;
-    if (!d->pack_temp) {
-        void* mem = nullptr;
-        const hipError_t e = on_device(dev, [&] { return hipMalloc(&mem, kPackTempBytes); });
-        if (e != hipSuccess) return hip_fail(e);
-        d->pack_temp = mem;
-    }
-    *ptr = d->pack_temp;
     return FP6M_OK;
 }
 
@@ -267,6 +207,118 @@ void verify_placement(int dev, DeviceState& d, hipStream_t stream)
         ok = false;
     }
     d.xcd_placement = ok ? 1 : 0;
+}
+
+// What a call needs to know about its device and its workspace's region, by value: the table may change under
+// another thread as soon as the lock is dropped (the region itself is pinned until the call has launched).
+struct Scratch {
+    int dev = -1, region = -1;
+    int cus = 0;
+    float* static_scratch = nullptr;
+    float* partials = nullptr;
+    uint16_t* gathered = nullptr;
+    int xcd_placement = 0;
+    ~Scratch()
+    {
+        if (region < 0) return;
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        g_devices[dev].regions[region].pins--;
+    }
+};
+
+bool capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;                                                  // (cannot tell: do nothing that a capture forbids)
+    }
+    return cap != hipStreamCaptureStatusNone;
+}
+
+// The region of `workspace` on `dev`, pinned until `out` goes out of scope.  A workspace that has none takes, in this
+// order: a region nobody owns that has memory (the built-in slots always do), one without memory (hipMalloc +
+// hipMemset, synchronous: the reduction protocols leave what they use zeroed and rely on finding it so), or the
+// unpinned region that has gone unused longest, after waiting for the device.  The last two are refused
+// (FP6M_ERR_SCRATCH) while `stream` is being captured.
+int workspace_region(int dev, const void* workspace, bool want_region, bool want_gather, hipStream_t stream, Scratch* out)
+{
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    DeviceState* d = nullptr;
+    if (int rc = device_state(dev, &d)) return rc;
+    verify_placement(dev, *d, stream);
+    out->cus = d->cus;
+    out->static_scratch = d->static_scratch;
+    out->xcd_placement = d->xcd_placement;
+    if (!want_region) return FP6M_OK;
+    for (int i = 0; i < kStaticSlots; i++)
+        if (!d->regions[i].partials) d->regions[i].partials = reinterpret_cast<float*>(d->slot_scratch + (size_t)i * kRegionBytes);
+    Region* r = nullptr;
+    for (Region& c : d->regions)
+        if (c.workspace == workspace) r = &c;
+    if (!r) {
+        Region *idle = nullptr, *bare = nullptr, *oldest = nullptr;
+        for (Region& c : d->regions) {
+            if (!c.workspace && c.partials && !idle) idle = &c;
+            if (!c.workspace && !c.partials && !bare) bare = &c;
+            if (c.workspace && !c.pins && (!oldest || c.last_use < oldest->last_use)) oldest = &c;
+        }
+        if (idle) {
+            r = idle;
+        } else if (capturing(stream)) {
+            return FP6M_ERR_SCRATCH;
+        } else if (bare) {
+            void* mem = nullptr;
+            const hipError_t e = on_device(dev, [&] {
+                hipError_t e2 = hipMalloc(&mem, kRegionBytes);
+                if (e2 == hipSuccess) e2 = hipMemset(mem, 0, kRegionBytes);
+                return e2;
+            });
+            if (e != hipSuccess) {
+                if (mem) (void)hipFree(mem);
+                return hip_fail(e);
+            }
+            bare->partials = static_cast<float*>(mem);
+            r = bare;
+        } else if (oldest) {
+            const hipError_t e = on_device(dev, [&] { return hipDeviceSynchronize(); });   // nothing in flight uses it now
+            if (e != hipSuccess) return hip_fail(e);
+            r = oldest;
+        } else {
+            return FP6M_ERR_SCRATCH;                                  // (every region pinned by a call in progress)
+        }
+        r->workspace = workspace;
+    }
+    if (want_gather && !r->gathered) {
+        if (capturing(stream)) return FP6M_ERR_SCRATCH;
+        void* mem = nullptr;
+        const hipError_t e = on_device(dev, [&] { return hipMalloc(&mem, kGatherBytes); });
+        if (e != hipSuccess) return hip_fail(e);
+        r->gathered = static_cast<uint16_t*>(mem);
+    }
+    r->last_use = ++d->tick;
+    r->pins++;
+    out->dev = dev;
+    out->region = (int)(r - d->regions);
+    out->partials = r->partials;
+    out->gathered = r->gathered;
+    return FP6M_OK;
+}
+
+// Scratch of the on-GPU packer (fp6m_pack.hip): one buffer per device (a pack call waits for its kernels).
+int pack_temp(int dev, void** ptr)
+{
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    DeviceState* d = nullptr;
+    if (int rc = device_state(dev, &d)) return rc;
+    if (!d->pack_temp) {
+        void* mem = nullptr;
+        const hipError_t e = on_device(dev, [&] { return hipMalloc(&mem, kPackTempBytes); });
+        if (e != hipSuccess) return hip_fail(e);
+        d->pack_temp = mem;
+    }
+    *ptr = d->pack_temp;
+    return FP6M_OK;
 }
 
 inline SliceRule make_rule(int units, int nslices)
@@ -419,19 +471,15 @@ int fp6m_tuning_set(const char* knob, int value)
 
 int fp6m_init(int dev)
 {
-    std::lock_guard<std::mutex> lock(fp6m::g_scratch_mutex);
-    fp6m::DeviceState* d = nullptr;
-    if (int rc = fp6m::device_state(dev, &d)) return rc;
-    fp6m::verify_placement(dev, *d, nullptr);
-    return FP6M_OK;
+    fp6m::Scratch sc;
+    return fp6m::workspace_region(dev, nullptr, false, false, nullptr, &sc);
 }
 
 int fp6m_init_workspace(int dev, const void* workspace, int with_gather)
 {
     if (!workspace) return FP6M_ERR_ARG;
-    fp6m::DeviceState* d = nullptr;
-    fp6m::Region* r = nullptr;
-    return fp6m::workspace_region(dev, workspace, with_gather != 0, &d, &r);
+    fp6m::Scratch sc;
+    return fp6m::workspace_region(dev, workspace, true, with_gather != 0, nullptr, &sc);
 }
 
 int fp6m_release_workspace(int dev, const void* workspace)
@@ -440,23 +488,16 @@ int fp6m_release_workspace(int dev, const void* workspace)
     if (dev < 0 || dev >= kMaxDevices) return FP6M_ERR_ARG;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     DeviceState& d = g_devices[dev];
-    if (!workspace) {                                                 // all regions of the device
-        const hipError_t e = free_regions(dev, d);
-        return e == hipSuccess ? FP6M_OK : hip_fail(e);
-    }
-    for (int i = 0; i < d.nregions; i++) {
-        if (d.regions[i].workspace != workspace) continue;
-        const Region r = d.regions[i];
-        const hipError_t e = on_device(dev, [&] {
-            hipError_t e2 = hipDeviceSynchronize();                   // nothing in flight may still use the region
-            if (e2 == hipSuccess) e2 = hipFree(r.partials);
-            if (e2 == hipSuccess && r.gathered) e2 = hipFree(r.gathered);
-            return e2;
-        });
-        if (e != hipSuccess) return hip_fail(e);
-        d.regions[i] = d.regions[--d.nregions];
-        d.regions[d.nregions] = Region{};
-        return FP6M_OK;
+    bool waited = false;
+    for (Region& r : d.regions) {                                     // workspace = NULL: every region of the device
+        if (!r.workspace || (workspace && r.workspace != workspace)) continue;
+        if (r.pins) return FP6M_ERR_ARG;                              // a call with this workspace is being made right now
+        if (!waited) {                                                // nothing in flight may still use the region
+            const hipError_t e = on_device(dev, [&] { return hipDeviceSynchronize(); });
+            if (e != hipSuccess) return hip_fail(e);
+            waited = true;
+        }
+        r.workspace = nullptr;                                        // (its memory stays with the region for the next owner)
     }
     return FP6M_OK;                                                   // no region: nothing to release
 }
@@ -521,24 +562,16 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     if (g128 && prob_k % 128 && !row_mix) return FP6M_ERR_PROB_SHAPE;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
-    DeviceState* device = nullptr;
-    Region* region = nullptr;
+    Scratch sc;
     size_t scratch_bytes = kScratchBytes;
     if (fixed_scratch) {
         if (fu.a_cols) return FP6M_ERR_ARG;                           // the gathered activations need a region's buffer
-        std::lock_guard<std::mutex> lock(g_scratch_mutex);
-        if (int rc = device_state(dev, &device)) return rc;
         scratch_bytes = kStaticTileBytes;
-    } else if (int rc = workspace_region(dev, workspace, fu.a_cols != nullptr, &device, &region)) {
-        return rc;
     }
-    const int cus = device->cus;
-    int xcd_placement;
-    {
-        std::lock_guard<std::mutex> lock(g_scratch_mutex);
-        verify_placement(dev, *device, st);
-        xcd_placement = device->xcd_placement;
-    }
+    if (int rc = workspace_region(dev, workspace, !fixed_scratch, fu.a_cols != nullptr, st, &sc)) return rc;
+    const int cus = sc.cus;
+    const int xcd_placement = sc.xcd_placement;
+    float* const scratch = fixed_scratch ? sc.static_scratch : sc.partials;
 
     GemmArgs a;
     a.b_int4 = static_cast<const uint32_t*>(B);
@@ -546,7 +579,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.b_fp6_4 = a.b_fp6_2 + (size_t)prob_k * qc / 16;
     a.s_int4 = static_cast<const uint16_t*>(s);
     a.s_fp6 = a.s_int4 + (g128 ? (size_t)(prob_k / 128) * n4 : (size_t)n4);
-    a.scratch = fixed_scratch ? device->static_scratch : region->partials;
+    a.scratch = scratch;
     a.counters = static_cast<int*>(workspace);
     a.cells = nullptr;
     a.n = prob_n;
@@ -624,7 +657,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         const long long ks8 = wgs8 > 0 ? cus / wgs8 : 0;
         if (mb == 4 && wgs4 <= cus && 2 * wgs4 > cus && prob_k >= 10240 && ks8 >= 2 && 4 * wgs8 * ks8 >= 3 * cus &&
             wgs8 * ks8 >= wgs4 && ks8 <= prob_k / (16LL * 128) &&
-            (size_t)(tiles_n + qc / kTileN) * ((rows8 + 127) / 128) * ks8 * (8 * 16 * kTileN * sizeof(float)) <= kScratchBytes)
+            (size_t)(tiles_n + qc / kTileN) * ((rows8 + 127) / 128) * ks8 * (8 * 16 * kTileN * sizeof(float)) <= scratch_bytes)
             mb = 8;
     }
     const int rows_per_tile = 16 * mb;
@@ -648,8 +681,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         auto gather_pass = [&]() {
             if (!fu.a_cols) return;
             dim3 ggrid((unsigned)((prob_k / 2 + 255) / 256), (unsigned)a.m);
-            hipLaunchKernelGGL(gather_a_kernel, ggrid, dim3(256), 0, st, a.A, fu.lda, fu.a_cols, region->gathered, prob_k);
-            a.A = region->gathered;
+            hipLaunchKernelGGL(gather_a_kernel, ggrid, dim3(256), 0, st, a.A, fu.lda, fu.a_cols, sc.gathered, prob_k);
+            a.A = sc.gathered;
         };
 
         const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
@@ -686,7 +719,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         a.m, prob_n, prob_k, wn, wk, mtiles, a.ksplit, grid.x, grid.y);
             fp6m::launch_wm(a, g128, wn, grid, st);
         } else if (mb == 1 && !row_mix && (tune.sk != kUnset ? tune.sk != 0 && a.m <= 4 : a.m == 1) && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24) &&
-                   (long long)prob_k * prob_n / 2 < (1LL << 32) && (long long)(prob_n / 128) * max_par >= 2) {
+                   (long long)prob_k * prob_n / 2 < (1LL << 32) && (long long)(prob_n / 128) * max_par >= 2 &&
+                   (g128 || n4 == 0 || units >= 2)) {
+            // (k = 64 with per-column scales stays with the workgroup kernel: an INT4 chunk of that single unit is two
+            // steps, shorter than the three the fetch side runs ahead, which the drawn-chunk variant cannot follow)
             // One row (decode), weight mixed along n: one wave per workgroup, equal shares of every region's (tile,
             // k unit) list (gemm_sk.h).  The kernel takes up to four rows, but every wave adds its part of a shared
             // tile with one atomic per element, and from two rows on that traffic costs more than the barriers and

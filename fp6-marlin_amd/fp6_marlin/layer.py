@@ -106,20 +106,22 @@ def pack_row_mix_weight(w, quant_rows):
 _workspaces = {}
 
 
-def shared_workspace(device, elems):
-    """The zeroed int32 workspace that every ``Layer.forward`` on `device`'s current stream uses: calls on one stream
-    never overlap, so they can share one workspace (and with it one partial-sum region of the library); different
-    streams get different ones, which keeps the rule "one call at a time per workspace".  It grows when a wider
-    layer turns up (the old tensor's region is released first)."""
+def shared_workspace(device, elems=0):
+    """The zeroed int32 workspace that ``Layer.forward`` uses on `device` when the caller passes none: one per device,
+    made on first use (65536 elements, enough for 524288 output features; it grows, as a new tensor, only beyond that).
+    The library allows one call at a time per workspace, so this default suits models whose layers run one after
+    the other on one stream -- also under HIP-graph capture, which changes the current stream but not the device.
+    Callers that run layers concurrently on several streams pass ``forward`` a workspace of their own per stream."""
     device = torch.device(device)
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream)
+    key = device.index if device.index is not None else torch.cuda.current_device()
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < elems:
-        if ws is not None:
-            cabi.release_workspace(ws)
-        ws = torch.zeros(max(int(elems), 8192), dtype=torch.int32, device=device)
-        _workspaces[key] = ws
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("fp6_marlin: the default workspace of this device does not exist yet (or is too small "
+                               "for this layer) and cannot be made while a HIP graph is being captured; run the layer "
+                               "once before the capture, or pass forward() a workspace")
+        ws = torch.zeros(max(int(elems), 65536), dtype=torch.int32, device=device)
+        _workspaces[key] = ws                                      # (a smaller one stays alive with whoever captured it)
     return ws
 
 
@@ -134,8 +136,8 @@ class Layer(nn.Module):
       ``meta``       int32 [7]: format version, infeatures, outfeatures, quant_cols, groupsize, word order
                      (0 reference, 1 gfx950), quant_rows; a checkpoint whose ``meta`` differs is refused
     The GEMM's ``workspace`` (zeroed int32, outfeatures // 128 * 16 elements at least) is not a buffer of the layer:
-    ``forward`` takes ``shared_workspace``'s tensor of the current (device, stream), because the library keeps a
-    16 MiB partial-sum region per workspace address and calls that cannot overlap should share one.
+    ``forward`` takes the one passed to it or else ``shared_workspace``'s tensor of the device, because the library
+    keeps a partial-sum region per workspace address and calls that cannot overlap should share one.
 
     Which output features are kept in FP6: by default the *last* ``quant_cols`` ones (what the reference's
     harness does after moving its chosen columns to the tail, test.py:123-152).  With ``fp6_channels`` (indices
@@ -246,12 +248,17 @@ class Layer(nn.Module):
             w_ref = own
         return w_ref
 
-    def forward(self, x, residual=None):
-        """y = x @ W (+ bias) (+ residual, float16 of y's shape), as one GEMM call."""
+    def forward(self, x, residual=None, workspace=None):
+        """y = x @ W (+ bias) (+ residual, float16 of y's shape), as one GEMM call.  ``workspace``: a zeroed int32 CUDA
+        tensor of at least outfeatures // 128 * 16 elements that no overlapping call uses (default: the device's
+        ``shared_workspace``)."""
         x2 = x.reshape(-1, x.shape[-1]).to(torch.float16).contiguous()
         out = torch.empty((x2.shape[0], self.n), dtype=torch.float16, device=x2.device)
         res = None if residual is None else residual.reshape(-1, self.n).to(torch.float16).contiguous()
-        workspace = shared_workspace(x2.device, self.n // 128 * 16)
+        if workspace is None:
+            workspace = shared_workspace(x2.device, self.n // 128 * 16)
+        elif workspace.numel() < self.n // 128 * 16 or workspace.device != x2.device:
+            raise ValueError("workspace must be an int32 tensor of at least outfeatures // 128 * 16 elements on x's device")
         if self.quant_rows:
             cabi.mul_rows(x2, self.B, out, self.s, workspace, self.quant_rows, a_cols=self.a_cols, bias=self.bias,
                           residual=res, layout=self.layout)

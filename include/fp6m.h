@@ -36,7 +36,7 @@ extern "C" {
 #define FP6M_ERR_ARG         5 /* null pointer, unsupported group_size / quant_cols                  */
 #define FP6M_ERR_HIP         6 /* a HIP runtime call failed; fp6m_last_hip_error() has the code      */
 #define FP6M_ERR_NO_GPU_CODE 7 /* the library was built without its gfx950 kernels                   */
-#define FP6M_ERR_SCRATCH     8 /* partial sums do not fit the scratch of an entry point that cannot grow it */
+#define FP6M_ERR_SCRATCH     8 /* partial sums do not fit fp6m_mul_static's scratch, or no room for another workspace's region */
 
 /* Human-readable text for a return code (static storage). */
 const char* fp6m_strerror(int code);
@@ -85,9 +85,10 @@ int fp6m_mul(const void* A, const void* B, void* C, const void* s, int prob_m, i
  *     array's address out of the first call;
  *   - a launch of more than 16 rows whose k split needs more than the 12 MiB the array has for partial tiles returns
  *     FP6M_ERR_SCRATCH (fp6m_mul would shrink the split instead).  The need is (workgroups that share column tiles) x
- *     (32 or 64 rows) x 128 columns x 4 bytes; the splits the dispatcher picks on a 256-CU device stay below 10 MiB
- *     for every shape, so this only triggers for splits forced with fp6m_tuning_set or on larger devices.  Launches
- *     of up to 16 rows never fail this way: without room for their cells (n * m * 8 bytes > 8 MiB) no tile is shared;
+ *     (32, 64 or 128 rows) x 128 columns x 4 bytes; the dispatcher sizes its own splits to the 12 MiB (it keeps 64-row
+ *     tiles where a split of 128-row tiles would not fit), so this only triggers for splits forced with
+ *     fp6m_tuning_set or on devices with more compute units.  Launches of up to 4 rows never fail this way (without
+ *     room for their cells, n * m * 8 bytes > 8 MiB, no tile is shared); those of 5 to 16 rows only with a forced split;
  *   - every call on a GPU shares that GPU's array: calls that overlap on one GPU race, whatever their workspaces
  *     and streams.  `workspace` keeps its role (tile counters, zero on entry and on exit).
  */
@@ -161,6 +162,7 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * regions / the FP6 region only), "cap" (the waves it aims at), "wgs" (exactly that many waves, one-unit chunks drawn
  * from the counters), "gather" (its own activation gather on / off), "cells" (0: the m <= 16 kernel sums the shared
  * tiles of up to four rows through partial tiles, like those of more rows, instead of in the accumulate-and-count cells),
+ * "xcd" (the m <= 16 kernel's partial tiles of 5 to 16 rows exchanged inside one XCD: 1 wherever possible, 0 never),
  * "verbose" (print every launch's configuration to stderr); knob = NULL clears all overrides.  Unknown knob ->
  * FP6M_ERR_ARG.  Not synchronised with GEMM calls running on other threads.  The library reads no environment
  * variables on a call (FP6M_VERBOSE is looked up once at load time).
@@ -173,25 +175,42 @@ size_t fp6m_workspace_elems(int prob_n, int max_par);
 /*
  * Device memory the GEMM keeps besides its operands, and what may run concurrently.
  *
- * Column tiles whose k range is shared by several workgroups are summed through fp32 partial tiles in device memory
- * (the reference sums them through C in fp16 under the locks in `workspace`, fp6_marlin_cuda_kernel.cu:645-696).
- * That scratch belongs to the workspace: every workspace address the library has seen on a device owns a 24 MiB
- * region (plus 64 MiB for gathered activations once a call with a_cols has used it).  The concurrency rule is
- * therefore the reference's, one call at a time per workspace (fp6_marlin_cuda.cpp:62-63): calls with different
- * workspaces may overlap on different streams, also when replayed from HIP graphs; two overlapping calls must not
- * share a workspace.
- * A region is allocated (hipMalloc + hipMemset, both synchronous) by the first call with a workspace, or ahead of
- * time by fp6m_init_workspace -- do that before HIP-graph capture or any other section that must not allocate.
- * Share one workspace between calls that never overlap (all layers of a model on one stream).  The library holds at
- * most FP6M_MAX_WORKSPACES regions per device: when another is needed it waits for the device
- * (hipDeviceSynchronize) and frees them all, which fails inside a capture.  fp6m_release_workspace frees one region
- * (call it before the workspace is freed), or all of a device's with workspace = NULL; it waits for the device first.
- * No counterpart in the reference.
+ * Column tiles whose k range is shared by several workgroups are summed through fp32 partial tiles or 64-bit cells in
+ * device memory (the reference sums them through C in fp16 under the locks in `workspace`,
+ * fp6_marlin_cuda_kernel.cu:645-696).  That scratch belongs to the workspace: every workspace address the library has
+ * seen on a device owns a 24 MiB region (plus 64 MiB for gathered activations once a call with a_cols has used it).
+ * The concurrency rule is therefore the reference's, one call at a time per workspace (fp6_marlin_cuda.cpp:62-63):
+ * calls with different workspaces may overlap on different streams, also when replayed from HIP graphs; two
+ * overlapping calls must not share a workspace.
+ * A device has FP6M_MAX_WORKSPACES regions.  The first FP6M_BUILTIN_WORKSPACES are part of the library's device code
+ * (96 MiB per GPU, held until the process ends): a call whose workspace gets one of them allocates nothing, never
+ * waits for the device and can be captured into a HIP graph as it is, like the reference's
+ * (fp6_marlin_cuda_kernel.cu:864-880 allocates nothing).  The others get their memory from hipMalloc + hipMemset (both
+ * synchronous) when a fifth, sixth .. workspace turns up, and keep it for good.  A workspace the library has not seen
+ * takes a region nobody owns; when there is none, the region whose workspace has gone unused longest is handed over
+ * after a hipDeviceSynchronize -- so callers that make a new workspace for every call (the reference's test.py:168 and
+ * bench.py:44 do) never run out, at the price of that wait from the seventeenth workspace on.  Consequences: keep at
+ * most FP6M_MAX_WORKSPACES workspaces in concurrent use per device (overlapping calls on more would share scratch); a
+ * graph captured with a workspace whose region has since been handed over must not be replayed while calls with the
+ * new owner are running; and a call under capture whose workspace has no region yet is refused (FP6M_ERR_SCRATCH)
+ * unless a region is free -- fp6m_init_workspace beforehand makes sure.  The gathered-activation buffer of
+ * fp6m_mul_fused (64 MiB, once per region) is always allocated with hipMalloc.  Share one workspace between calls that
+ * never overlap (all layers of a model on one stream).  fp6m_release_workspace gives a workspace's region up (call it
+ * before the workspace is freed), or all of a device's with workspace = NULL; it waits for the device first, and
+ * graphs captured with that workspace must not be replayed afterwards.  No counterpart in the reference.
  */
-#define FP6M_MAX_WORKSPACES 128
-/* Looks up the device's compute-unit count; optional (the first GEMM call does it too).  Allocates nothing. */
+#define FP6M_MAX_WORKSPACES 16
+#define FP6M_BUILTIN_WORKSPACES 4
+/*
+ * Looks up the device's properties (compute units, addresses of the built-in scratch) and checks, with a few launches
+ * of a probe kernel, how the device deals a dispatch's workgroups to its XCDs (the m <= 16 kernel exchanges partial
+ * tiles inside one XCD's L2 only where that check has passed).  Waits for the device; allocates nothing.  Optional:
+ * the first GEMM call on a device does the same, unless its stream is being captured, in which case the check is left
+ * to a later call.
+ */
 int fp6m_init(int dev);
-/* Region of `workspace`; with_gather != 0 also allocates its gathered-activation buffer. */
+/* Region of `workspace` now rather than in its first call; with_gather != 0 also allocates its gathered-activation
+ * buffer (needed before capturing an fp6m_mul_fused call that passes a_cols with more than one row). */
 int fp6m_init_workspace(int dev, const void* workspace, int with_gather);
 int fp6m_release_workspace(int dev, const void* workspace);
 

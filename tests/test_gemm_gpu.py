@@ -366,6 +366,10 @@ def test_one_wave_decode_kernel(oracle):
         run(oracle, m, 640, 1024, qc=-1, gs=128, env=dict(e, FP6M_SHARE=1))       # all INT4, one unit per chunk
         run(oracle, m, 768, 192, 64, 256, qc=-1, env=dict(e, FP6M_SHARE=2))       # three units per tile, no group scales
         run(oracle, m, 256, 64, 64, 256, qc=-1, env=e)                            # a single unit
+        # k = 64 without group scales and fewer waves than tiles: an INT4 chunk of the single unit would be shorter than
+        # the fetch side's look-ahead, which drawn chunks cannot follow, so the workgroup kernel takes these
+        run(oracle, m, 1024, 64, 64, 256, qc=-1, env=dict(e, FP6M_WGS=3))
+        run(oracle, m, 1024, 64, 64, 256, qc=256, env=dict(e, FP6M_WGS=3))
     run(oracle, 1, 512, 2048, qc=256, gs=128, env={"FP6M_SK": 0})                 # one row on the workgroup kernel
     run(oracle, 1, 768, 1024, qc=128, env={"FP6M_SK": 0})
     for gs in (-1, 128):
@@ -542,6 +546,39 @@ def test_layer_forward(oracle):
     assert y.shape == (2, 5, 768)
     y_ref = (x.reshape(-1, 1024).float() @ w_ref.float()).reshape(2, 5, 768)
     assert oracle.rel_err(y.numpy(), y_ref.numpy()) <= TOL
+
+
+def test_layer_forward_captured_in_a_hip_graph(oracle):
+    """A Layer that has run once can be captured with torch.cuda.graph (whose capture stream is not the stream of the
+    warm-up) and replayed: the default workspace belongs to the device, not to the stream.  Every replay, with eager
+    forwards in between, gives the eager result bit for bit; a caller's own workspace works the same way."""
+    import fp6_marlin
+    k, n, m = 1024, 1536, 8
+    rng = np.random.default_rng(11)
+    lin = torch.nn.Linear(k, n, bias=False).half()
+    lin.weight.data = torch.from_numpy(rng.normal(0, 0.02, (n, k)).astype(np.float16))
+    layer = fp6_marlin.Layer(k, n, groupsize=128, quant_cols=256)
+    w_ref = layer.pack(lin)
+    layer = layer.to(dev())
+    x = torch.from_numpy(rng.normal(0, 1, (m, k)).astype(np.float16)).to(dev())
+    want = layer(x).clone()                                              # warm-up on the current stream
+    assert oracle.rel_err(want.cpu().numpy(), oracle.matmul_ref(x.cpu().numpy(), w_ref.numpy())) <= TOL
+    # (a workspace of the caller's own: given its region ahead of the capture, because by now the earlier tests'
+    # workspaces hold every region, and a capture cannot wait for the device to take one over)
+    own = fp6_marlin.init_workspace(torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev()))
+    for ws in (None, own):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = layer(x, workspace=ws)
+        for _ in range(3):
+            y.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, want)
+            assert torch.equal(layer(x, workspace=ws), want)             # eager work between the replays
+    with pytest.raises(ValueError):
+        layer(x, workspace=torch.zeros(8, dtype=torch.int32, device=dev()))
+    fp6_marlin.release_workspace(own)
 
 
 def test_layer_with_chosen_fp6_channels_bias_residual_and_checkpoint(oracle):
