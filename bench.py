@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]          one JSON line (the driver's contract)
     python bench.py --sweep sweep.json                           per-shape table for all benchmark configurations
     python bench.py --shape 128,8192,8192                        one shape (m,k,n[,quant_cols,group_size])
+    python bench.py --models                                     the reference's own benchmark (bench.py:57-119): five models' layers at batch 16
 
 Workload of the JSON line: decode (M=1) through Llama-2-7B layer shapes (K x N) 4096x12288, 4096x4096,
 4096x22016, 11008x4096; INT4 with group-128 scales plus 256 FP6 columns.  A *step* is one layer: those four
@@ -15,8 +16,8 @@ value        packed-weight GB/s over the timed steps: algorithmic weight bytes /
              weight bytes = K(N-qc)/2 + K*qc*3/4 + scale bytes.
 roofline     the GEMM kernel against the 8 TB/s HBM peak: algorithmic bytes per launch / mean time per
              launch, measured with HIP events on the launch stream over the same timed region.
-cpu_baseline the oracle's CPU path (quantise + prepack + dequantise-then-matmul) on one bounded sample
-             shape, single-threaded like the reference, on this box's host cores.
+cpu_baseline the oracle's CPU path (quantise + prepack + dequantise-then-matmul) on config 0 (16 x 4096 x 4096), stage
+             by stage, single-threaded like the reference (`value`) and on all cores, on this box's host cores.
 Also reported: a fp16 torch.matmul (hipBLASLt/rocBLAS) over the same shapes and rotation, and the speed-up.
 """
 import argparse
@@ -52,12 +53,15 @@ class Problem:
     benchmark's calls run back to back on one stream (the library keeps a partial-sum region per workspace)."""
     shared_ws = None
 
-    def __init__(self, torch, m, k, n, qc, gs, gen, fp16_ref=False):
+    def __init__(self, torch, m, k, n, qc, gs, gen, fp16_ref=False, on_device=False):
         dev = torch.device("cuda:0")
         n4 = n - qc
         words = k * n4 // 8 + k * qc * 3 // 16
         self.m, self.k, self.n, self.qc, self.gs = m, k, n, qc, gs
-        self.B = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
+        if on_device:                                                    # (layers of hundreds of MB: the host generator takes seconds)
+            self.B = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), dtype=torch.int32, device=dev)
+        else:
+            self.B = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
         ns = (n4 if gs == -1 else (k // gs) * n4) + qc
         self.s = (torch.rand(ns, generator=gen) * 0.01 + 0.001).half().to(dev)
         self.A = torch.randn((m, k), generator=gen).half().to(dev)
@@ -116,17 +120,89 @@ def time_region(torch, fn, iters):
     return t1 - t0, start.elapsed_time(stop) * 1e-3
 
 
-def cpu_baseline(torch):
-    """The reference's CPU path restated (oracle/) on one layer of the headline workload (decode M=1, the four
-    Llama-2-7B shapes): quantise + prepack, then dequantise-then-matmul, one thread, as the reference's own CPU
-    routines and harness run it.  The shipped threaded host packers are timed beside it for the note only."""
+def _median(fn, reps):
+    ts = []
+    out = None
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        out = fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2], out
+
+
+def cpu_config0(torch, threaded):
+    """The reference's CPU path on config 0 (M=16, K=4096, N=4096, 256 FP6 columns, INT4 g128), its five stages
+    timed separately (median of five): (1) FP6 scale + clamp + cast (test.py:19-32, weight_quant.cpp:27-124),
+    (2) FP6 2+4 prepack (weight_prepacking.cpp:123-177), (3) INT4 quantise + Marlin pack (test.py:85-121),
+    (4) dequantise to the fp16 check weight (weight_prepacking.cpp:180-217, test.py:98), (5) the matmul on the CPU
+    (fp32, the fp16 inputs are exact in it).  threaded=False: the oracle's restatement on one thread, as the reference
+    runs (weight_quant.cpp:114 has its OpenMP pragma commented out); threaded=True: this package's own host
+    routines and torch on all cores."""
     import numpy as np
-    import fp6_marlin
+    m, k, n, qc, gs = 16, 4096, 4096, 256, 128
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn((m, k), generator=g).half()
+    w = (torch.randn((k, n), generator=g) * 0.02).half()
+    w4, w6 = w[:, : n - qc].contiguous(), w[:, n - qc:].contiguous()
+    if threaded:
+        from fp6_marlin import cabi as api
+        asnp = lambda t: t                                               # (the package's routines take tensors)
+    else:
+        from oracle import fp6m_oracle as api
+        asnp = lambda t: t.numpy()
+
+    def fp6_cast():
+        s = torch.max(torch.abs(w6), 0, keepdim=True)[0]
+        s *= 1.0 / 28.0
+        s = s.reshape(-1)
+        x = w6 / s
+        x = torch.where(torch.abs(x) < 0.0625, torch.zeros_like(x), x)
+        x = torch.clamp(x, -28.0, 28.0)
+        return api.fp6_quantize(asnp(x)), s
+
+    t1, (q6, s6) = _median(fp6_cast, 5)
+    t2, _ = _median(lambda: api.fp6_prepack(q6), 5)
+
+    def int4():
+        codes, s, ref = api.int4_quantize(asnp(w4), gs)
+        return api.int4_pack(codes), codes, s
+
+    t3, (_, codes, s4) = _median(int4, 5)
+
+    def dequant():
+        r6 = api.fp6_dequant(q6, asnp(s6))
+        r6 = torch.as_tensor(r6).t()
+        c = torch.as_tensor(codes).float() - 8.0
+        r4 = (c.reshape(k // gs, gs, n - qc) * torch.as_tensor(s4).float().reshape(k // gs, 1, n - qc)).reshape(k, n - qc).half()
+        return torch.cat([r4, r6], dim=1).contiguous()
+
+    t4, w_ref = _median(dequant, 5)
+    t5, _ = _median(lambda: torch.matmul(a.float(), w_ref.float()), 5)
+    total = t1 + t2 + t3 + t4 + t5
+    nbytes = weight_bytes(k, n, qc, gs)
+    return {"seconds": round(total, 4), "GBs": round(nbytes / total / 1e9, 4),
+            "stages_s": {"fp6_scale_clamp_cast": round(t1, 4), "fp6_prepack": round(t2, 4), "int4_quantise_pack": round(t3, 4),
+                         "dequantise": round(t4, 4), "matmul_fp32": round(t5, 5)},
+            "torch_threads": torch.get_num_threads()}
+
+
+def cpu_baseline(torch):
+    """The reference's CPU path restated (oracle/), timed on this box's host cores: config 0 stage by stage, on one
+    thread (`value`; the reference is single-threaded) and on all cores (this package's threaded host routines),
+    and one layer of the headline workload (decode M=1, the four Llama-2-7B shapes) on one thread."""
+    import numpy as np
     from oracle import fp6m_oracle as oracle
-    m, qc, gs = 1, 256, 128
     threads = torch.get_num_threads()
     torch.set_num_threads(1)
-    t_prep = t_mm = t_ship = 0.0
+    try:
+        one = cpu_config0(torch, threaded=False)
+    finally:
+        torch.set_num_threads(threads)
+    many = cpu_config0(torch, threaded=True)
+    m, qc, gs = 1, 256, 128
+    torch.set_num_threads(1)
+    t_prep = t_mm = 0.0
     nbytes = 0
     try:
         rng = np.random.default_rng(0)
@@ -142,18 +218,51 @@ def cpu_baseline(torch):
             t_mm += t2 - t1
             nbytes += weight_bytes(k, n, qc, gs)
             del c, b, s, w_ref
-            torch.set_num_threads(threads)
-            t3 = time.perf_counter()
-            fp6_marlin.pack_mixed_weight(torch.from_numpy(w), qc, gs)
-            t_ship += time.perf_counter() - t3
-            torch.set_num_threads(1)
     finally:
         torch.set_num_threads(threads)
-    return {"value": nbytes / (t_prep + t_mm) / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"one layer of the headline workload (M=1, the four Llama-2-7B shapes, INT4 g128 + 256 FP6 cols, "
-                      f"{nbytes} packed weight bytes), one thread: quantise+prepack+dequantise {t_prep:.2f} s, "
-                      f"fp32 dequantised matmul {t_mm:.3f} s ({nbytes / t_mm / 1e9:.2f} GB/s for the matmul alone); "
-                      f"the shipped host packers take {t_ship:.2f} s on {os.cpu_count()} logical cores"}
+    return {"value": one["GBs"], "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "config 0 (M=16, K=4096, N=4096, 256 FP6 columns, INT4 g128; 8,897,024 packed weight bytes): quantise + "
+                      "prepack + dequantise + fp32 matmul, medians of five per stage, the oracle's restatement on one thread",
+            "one_thread": one, "all_cores": dict(many, cores=os.cpu_count(), kind="this package's threaded host routines + torch"),
+            "os_cpu_count": os.cpu_count(), "torch_num_threads": threads,
+            "headline_layer_one_thread": {
+                "GBs": round(nbytes / (t_prep + t_mm) / 1e9, 4), "weight_bytes": nbytes,
+                "quantise_prepack_dequantise_s": round(t_prep, 2), "matmul_fp32_s": round(t_mm, 3),
+                "sample": "one layer of the headline workload (M=1, the four Llama-2-7B shapes, INT4 g128 + 256 FP6 columns)"}}
+
+
+# Layer sets of the reference's own benchmark (bench.py:57-85: k x n per layer) and what its chart shows for them at
+# batch 16 on an RTX 4090D (assets/models.png, read off the bars: all INT4 / INT4 + 256 FP6 columns).
+REFERENCE_MODELS = {
+    "Llama7B": [(4096, 3 * 4096), (4096, 4096), (4096, 2 * 10752), (10752, 4096)],
+    "Llama13B": [(5120, 3 * 5120), (5120, 5120), (5120, 2 * 13568), (13568, 5120)],
+    "Llama33B": [(6656, 3 * 6656), (6656, 6656), (6656, 2 * 17664), (17664, 6656)],
+    "Llama65B": [(8192, 3 * 8192), (8192, 8192), (8192, 2 * 21760), (21760, 8192)],
+    "Falcon180B": [(14848, 14848 * 5 + 1024), (14848 * 5, 14848)],
+}
+REFERENCE_CHART_4090D = {"Llama7B": (3.89, 3.73), "Llama13B": (4.10, 4.01), "Llama33B": (3.80, 3.77),
+                         "Llama65B": (3.84, 3.78), "Falcon180B": (3.88, 3.84)}
+
+
+def reference_models(torch, fp6_marlin, gen, calls_target=40):
+    """The reference's published measurement (bench.py:57-85, 100-119): batch 16, per-channel scales, quant_cols -1 and
+    256, over each model's layers; speed-up = total fp16 time / total time of the quantised GEMMs (its time-weighted
+    mean of the per-layer speed-ups).  Timing protocol as everywhere here (HIP graphs over > 640 MB of rotated
+    weights), not the reference's 100 calls on one weight."""
+    rows = []
+    for model, layers in REFERENCE_MODELS.items():
+        for j, qc in enumerate((0, 256)):
+            per = [measure_shape(torch, fp6_marlin, gen, model, 16, k, n, qc, -1, calls_target=calls_target, on_device=True)
+                   for k, n in layers]
+            t, t16 = sum(r["us"] for r in per), sum(r["fp16_us"] for r in per)
+            nbytes = sum(weight_bytes(k, n, qc, -1) for k, n in layers)
+            rows.append({"tag": f"reference bench {model} M=16 quant_cols={qc if qc else -1} group_size=-1", "m": 16,
+                         "layers": [f"{k}x{n}" for k, n in layers], "us": round(t, 2), "fp16_us": round(t16, 2),
+                         "speedup_vs_fp16": round(t16 / t, 2), "weight_GBs": round(nbytes / t / 1e3, 1),
+                         "hbm_frac": round(nbytes / t / 1e3 / HBM_PEAK_GBS, 4),
+                         "layer_us": [r["us"] for r in per], "layer_fp16_us": [r["fp16_us"] for r in per],
+                         "reference_chart_speedup_rtx4090d": REFERENCE_CHART_4090D[model][j]})
+    return rows
 
 
 def graphed(torch, step, layers, steps):
@@ -245,9 +354,11 @@ def headline(args):
     # the batch sweep on 8192 x 8192, each next to the fp16 GEMM of the same shape
     if not args.headline_only:
         regimes = [(f"70B M={mm}", mm, k, n) for mm in (1, 16) for (k, n) in LLAMA70B]
+        regimes += [("7B M=16", 16, k, n) for (k, n) in LLAMA7B]
         regimes += [(f"batch sweep M={mm}", mm, 8192, 8192) for mm in (2, 4, 8, 32, 64, 128, 256, 512, 1024)]
         out["other_regimes"] = [measure_shape(torch, fp6_marlin, gen, tag, mm, k, n, qc, gs, calls_target=60)
                                 for tag, mm, k, n in regimes]
+        out["other_regimes"] += reference_models(torch, fp6_marlin, gen)
     print(json.dumps(out), flush=True)
 
 
@@ -271,14 +382,17 @@ def traffic_probe():
           [p.bytes for p in probs[0]], flush=True)
 
 
-def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100, layout="reference"):
+def measure_shape(torch, fp6_marlin, gen, tag, m, k, n, qc, gs, calls_target=100, layout="reference", on_device=False):
     """One (m, k, n) GEMM against fp16 torch.matmul (hipBLASLt), both replayed from HIP graphs that walk
     over > 512 MB of distinct weights."""
     nbytes = weight_bytes(k, n, qc, gs)
     copies = max(2, min(24, int(640e6 // nbytes) + 1))
-    probs = [Problem(torch, m, k, n, qc, gs, gen) for _ in range(copies)]
-    w16 = [(torch.randn((k, n), generator=gen) * 0.02).half().cuda()
-           for _ in range(max(2, min(copies, int(640e6 // (2 * k * n)) + 1)))]
+    probs = [Problem(torch, m, k, n, qc, gs, gen, on_device=on_device) for _ in range(copies)]
+    n16 = max(2, min(copies, int(640e6 // (2 * k * n)) + 1))
+    if on_device:
+        w16 = [(torch.randn((k, n), device="cuda") * 0.02).half() for _ in range(n16)]
+    else:
+        w16 = [(torch.randn((k, n), generator=gen) * 0.02).half().cuda() for _ in range(n16)]
 
     def f(i):
         if layout == "gfx950":
@@ -500,6 +614,8 @@ def main():
     ap.add_argument("--fused", type=str, default=None, help="m,k,n[,quant_cols,group_size]: time mul_fused against mul + torch kernels")
     ap.add_argument("--rows", type=str, default=None, help="m,k,n[,quant_rows]: time the row-mixed GEMM against two mul calls and an addition")
     ap.add_argument("--pack", type=str, default=None, help="k,n[,quant_cols,group_size]: time the on-GPU weight packer")
+    ap.add_argument("--models", action="store_true", help="the reference's own benchmark: its five models' layers at batch 16, "
+                                                          "quant_cols -1 and 256, per-channel scales, time-weighted speed-up over fp16")
     ap.add_argument("--headline-only", action="store_true", help="skip the other regimes' rows of the JSON line")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -510,6 +626,12 @@ def main():
                  "run with --gpus 1")
     if args.traffic_probe:
         traffic_probe()
+    elif args.models:
+        import torch
+        import fp6_marlin
+        fp6_marlin.init(0)
+        for row in reference_models(torch, fp6_marlin, torch.Generator().manual_seed(0)):
+            print(json.dumps(row), flush=True)
     elif args.sweep:
         sweep(args)
     elif args.shape:

@@ -68,7 +68,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -109,6 +109,7 @@ struct DeviceState {
     int xcd_placement = -1;            // 1: workgroup b of a grid runs on XCD b % 8 (verified by verify_placement), 0: not so, -1: not looked at yet
     float* static_scratch = nullptr;   // device address of this GPU's copy of g_static_scratch
     unsigned char* slot_scratch = nullptr;   // ... and of g_slot_scratch
+    unsigned char* pool = nullptr;           // kStaticSlots regions from one hipMalloc (see workspace_region)
     unsigned long long tick = 0;
     void* pack_temp = nullptr;      // kPackTempBytes for the on-GPU packer's flag and column maxima
     Region regions[kMaxRegions];
@@ -251,33 +252,50 @@ int workspace_region(int dev, const void* workspace, bool want_region, bool want
     out->static_scratch = d->static_scratch;
     out->xcd_placement = d->xcd_placement;
     if (!want_region) return FP6M_OK;
-    for (int i = 0; i < kStaticSlots; i++)
-        if (!d->regions[i].partials) d->regions[i].partials = reinterpret_cast<float*>(d->slot_scratch + (size_t)i * kRegionBytes);
     Region* r = nullptr;
     for (Region& c : d->regions)
         if (c.workspace == workspace) r = &c;
     if (!r) {
-        Region *idle = nullptr, *bare = nullptr, *oldest = nullptr;
-        for (Region& c : d->regions) {
-            if (!c.workspace && c.partials && !idle) idle = &c;
-            if (!c.workspace && !c.partials && !bare) bare = &c;
+        const bool may_wait = !capturing(stream);
+        Region *builtin = nullptr, *idle = nullptr, *bare = nullptr, *oldest = nullptr;
+        for (int i = 0; i < kMaxRegions; i++) {
+            Region& c = d->regions[i];
+            if (!c.workspace && i < kStaticSlots && !builtin) builtin = &c;
+            if (!c.workspace && i >= kStaticSlots && c.partials && !idle) idle = &c;
+            if (!c.workspace && i >= kStaticSlots && !c.partials && !bare) bare = &c;
             if (c.workspace && !c.pins && (!oldest || c.last_use < oldest->last_use)) oldest = &c;
         }
-        if (idle) {
+        auto allocate = [&](size_t bytes, void** mem) {
+            const hipError_t e = on_device(dev, [&] {
+                hipError_t e2 = hipMalloc(mem, bytes);
+                if (e2 == hipSuccess) e2 = hipMemset(*mem, 0, bytes);
+                return e2;
+            });
+            if (e != hipSuccess && *mem) (void)hipFree(*mem);
+            return e;
+        };
+        if (builtin) {
+            // The first kStaticSlots regions: their memory is the device's pool, one hipMalloc made the first time a
+            // call may wait for it (so not by a call that is being captured), and until then the slots of the code
+            // object's own array.  Atomics on the latter are slower (the cells of a 4096 x 4096 decode GEMM: 5.7 -> 6.6 us
+            // per launch), so the pool is preferred as soon as it exists.
+            const int i = (int)(builtin - d->regions);
+            if (!d->pool && may_wait) {
+                void* mem = nullptr;
+                const hipError_t e = allocate(kStaticSlots * kRegionBytes, &mem);
+                if (e != hipSuccess) return hip_fail(e);
+                d->pool = static_cast<unsigned char*>(mem);
+            }
+            builtin->partials = reinterpret_cast<float*>((d->pool ? d->pool : d->slot_scratch) + (size_t)i * kRegionBytes);
+            r = builtin;
+        } else if (idle) {
             r = idle;
-        } else if (capturing(stream)) {
+        } else if (!may_wait) {
             return FP6M_ERR_SCRATCH;
         } else if (bare) {
             void* mem = nullptr;
-            const hipError_t e = on_device(dev, [&] {
-                hipError_t e2 = hipMalloc(&mem, kRegionBytes);
-                if (e2 == hipSuccess) e2 = hipMemset(mem, 0, kRegionBytes);
-                return e2;
-            });
-            if (e != hipSuccess) {
-                if (mem) (void)hipFree(mem);
-                return hip_fail(e);
-            }
+            const hipError_t e = allocate(kRegionBytes, &mem);
+            if (e != hipSuccess) return hip_fail(e);
             bare->partials = static_cast<float*>(mem);
             r = bare;
         } else if (oldest) {
@@ -459,7 +477,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -821,6 +839,60 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if (w4 > chunks4) w4 = chunks4;
                 if (w6 > chunks6) w6 = chunks6;
             }
+            // Chunk lengths by generation.  The first 4 x CUs waves of a launch get a SIMD each, the next 4 x CUs share one
+            // with an older wave, which the SIMD serves first: with equal chunks the generations finish one after the
+            // other (per-wave timelines, loop ends in us: 8192 x 57344 27.7 / 37.0, 8192 x 8192 5.5 / 7.1,
+            // 4096 x 22016 6.4 / 8.0 / 10.0) and the launch ends on a thinning tail.  So when the plan above needs more
+            // than one generation, the INT4 tiles are dealt to the generations in order, each with its own chunk length:
+            // a later generation's chunks shorter by about its waves' share of the SIMD (e), so that all end together.
+            // Of the first generation's chunk counts per tile, the one with the smallest (chunk length / e) over the
+            // generations that the tiles then reach is taken (kernel: sk_generation_order and the sub-lists of SkArgs).
+            long long gen_cpt[3] = {cpt4, cpt4, cpt4}, gen_q[3] = {q4, q4, q4}, gen_tiles[3] = {tiles4, 0, 0};
+            const long long gen_size = 4LL * cus;
+            sk.gen_waves = 0;
+            const bool plain_plan = tune.wgs == kUnset && tune.share == kUnset && tune.share6 == kUnset && env_ks < 1 && sms <= 0 &&
+                                    cells_fit && w4 == chunks4 && w6 == chunks6;
+            if (plain_plan && tiles4 > 0 && chunks4 + chunks6 > gen_size && chunks6 < gen_size && waves_wanted >= 2 * gen_size &&
+                !(tune.gen != kUnset && tune.gen == 0)) {
+                const double e[3] = {1.0, (tune.gen2 != kUnset ? tune.gen2 : 66) / 100.0, (tune.gen3 != kUnset ? tune.gen3 : 30) / 100.0};
+                const long long cap[3] = {gen_size - chunks6, gen_size,
+                                          waves_wanted - 2 * gen_size < gen_size ? waves_wanted - 2 * gen_size : gen_size};
+                const long long min_units = g128 ? 1 : 2;
+                auto fit = [&](long long len) {                        // a length whose last chunk of a tile is not too short
+                    if (len < min_units) len = min_units;
+                    if (len * 32 < u4) len = (u4 + 31) / 32;
+                    while (len < u4 && u4 % len != 0 && u4 % len < min_units) len++;
+                    return len > u4 ? u4 : len;
+                };
+                const long long last_gen = (chunks4 + chunks6 - 1) / gen_size;
+                double best = (double)q4 / e[last_gen < 2 ? last_gen : 2];          // the plan above, under the same model
+                for (long long cpt_a = 1; cpt_a <= 32 && cpt_a <= u4 / min_units; cpt_a++) {
+                    long long len[3], cpt[3], t[3], left = tiles4;
+                    double cost = 0;
+                    for (int g = 0; g < 3; g++) {
+                        len[g] = fit(g == 0 ? (u4 + cpt_a - 1) / cpt_a : (long long)((double)len[0] * e[g] + 0.5));
+                        if (g > 0 && len[g] > len[g - 1]) len[g] = len[g - 1];
+                        cpt[g] = (u4 + len[g] - 1) / len[g];
+                        t[g] = cap[g] / cpt[g] < left ? cap[g] / cpt[g] : left;
+                        left -= t[g];
+                        if (t[g] > 0 && (double)len[g] / e[g] > cost) cost = (double)len[g] / e[g];
+                    }
+                    if (left > 0 || cost >= best) continue;
+                    best = cost;
+                    for (int g = 0; g < 3; g++) {
+                        gen_cpt[g] = cpt[g];
+                        gen_q[g] = len[g];
+                        gen_tiles[g] = t[g];
+                    }
+                    sk.gen_waves = (int)gen_size;
+                }
+                if (sk.gen_waves) {
+                    q4 = gen_q[0];
+                    cpt4 = gen_cpt[0];
+                    chunks4 = gen_tiles[0] * gen_cpt[0] + gen_tiles[1] * gen_cpt[1] + gen_tiles[2] * gen_cpt[2];
+                    w4 = chunks4;
+                }
+            }
             sk.waves = (int)(w4 + w6);
             sk.waves6 = (int)w6;
             sk.units4 = (int)u4;
@@ -831,6 +903,16 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             sk.cpt6 = (int)cpt6;
             sk.magic_cpt4 = magic40(cpt4);
             sk.magic_cpt6 = magic40(cpt6);
+            sk.tiles4a = (int)gen_tiles[0];
+            sk.tiles4b = (int)gen_tiles[1];
+            sk.q4b = (int)gen_q[1];
+            sk.cpt4b = (int)gen_cpt[1];
+            sk.q4c = (int)gen_q[2];
+            sk.cpt4c = (int)gen_cpt[2];
+            auto magic32 = [](long long d) { return d >= 2 ? (uint32_t)((0x100000000ULL + (unsigned long long)d - 1) / (unsigned long long)d) : 0u; };
+            sk.magic32_cpt4b = magic32(gen_cpt[1]);
+            sk.magic32_cpt4c = magic32(gen_cpt[2]);
+            sk.pad[0] = sk.pad[1] = sk.pad[2] = sk.pad[3] = 0;
             sk.total4 = chunks4 > w4 ? (int)chunks4 : 0;               // 0: one chunk per wave, no counter traffic
             sk.total6 = chunks6 > w6 ? (int)chunks6 : 0;
             // The activation gather: by the kernel itself for one row and one chunk per wave (two dependent loads per
@@ -841,7 +923,6 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             sk.A = a.A;
             sk.a_cols = gather_inside ? fu.a_cols : nullptr;
             sk.lda = gather_inside ? fu.lda : 0;
-            sk.pad = 0;
             sk.counters = a.counters;
             // Counters: atomics on one address complete one after the other, about 0.3 us apart, and a wave's loads
             // queue behind its own draw, so no more than four waves share a counter (with 64 counters for 2560 waves
@@ -856,7 +937,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             sk.groups = (int)(groups4 | (groups6 << 16));
             if (tune.verbose)
                 fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: one-wave workgroups %lld (FP6) + %lld (INT4), chunks %lld of %lld units + "
-                        "%lld of %lld units\n", a.m, prob_n, prob_k, w6, w4, chunks6, q6, chunks4, q4);
+                        "%lld of %lld units%s", a.m, prob_n, prob_k, w6, w4, chunks6, q6, chunks4, q4, sk.gen_waves ? "" : "\n");
+            if (tune.verbose && sk.gen_waves)
+                fprintf(stderr, " (by generation: %lld tiles x %lld chunks of %lld, %lld x %lld of %lld, %lld x %lld of %lld)\n",
+                        gen_tiles[0], gen_cpt[0], gen_q[0], gen_tiles[1], gen_cpt[1], gen_q[1], gen_tiles[2], gen_cpt[2], gen_q[2]);
             dim3 grid((unsigned)sk.waves, 1);
             // variants: group scales or not; one chunk per wave with or without the gather, or chunks drawn from counters
             void (*kernel)(const SkArgs) = nullptr;

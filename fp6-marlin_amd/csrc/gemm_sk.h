@@ -36,7 +36,7 @@ namespace fp6m {
 // fp16's; a part that is not finite or is out of range saturates, which makes the element infinite.  The cells
 // live in the scratch region that belongs to the call's workspace, are zero when no call is in flight, and are left
 // zero.
-// Kernel arguments, laid out as three 64-byte blocks and a 16-byte one that the kernel fetches itself with four
+// Kernel arguments, laid out as four 64-byte blocks that the kernel fetches itself with four
 // scalar loads behind one wait (left to the compiler, the loads of the fields come in several dependent batches, each a
 // round trip to a cold line before the wave's first weight load).
 struct SkArgs {
@@ -66,10 +66,16 @@ struct SkArgs {
     const uint16_t* bias;
     const uint16_t* residual;
     unsigned long long* timeline;   // performance debugging builds only
-    // block 3 (16 bytes): the activation gather of fp6m_mul_fused, done by the kernel itself (GR > 0)
+    // block 3: the activation gather of fp6m_mul_fused, done by the kernel itself (GR > 0)
     const int32_t* a_cols;    // column kk of the GEMM's A is column a_cols[kk] (clamped) of the caller's matrix
     int lda;                  // the caller's row length
-    int pad;
+    // ... and the INT4 region's tiles in up to three sub-lists with a chunk length each (see sk_generation_order):
+    // tiles [0, tiles4a) in chunks of q4 units, [tiles4a, tiles4a + tiles4b) of q4b, the rest of q4c.
+    int gen_waves;            // waves of the whole chip that find a SIMD of their own (4 x CUs); 0: the plain order
+    int q4b, cpt4b, q4c, cpt4c;
+    int tiles4a, tiles4b;     // (all tiles in the first sub-list: tiles4a = the region's tiles)
+    uint32_t magic32_cpt4b, magic32_cpt4c;   // n / cpt as the high half of n * magic (exact for n, cpt < 2^16: a wave per chunk)
+    int pad[4];
     static constexpr int k4 = 0;    // (the row mix does not come here)
 };
 // What the fused-epilogue helpers of gemm_common.h read.
@@ -80,31 +86,29 @@ struct SkEpilogue {
     const uint16_t* residual;
     uint16_t* C;
 };
-static_assert(sizeof(SkArgs) == 208 && offsetof(SkArgs, m) == 64 && offsetof(SkArgs, magic_cpt4) == 128 &&
+static_assert(sizeof(SkArgs) == 256 && offsetof(SkArgs, m) == 64 && offsetof(SkArgs, magic_cpt4) == 128 &&
                   offsetof(SkArgs, a_cols) == 192,
-              "three 64-byte blocks and one of 16 bytes");
+              "four 64-byte blocks");
 
 __device__ __forceinline__ SkArgs load_sk_args()
 {
     typedef uint32_t u16v __attribute__((ext_vector_type(16)));
-    u16v b0, b1, b2;
-    u4 b3;
+    u16v b0, b1, b2, b3;
     const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile(
         "s_load_dwordx16 %0, %4, 0x0\n\ts_load_dwordx16 %1, %4, 0x40\n\ts_load_dwordx16 %2, %4, 0x80\n\t"
-        "s_load_dwordx4 %3, %4, 0xc0\n\ts_waitcnt lgkmcnt(0)"
+        "s_load_dwordx16 %3, %4, 0xc0\n\ts_waitcnt lgkmcnt(0)"
         : "=&s"(b0), "=&s"(b1), "=&s"(b2), "=&s"(b3) : "s"(ka));
     struct Words {
-        uint32_t w[52];
+        uint32_t w[64];
     } raw;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         raw.w[i] = b0[i];
         raw.w[16 + i] = b1[i];
         raw.w[32 + i] = b2[i];
+        raw.w[48 + i] = b3[i];
     }
-#pragma unroll
-    for (int i = 0; i < 4; i++) raw.w[48 + i] = b3[i];
     return __builtin_bit_cast(SkArgs, raw);
 }
 
@@ -171,16 +175,37 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     kc.top2 = vgpr_const(0xc0c0c0c0u);
     kc.exp_man = vgpr_const(0x9f009f00u);
 
-    // ---- chunks
-    const int q = FP6 ? p.q6 : p.q4, cpt = FP6 ? p.cpt6 : p.cpt4;
+    // ---- chunks.  INT4 region without drawn chunks: the sub-list that chunk j lies in sets the chunk length (a wave has
+    // one chunk, so one sub-list); `tile0` = tiles of the sub-lists before it, `j` becomes the index inside it.
+    // (The later sub-lists' tile is found with a 32-bit multiply-high: selecting among three 64-bit constants made the
+    // compiler keep them in an array in scratch memory, which cost every launch a microsecond.)
+    int q = FP6 ? p.q6 : p.q4, cpt = FP6 ? p.cpt6 : p.cpt4, tile0 = 0;
     const int units = FP6 ? p.units6 : p.units4;
     const unsigned long long magic_cpt = FP6 ? p.magic_cpt6 : p.magic_cpt4;
+    int first_tile = -1;                                   // tile, inside its sub-list, of the wave's own chunk
+    if constexpr (!FP6 && !DRAW) {
+        const int chunks_a = p.tiles4a * p.cpt4, chunks_b = p.tiles4b * p.cpt4b;
+        if (j >= chunks_a + chunks_b) {                    // (uniform)
+            j -= chunks_a + chunks_b;
+            tile0 = p.tiles4a + p.tiles4b;
+            q = p.q4c;
+            cpt = p.cpt4c;
+            first_tile = cpt <= 1 ? j : (int)__umulhi((uint32_t)j, p.magic32_cpt4c);
+        } else if (j >= chunks_a) {
+            j -= chunks_a;
+            tile0 = p.tiles4a;
+            q = p.q4b;
+            cpt = p.cpt4b;
+            first_tile = cpt <= 1 ? j : (int)__umulhi((uint32_t)j, p.magic32_cpt4b);
+        }
+    }
+    if (first_tile < 0) first_tile = (int)mul_shift40(magic_cpt, (uint32_t)j);
     static_assert(GR == 0 || !DRAW, "the gather follows one chunk");
     const int total = !DRAW ? 0 : (FP6 ? p.total6 : p.total4);    // 0: one chunk per wave, nothing to draw
     const int region_waves = FP6 ? p.waves6 : p.waves - p.waves6;
     const int region_n = FP6 ? p.qc : p.n4;
     // chunk id -> tile of the region, first unit, units
-    auto chunk_tile = [&](int ch) { return (int)mul_shift40(magic_cpt, (uint32_t)ch); };
+    auto chunk_tile = [&](int ch) { return DRAW ? (int)mul_shift40(magic_cpt, (uint32_t)ch) : first_tile; };   // (no draw: ch == j)
     auto chunk_len = [&](int kb) { return units - kb < q ? units - kb : q; };
     // A single counter would see every wave's first draw at the same moment (thousands of atomics on one address:
     // tens of microseconds).  The list is therefore dealt into `groups` sub-lists (chunk c belongs to sub-list
@@ -218,6 +243,7 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
     int i_tcol = chunk_tile(j);
     int i_step = (j - i_tcol * cpt) * q * unit_steps;
     int i_left = chunk_len((j - i_tcol * cpt) * q) * unit_steps;
+    i_tcol += tile0;
     const uint32_t step4 = 2 * (uint32_t)row4, step2 = 2 * (uint32_t)row2;
     uint32_t off4 = (uint32_t)i_tcol * (uint32_t)tile_stride4 + (uint32_t)i_step * step4;
     uint32_t off2 = (uint32_t)i_tcol * (uint32_t)tile_stride2 + (uint32_t)i_step * step2;
@@ -252,7 +278,7 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
             const int next = group + groups * drawn_index;
             if (drawn_index < group_total) {
                 f_chunk = next;
-                i_tcol = chunk_tile(next);
+                i_tcol = chunk_tile(next);                // (drawn chunks: one sub-list, tile0 = 0)
                 const int kb = (next - i_tcol * cpt) * q;
                 i_step = kb * unit_steps;
                 i_left = chunk_len(kb) * unit_steps;
@@ -461,9 +487,10 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
 
     int c_chunk = j;                                      // the chunk the multiply side is on
     while (true) {                                                       // (uniform) one chunk per trip
-        const int tcol = chunk_tile(c_chunk);
+        int tcol = chunk_tile(c_chunk);
         const int kb = (c_chunk - tcol * cpt) * q;
         const int len = chunk_len(kb);
+        tcol += tile0;
         const int tile = FP6 ? tcol : p.tiles6 + tcol;
         const int col0 = (FP6 ? p.n4 : 0) + tcol * kTileN;
         h2 sv = {(_Float16)1.0f, (_Float16)1.0f};
@@ -609,6 +636,24 @@ __device__ __forceinline__ void sk_wave(const SkArgs& p, int j, FP6M_AS3 unsigne
 
 constexpr int kSkWaveLds = wave_lds_bytes(4, 3, 4) + 4 * kRedStride * 4;   // ring, then the four-row slab
 
+// Position of workgroup (= wave) b in the chunk list.  The chip gives the first gen_waves waves of a launch a SIMD each
+// (workgroup b is the (b / 8)-th on its XCD, and an XCD's first gen_waves / 8 land on different SIMDs); the next
+// gen_waves share a SIMD with one of those, and so on.  A SIMD serves its older wave first: with equal chunks the
+// second generation finishes a third later than the first and the third later still, and the launch ends on a thinning
+// tail (8192 x 57344 at one row: loops end at 27.7 us in the first generation, at 37 us in the second).  The host
+// therefore gives later generations shorter chunks, and this order puts them where they belong: generation-major, and
+// inside a generation every XCD a contiguous range, as xcd_contiguous_id does for the whole list (gen_waves = 0).
+__device__ __forceinline__ int sk_generation_order(int b, int total, int gen_waves)
+{
+    if (gen_waves == 0 || total <= gen_waves) return xcd_contiguous_id(b, total);
+    const int per = gen_waves >> 3;                        // waves of one generation on one XCD
+    const int x = b & 7, i = b >> 3;
+    const int g = (i >= per) + (i >= 2 * per) + (i >= 3 * per);   // (the host plans at most four generations)
+    const int rest = total - g * gen_waves;                // waves of this and later generations
+    if (rest >= gen_waves) return g * gen_waves + x * per + (i - g * per);
+    return g * gen_waves + xcd_contiguous_id(((i - g * per) << 3) | x, rest);   // the last, partly filled generation
+}
+
 // second launch-bound argument = waves per SIMD the register budget must allow (HIP semantics)
 // EXTRAS = false: the build for one row, without a fused epilogue, on reference-order words (the arguments that select
 // anything else are overwritten with constants: the presence of the epilogue's branches cost the plain call 1-3 %, the
@@ -633,7 +678,7 @@ __global__ __launch_bounds__(64, 3) void gemm_sk_kernel(const SkArgs in_kernarg_
         p.timeline[(size_t)blockIdx.x * 8 + 5] = ((unsigned long long)xcc << 32) | hw;
     }
 #endif
-    const int logical = xcd_contiguous_id(blockIdx.x, p.waves);
+    const int logical = sk_generation_order(blockIdx.x, p.waves, p.gen_waves);
     if (logical < p.waves6)                                              // the FP6 region's waves come first
         sk_wave<true, G128, GR, DRAW>(p, logical, (FP6M_AS3 unsigned char*)smem);
     else

@@ -163,6 +163,8 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * from the counters), "gather" (its own activation gather on / off), "cells" (0: the m <= 16 kernel sums the shared
  * tiles of up to four rows through partial tiles, like those of more rows, instead of in the accumulate-and-count cells),
  * "xcd" (the m <= 16 kernel's partial tiles of 5 to 16 rows exchanged inside one XCD: 1 wherever possible, 0 never),
+ * "gen" (0: the decode kernel's chunks all of one length), "gen2" / "gen3" (per cent: the share of a SIMD that its planner
+ * assumes for the waves of the second / third generation, which sets their chunk lengths),
  * "verbose" (print every launch's configuration to stderr); knob = NULL clears all overrides.  Unknown knob ->
  * FP6M_ERR_ARG.  Not synchronised with GEMM calls running on other threads.  The library reads no environment
  * variables on a call (FP6M_VERBOSE is looked up once at load time).
@@ -182,11 +184,16 @@ size_t fp6m_workspace_elems(int prob_n, int max_par);
  * The concurrency rule is therefore the reference's, one call at a time per workspace (fp6_marlin_cuda.cpp:62-63):
  * calls with different workspaces may overlap on different streams, also when replayed from HIP graphs; two
  * overlapping calls must not share a workspace.
- * A device has FP6M_MAX_WORKSPACES regions.  The first FP6M_BUILTIN_WORKSPACES are part of the library's device code
- * (96 MiB per GPU, held until the process ends): a call whose workspace gets one of them allocates nothing, never
- * waits for the device and can be captured into a HIP graph as it is, like the reference's
- * (fp6_marlin_cuda_kernel.cu:864-880 allocates nothing).  The others get their memory from hipMalloc + hipMemset (both
- * synchronous) when a fifth, sixth .. workspace turns up, and keep it for good.  A workspace the library has not seen
+ * A device has FP6M_MAX_WORKSPACES regions.  The first FP6M_BUILTIN_WORKSPACES share one pool that is allocated once
+ * per device (hipMalloc + hipMemset, synchronous) by the first call that may wait for it -- fp6m_init_workspace, or the
+ * first GEMM call whose stream is not being captured -- after which a call with a new workspace allocates nothing and
+ * never waits for the device.  A call that is being captured before the pool exists uses, for its workspace, a slot of
+ * an array that is part of the library's device code (96 MiB per GPU, held until the process ends) instead: it
+ * allocates nothing either and can be captured as it is, like the reference's (fp6_marlin_cuda_kernel.cu:864-880), but
+ * atomics on that memory are slower (a 4096 x 4096 decode GEMM takes 6.6 instead of 5.7 us), so give a workspace its
+ * region with fp6m_init_workspace, or run one call with it, before capturing where that matters.  The other regions
+ * get their memory from hipMalloc + hipMemset when a fifth, sixth .. workspace turns up (not under capture), and keep
+ * it for good.  A workspace the library has not seen
  * takes a region nobody owns; when there is none, the region whose workspace has gone unused longest is handed over
  * after a hipDeviceSynchronize -- so callers that make a new workspace for every call (the reference's test.py:168 and
  * bench.py:44 do) never run out, at the price of that wait from the seventeenth workspace on.  Consequences: keep at

@@ -454,8 +454,13 @@ def test_baseline_config4_edge_shapes(oracle):
         fp6_marlin.mul(A.to(dev()), B.to(dev()), C, s.to(dev()), ws, 512)
         torch.cuda.synchronize()
         c_ref = (A.to(dev()).float() @ ref.to(dev()).float()).cpu().numpy()
-        err = oracle.rel_err(C.cpu().numpy(), c_ref)
+        c = C.cpu().numpy()
+        assert np.isfinite(c).all()
+        err = oracle.rel_err(c, c_ref)
         assert err <= TOL, err
+        for name, sl in (("INT4", slice(0, n - 512)), ("FP6", slice(n - 512, n))):     # each region alone, like `run`
+            e = oracle.rel_err(c[:, sl], c_ref[:, sl])
+            assert e <= TOL, f"rel err {e} on the {name} columns"
         assert int(ws.abs().sum().item()) == 0
 
 
@@ -531,6 +536,56 @@ def test_baseline_full_sizes_against_unpacked_words(oracle, kn, ms):
         assert lin.item() <= TOL, (m, k, n, lin.item())
         del ref
     del w, Bd, sd
+    torch.cuda.empty_cache()
+
+
+def test_decode_chunk_lengths_by_generation(capfd):
+    """One row on shapes whose chunk list exceeds the first generation of waves (4 x CUs): later generations get their
+    own, shorter chunks (`gen2` / `gen3`: their waves' assumed share of a SIMD in per cent; `gen` = 0: equal chunks).
+    Random words against the pinned unpacker, per 128-column tile, for the default and for forced ratios that send
+    tiles to two and to three generations, with group scales and without; every setting twice, bit-identical; a
+    column of A set to a unit vector returns the dequantised weight row exactly under every plan."""
+    import fp6_marlin
+    seen = set()
+    for (k, n, qc, gs) in [(4096, 12288, 256, 128), (8192, 8192, 256, -1), (2048, 28672, 512, 128)]:
+        g = torch.Generator().manual_seed(5 + k + n)
+        n4 = n - qc
+        B = torch.randint(-2 ** 31, 2 ** 31 - 1, (k * n4 // 8 + k * qc * 3 // 16,), generator=g, dtype=torch.int64).to(torch.int32)
+        ns = (n4 if gs == -1 else (k // gs) * n4) + qc
+        s = (torch.rand(ns, generator=g) * 0.01 + 0.001).half()
+        w = fp6_marlin.unpack_to_fp16(B, s, k, n, qc, gs).to(dev())
+        Bd, sd = B.to(dev()), s.to(dev())
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+        a = torch.randn((1, k), generator=g).half().to(dev())
+        hot = torch.zeros((1, k), dtype=torch.half, device=dev())
+        hot[0, k // 3] = 1.0
+        ref = a.float() @ w.float()
+        plans = set()
+        for knobs in ({"gen": 0}, {}, {"gen2": 50, "gen3": 45}, {"gen2": 90, "gen3": 80}, {"gen2": 40, "gen3": 10}):
+            print(f"case gen k={k} n={n} gs={gs} knobs={knobs}", flush=True)
+            with fp6_marlin.cabi.tuning(verbose=1, **knobs):
+                outs = []
+                for rep in range(2):
+                    C = torch.full((1, n), float("nan"), dtype=torch.half, device=dev())
+                    fp6_marlin.mul(a, Bd, C, sd, ws, qc, -1, -1, -1, 16, gs)
+                    torch.cuda.synchronize()
+                    outs.append(C)
+                plans.add(capfd.readouterr().err.strip().splitlines()[-1])
+                assert torch.equal(outs[0], outs[1])
+                te = tile_errors(outs[0], ref)
+                assert te.max().item() <= TOL, (k, n, knobs, int(te.argmax()), te.max().item())
+                C = torch.full((1, n), float("nan"), dtype=torch.half, device=dev())
+                fp6_marlin.mul(hot, Bd, C, sd, ws, qc, -1, -1, -1, 16, gs)
+                torch.cuda.synchronize()
+                capfd.readouterr()
+                assert torch.equal(C[0], w[k // 3]), (k, n, knobs)
+        assert int(ws.abs().sum().item()) == 0
+        assert len(plans) >= 2, plans                                    # the settings really led to different plans
+        seen |= plans
+        del w, Bd, sd
+    import re
+    assert any(re.search(r"by generation: \d+ tiles x \d+ chunks of \d+, [1-9]\d* x \d+ of \d+, 0 x", p) for p in seen), seen    # two generations
+    assert any(re.search(r"by generation: \d+ tiles x \d+ chunks of \d+, [1-9]\d* x \d+ of \d+, [1-9]", p) for p in seen), seen  # three
     torch.cuda.empty_cache()
 
 

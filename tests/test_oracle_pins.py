@@ -255,6 +255,42 @@ def test_int4_rounding_ties(oracle):
         assert np.array_equal(c2.numpy(), codes) and np.array_equal(s2.numpy(), s) and np.array_equal(r2.numpy(), ref)
 
 
+# --------------------------------------------------------------------------- FP6 scale rule of the harness
+
+def test_fp6_scale_rule_of_the_harness(oracle):
+    """gen_fp6_weight's scale, threshold and clamp (test.py:19-27) against an evaluation that shares none of its
+    lines (tests/fp6_scale_vectors.py): columns whose maxima are 28, 14 and 1.75 must get the scales 1, 0.5 and
+    0.0625 exactly (a divisor other than 28 fails here); every e3m2 value and its binary16 neighbours must land on
+    the right side of the truncation; entries below 0.0625 must come out as zero and an entry whose quotient rounds
+    above 28 as +-28 (a dropped threshold or clamp makes the cast refuse them); random columns bit for bit."""
+    import torch
+    import fp6_marlin
+    import fp6_scale_vectors as fv
+    w = fv.vectors()
+    k, n = w.shape
+    s_want, ref_true = fv.expected(w)
+    assert s_want[0] == 1.0 and s_want[1] == 0.5 and s_want[2] == 0.0625
+    a = fv.over_range_maximum()
+    assert ref_true[0, 3] == np.float16(np.float32(28) * np.float32(s_want[3])) and ref_true[1, 3] == -ref_true[0, 3]
+    assert (ref_true[:, 0][np.abs(w[:, 0]) < 0.0625] == 0).all()
+    # the harness itself (square w): codes of w / s, read back through its untransposed quantiser and dequantiser
+    _, ref_want = fv.expected(w, harness=True)
+    ref, packed, s_perm = oracle.gen_fp6_weight(w)
+    s_nat = np.array([s_perm[32 * (c // 32) + kr.scale_slot(c % 32)] for c in range(n)], dtype=np.float16)
+    assert np.array_equal(s_nat.view(np.uint16), s_want.view(np.uint16))
+    assert np.array_equal(ref.astype(np.float32), ref_want.astype(np.float32))        # (+0 and -0 compare equal)
+    # the shipped host packer (the rule's torch lines live there a second time) on the same vectors: the harness's
+    # layout bit for bit, and the true transpose (what Layer.pack uses) against the plain evaluation
+    B, s2, r2 = fp6_marlin.pack_mixed_weight(torch.from_numpy(w), n, -1)
+    assert np.array_equal(B.numpy(), packed.reshape(-1)) and np.array_equal(s2.numpy(), s_perm)
+    assert np.array_equal(r2.numpy().astype(np.float32), ref_want.astype(np.float32))
+    B, s2, r2 = fp6_marlin.pack_mixed_weight(torch.from_numpy(w), n, -1, harness_layout=False)
+    assert np.array_equal(s2.numpy(), s_perm)
+    assert np.array_equal(r2.numpy().astype(np.float32), ref_true.astype(np.float32))
+    assert np.array_equal((kr.decode_fp6(B.numpy(), k, n) * s_nat[None, :]).astype(np.float16).astype(np.float32),
+                          ref_true.astype(np.float32))
+
+
 # --------------------------------------------------------------------------- wire format (MX)
 
 def test_mixed_wire_format(oracle):

@@ -65,6 +65,28 @@ def test_every_fp6_code_and_range_errors():
         fp6_marlin.pack_mixed_weight(w.to(dev()), 96, -1)
 
 
+def test_fp6_scale_rule_vectors_through_the_gpu_packer():
+    """The constructed columns of tests/fp6_scale_vectors.py (exact scales 1, 0.5, 0.0625; values around every e3m2
+    grid point; entries below the 0.0625 threshold; a quotient that rounds above 28) through the on-GPU packer: scales
+    and check weight against the independent numpy evaluation, words against the host packer."""
+    import fp6_marlin
+    import fp6_scale_vectors as fv
+    import kernel_rules as kr
+    w = fv.vectors()
+    k, n = w.shape
+    s_want, ref_want = fv.expected(w)
+    # (the harness layout reads the flat [k, n] buffer as [n, k] without transposing; with k == n that is the transpose)
+    wt = torch.from_numpy(np.ascontiguousarray(w.T))
+    Bd, sd, rd = fp6_marlin.pack_mixed_weight(wt.to(dev()), n, -1, harness_layout=True)
+    Bh, sh, rh = fp6_marlin.pack_mixed_weight(wt, n, -1, harness_layout=True)
+    assert torch.equal(Bd.cpu(), Bh) and same_bits(sd, sh) and same_values(rd, rh)
+    Bd, sd, rd = fp6_marlin.pack_mixed_weight(torch.from_numpy(w).to(dev()), n, -1, harness_layout=False)
+    s_perm = sd.cpu().numpy()
+    s_nat = np.array([s_perm[32 * (c // 32) + kr.scale_slot(c % 32)] for c in range(n)], dtype=np.float16)
+    assert np.array_equal(s_nat.view(np.uint16), s_want.view(np.uint16))
+    assert np.array_equal(rd.cpu().numpy().astype(np.float32), ref_want.astype(np.float32))
+
+
 def test_layer_pack_on_gpu_matches_cpu_and_runs():
     import fp6_marlin
     torch.manual_seed(3)

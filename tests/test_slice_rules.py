@@ -164,3 +164,65 @@ def test_xcd_placement_covers_every_tile_part_once_on_one_xcd():
         for (fp6, group, part), x in seen.items():                                   # all parts of a tile on one XCD
             assert x == seen[(fp6, group, 0)]
         assert grid <= 8 * (-(-(tiles6 * ks6 + tiles4 * ks4) // 8) + max(ks6, ks4) * 2)   # little padding
+
+
+# ---- the decode kernel's generation-major wave order and its chunk sub-lists (gemm_sk.h: sk_generation_order, the
+# sub-list selection at the top of sk_wave; fp6m_gemm.hip: the chunk lengths by generation)
+
+def xcd_contiguous_id(b, total):
+    q, r, x = total >> 3, total & 7, b & 7
+    return x * q + min(x, r) + (b >> 3)
+
+
+def sk_generation_order(b, total, gen_waves):
+    if gen_waves == 0 or total <= gen_waves:
+        return xcd_contiguous_id(b, total)
+    per = gen_waves >> 3
+    x, i = b & 7, b >> 3
+    g = (i >= per) + (i >= 2 * per) + (i >= 3 * per)
+    rest = total - g * gen_waves
+    if rest >= gen_waves:
+        return g * gen_waves + x * per + (i - g * per)
+    return g * gen_waves + xcd_contiguous_id(((i - g * per) << 3) | x, rest)
+
+
+def test_generation_major_order_is_a_permutation_that_keeps_generations_apart():
+    for gen_waves in (0, 64, 1024):
+        for total in (1, 7, 8, 63, 64, 65, 100, 128, 129, 200, 1023, 1024, 1025, 1800, 2047, 2048, 2049, 2784, 2816, 4096):
+            if gen_waves and total > 4 * gen_waves:
+                continue                                                 # (the host plans at most four generations)
+            order = [sk_generation_order(b, total, gen_waves) for b in range(total)]
+            assert sorted(order) == list(range(total)), (gen_waves, total)
+            if gen_waves and total > gen_waves:
+                for b, pos in enumerate(order):                           # workgroup b is of generation (b / 8) / (gen / 8)
+                    assert pos // gen_waves == (b >> 3) // (gen_waves >> 3), (gen_waves, total, b)
+
+
+def test_chunk_sub_lists_cover_every_tile_once():
+    """Chunk j of the INT4 region -> (tile, first unit, units) through the three sub-lists, as the top of sk_wave does."""
+    for units in (32, 64, 86, 224):
+        for (ta, tb, tc), (qa, qb, qc) in [((252, 170, 26), (16, 11, 10)), ((5, 0, 0), (7, 7, 7)), ((3, 4, 5), (9, 5, 2)),
+                                           ((0, 6, 1), (8, 3, 3))]:
+            cpt = [-(-units // q) for q in (qa, qb, qc)]
+            chunks = [ta * cpt[0], tb * cpt[1], tc * cpt[2]]
+            covered = {}
+            for j in range(sum(chunks)):
+                if j >= chunks[0] + chunks[1]:
+                    jj, tile0, q, c = j - chunks[0] - chunks[1], ta + tb, qc, cpt[2]
+                elif j >= chunks[0]:
+                    jj, tile0, q, c = j - chunks[0], ta, qb, cpt[1]
+                else:
+                    jj, tile0, q, c = j, 0, qa, cpt[0]
+                if j < chunks[0]:
+                    tile = (jj * (((1 << 40) + c - 1) // c)) >> 40           # 40-bit reciprocal (also serves drawn chunks)
+                else:
+                    tile = jj if c <= 1 else (jj * (((1 << 32) + c - 1) // c)) >> 32   # 32-bit multiply-high
+                assert tile == jj // c
+                kb = (jj - tile * c) * q
+                length = min(q, units - kb)
+                assert length > 0
+                for u in range(kb, kb + length):
+                    key = (tile0 + tile, u)
+                    assert key not in covered
+                    covered[key] = j
+            assert len(covered) == (ta + tb + tc) * units
