@@ -68,7 +68,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset;
+    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -347,6 +347,29 @@ inline SliceRule make_rule(int units, int nslices)
     return r;
 }
 
+// k slices of the `ks` parts x `wk` waves of a tile (WaveRule, gemm_common.h).  With eight waves per workgroup and at
+// least two units for every wave, the second wave of every SIMD (waves 4-7) gets `young_pct` per cent of what the
+// first gets; otherwise all waves get the same.  What does not divide goes to the older waves first.
+inline WaveRule make_wave_rule(long long units, long long ks, int wk, int young_pct)
+{
+    WaveRule r;
+    if (ks < 1) ks = 1;
+    const long long per_part = units / ks;
+    long long lo = per_part / wk, ly = lo;
+    if (wk == 8 && per_part >= 16 && young_pct > 0 && young_pct < 100) {
+        lo = (per_part * 100 + 2 * (100 + young_pct)) / (4 * (100 + young_pct));     // per_part / (4 (1 + share)), rounded
+        if (4 * lo > per_part) lo = per_part / 4;
+        ly = (per_part - 4 * lo) / 4;
+        if (ly > lo) ly = lo;
+    }
+    const long long rem = units - ks * (4 * lo + (wk - 4) * ly);
+    r.lo = (int)lo;
+    r.ly = (int)ly;
+    r.eo = (int)(rem < 4 * ks ? rem : 4 * ks);
+    r.ey = (int)(rem - r.eo);
+    return r;
+}
+
 inline FastDiv make_div(long long d, long long max_n)
 {
     FastDiv f;
@@ -477,7 +500,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3}, {"young", &g_tuning.young},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -610,6 +633,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.slices4 = 0;
     a.xcd_local = 0;
     a.xm4_lo = a.xm4_hi = a.xm6_lo = a.xm6_hi = 0;
+    a.wrule[0] = a.wrule[1] = WaveRule{0, 0, 0, 0};
     if (row_mix) {
         // every tile spans all n columns of both segments: INT4 words of rows [0, k4), then the FP6 planes of the rest
         a.b_fp6_2 = a.b_int4 + (size_t)k4 * prob_n / 8;
@@ -632,6 +656,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     // workgroups per CU) beyond; 128 rows for large launches whose grid allows it (below).
     int mb = prob_m <= 16 ? 1 : (prob_m <= 32 ? 2 : 4);
     const Tuning tune = g_tuning;              // tuning/testing overrides (all unset in production)
+    // share of a SIMD that the second of two waves of a workgroup gets, in per cent of the first one's (make_wave_rule).
+    // Measured (alternating, us, equal slices -> 72 %): 8192 x 8192 at 8 / 16 / 128 / 256 rows 12.65 -> 12.03 / 13.2 -> 12.65 /
+    // 27.95 -> 27.4 / 42.3 -> 41.2, 8192 x 10240 at 16 rows 14.3 -> 13.7; 60 % and 85 % within 1 % of it.
+    const int young_pct = tune.young != kUnset ? tune.young : 72;
     if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4 || tune.mb == 8)) mb = tune.mb;
     // gemm_wm_kernel (four 64-row tiles share the dequantised fragments of a tile through LDS) was the kernel of launches
     // of 1024 rows and more until the 128-row tiles of the private-fragment kernel (below) got their dequantisation as
@@ -1062,6 +1090,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             } else {
                 a.rule[0] = make_rule(units, a.ks4 * cfg.wk);
                 a.rule[1] = make_rule(units, (a.ks6 > 0 ? a.ks6 : 1) * cfg.wk);
+                a.wrule[0] = make_wave_rule(units, a.ks4, cfg.wk, young_pct);
+                a.wrule[1] = make_wave_rule(units, a.ks6 > 0 ? a.ks6 : 1, cfg.wk, young_pct);
             }
             long long wgs = (long long)a.groups6 * a.ks6 + (long long)a.groups4 * a.ks4;
             a.div[0] = make_div(a.groups4, wgs);
@@ -1154,6 +1184,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             } else {
                 a.rule[0] = make_rule(units, a.ks4 * wk);
                 a.rule[1] = make_rule(units, a.ks6 * wk);
+                a.wrule[0] = make_wave_rule(units, a.ks4, wk, young_pct);
+                a.wrule[1] = make_wave_rule(units, a.ks6, wk, young_pct);
             }
             const long long wgs = (long long)a.tiles6 * a.ks6 + (long long)(a.tiles - a.tiles6) * a.ks4;
             a.div[0] = make_div(a.ks4, wgs);

@@ -34,6 +34,29 @@ __host__ __device__ inline int slice_begin(const SliceRule& r, int i)
     return i * r.q + (extra > 0 ? extra : 0);
 }
 
+// The k slices of a tile by wave, in units.  A workgroup of eight waves puts two on every SIMD, and the SIMD serves
+// the one that arrived first (waves 0-3) ahead of the other (waves 4-7): with equal slices the second wave of every
+// SIMD leaves its loop a third later than the first (8192 x 8192 at 128 rows: 14.3 against 19.6 us), and the
+// workgroup's reduction waits for it.  So a part (workgroup) of a tile gives its first four waves `lo` units each and
+// the others `ly` <= lo; what does not divide goes, a unit each, to the first `eo` older waves in (part, wave) order,
+// then to the first `ey` younger ones.  Four-wave workgroups have older waves only.  Slices follow each other along
+// k in (part, wave) order.
+struct WaveRule {
+    int lo, ly, eo, ey;
+};
+__host__ __device__ inline int wave_rule_begin(const WaveRule& r, int wk, int part, int wave)
+{
+    const int no = 4, ny = wk - 4;
+    const int eo_before = r.eo < no * part ? r.eo : no * part, ey_before = r.ey < ny * part ? r.ey : ny * part;
+    int eo_here = r.eo - no * part, ey_here = r.ey - ny * part;
+    eo_here = eo_here < 0 ? 0 : (eo_here > no ? no : eo_here);
+    ey_here = ey_here < 0 ? 0 : (ey_here > ny ? ny : ey_here);
+    const int base = part * (no * r.lo + ny * r.ly) + eo_before + ey_before;
+    if (wave < no) return base + wave * r.lo + (wave < eo_here ? wave : eo_here);
+    const int y = wave - no;                               // (wave == wk: the begin of the next part)
+    return base + no * r.lo + eo_here + y * r.ly + (y < ey_here ? y : ey_here);
+}
+
 // n / d for n, d < 65536 as the high half of n * ceil(2^32 / d) (exact in that range: the error term n * e / 2^32 stays
 // below 1 / d); magic 0 stands for a plain division (d = 1, or operands out of range).
 struct FastDiv {
@@ -68,7 +91,8 @@ struct GemmArgs {
     int k4, slices4;          // 0 = column mix
     // Division-free bookkeeping, prepared by the host (a 64-bit division costs a wave hundreds of scalar
     // instructions before its first load):
-    SliceRule rule[2];        // k slices of a tile: [0] INT4 tiles / INT4 rows (all tiles for m > 16), [1] FP6
+    SliceRule rule[2];        // k slices of a tile (row mix, shared-fragment kernel): [0] INT4 tiles / INT4 rows, [1] FP6
+    WaveRule wrule[2];        // ... (everything else): [0] INT4 tiles, [1] FP6 tiles
     FastDiv div[2];           // m <= 16: by groups4 / groups6;  m > 16: by ks4 / ks6 (the large-m kernel: [0] by ksplit)
     // weight planes in the gfx950 order (fp6m_repack_gfx950): [tile][k-block][MFMA lane] instead of the reference's
     // [k-block][64-column group][fragment owner]
@@ -131,6 +155,8 @@ __device__ __forceinline__ void preload_args(const GemmArgs& p)
     asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
                         "s"(p.div[0].d), "s"(p.div[0].magic), "s"(p.div[1].d), "s"(p.div[1].magic), "s"(p.fused));
     asm volatile("" : : "s"(p.xcd_local), "s"(p.xm4_lo), "s"(p.xm4_hi), "s"(p.xm6_lo), "s"(p.xm6_hi));
+    asm volatile("" : : "s"(p.wrule[0].lo), "s"(p.wrule[0].ly), "s"(p.wrule[0].eo), "s"(p.wrule[0].ey), "s"(p.wrule[1].lo),
+                        "s"(p.wrule[1].ly), "s"(p.wrule[1].eo), "s"(p.wrule[1].ey));
 }
 
 // The XCD (accelerator die: 32 CUs with an L2 of their own) this wave runs on.
@@ -334,10 +360,11 @@ template <bool G128, int WK = kWaves>
 __device__ __forceinline__ void wave_k_range(const GemmArgs& p, bool fp6, int part, int wave, int& begin, int& end)
 {
     constexpr int unit_steps = G128 ? 4 : 2;
-    const int wv = part * WK + wave;
-    const SliceRule rule = {fp6 ? p.rule[1].q : p.rule[0].q, fp6 ? p.rule[1].first_long : p.rule[0].first_long};
-    begin = slice_begin(rule, wv) * unit_steps;
-    end = slice_begin(rule, wv + 1) * unit_steps;
+    // (both entries are read at fixed offsets and selected by value: an index would become a dependent scalar load)
+    const WaveRule rule = {fp6 ? p.wrule[1].lo : p.wrule[0].lo, fp6 ? p.wrule[1].ly : p.wrule[0].ly,
+                           fp6 ? p.wrule[1].eo : p.wrule[0].eo, fp6 ? p.wrule[1].ey : p.wrule[0].ey};
+    begin = wave_rule_begin(rule, WK, part, wave) * unit_steps;
+    end = wave_rule_begin(rule, WK, part, wave + 1) * unit_steps;
 }
 
 // ------------------------------------------------------------------------------------------------ loads, waits, dequantisers

@@ -556,7 +556,8 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
         group = local - ti.part * groups;
     }
     const int ks = ti.fp6 ? p.ks6 : p.ks4;
-    const SliceRule srule = {ti.fp6 ? p.rule[1].q : p.rule[0].q, ti.fp6 ? p.rule[1].first_long : p.rule[0].first_long};
+    const WaveRule wrule = {ti.fp6 ? p.wrule[1].lo : p.wrule[0].lo, ti.fp6 ? p.wrule[1].ly : p.wrule[0].ly,
+                            ti.fp6 ? p.wrule[1].eo : p.wrule[0].eo, ti.fp6 ? p.wrule[1].ey : p.wrule[0].ey};
     ti.tcol = group * WN + wn;
     ti.region_n = ti.fp6 ? p.qc : p.n4;
     const bool tile_valid = ti.tcol * kTileN < ti.region_n;
@@ -566,8 +567,8 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
 
     constexpr int unit_steps = G128 ? 4 : 2;
     const int kp = ti.part * WK + wk;
-    int step_begin = slice_begin(srule, kp) * unit_steps;
-    int step_end = slice_begin(srule, kp + 1) * unit_steps;
+    int step_begin = wave_rule_begin(wrule, WK, ti.part, wk) * unit_steps;
+    int step_end = wave_rule_begin(wrule, WK, ti.part, wk + 1) * unit_steps;
     ti.a_step0 = 0;
     const bool region6 = ti.fp6;                                         // the workgroup's column region
     if (p.k4) row_mix_slice(p, kp, ti, step_begin, step_end);            // per wave: INT4 or FP6 rows of the tile

@@ -226,3 +226,58 @@ def test_chunk_sub_lists_cover_every_tile_once():
                     assert key not in covered
                     covered[key] = j
             assert len(covered) == (ta + tb + tc) * units
+
+
+# ---- k slices by wave with the second wave of every SIMD given less (gemm_common.h: WaveRule / wave_rule_begin;
+# fp6m_gemm.hip: make_wave_rule)
+
+def make_wave_rule(units, ks, wk, young_pct):
+    ks = max(ks, 1)
+    per_part = units // ks
+    lo = ly = per_part // wk
+    if wk == 8 and per_part >= 16 and 0 < young_pct < 100:
+        lo = (per_part * 100 + 2 * (100 + young_pct)) // (4 * (100 + young_pct))
+        if 4 * lo > per_part:
+            lo = per_part // 4
+        ly = min((per_part - 4 * lo) // 4, lo)
+    rem = units - ks * (4 * lo + (wk - 4) * ly)
+    eo = min(rem, 4 * ks)
+    return lo, ly, eo, rem - eo
+
+
+def wave_rule_begin(rule, wk, part, wave):
+    lo, ly, eo, ey = rule
+    no, ny = 4, wk - 4
+    eo_here = min(max(eo - no * part, 0), no)
+    ey_here = min(max(ey - ny * part, 0), ny)
+    base = part * (no * lo + ny * ly) + min(eo, no * part) + min(ey, ny * part)
+    if wave < no:
+        return base + wave * lo + min(wave, eo_here)
+    y = wave - no
+    return base + no * lo + eo_here + y * ly + min(y, ey_here)
+
+
+def test_wave_slices_tile_the_k_range_and_favour_the_older_waves():
+    for wk in (4, 8):
+        for units in list(range(1, 70)) + [86, 128, 172, 224, 448]:
+            for ks in (1, 2, 3, 4, 5, 7, 8, 16):
+                if ks * wk > units and units > 8:
+                    continue                                              # (the host keeps a unit for every wave)
+                for pct in (100, 85, 70, 50):
+                    rule = make_wave_rule(units, ks, wk, pct)
+                    assert min(rule) >= 0 and rule[3] <= (wk - 4) * ks and rule[2] <= 4 * ks, (units, ks, wk, pct, rule)
+                    pos = 0
+                    for part in range(ks):
+                        lens = []
+                        for w in range(wk):
+                            b, e = wave_rule_begin(rule, wk, part, w), wave_rule_begin(rule, wk, part, w + 1)
+                            assert b == pos and e >= b, (units, ks, wk, pct, part, w)
+                            pos = e
+                            lens.append(e - b)
+                        assert wave_rule_begin(rule, wk, part, wk) == (wave_rule_begin(rule, wk, part + 1, 0))
+                        if wk == 8:
+                            assert min(lens[:4]) >= max(lens[4:]), (units, ks, pct, lens)       # older waves never get less
+                            if pct < 100 and units // ks >= 16:
+                                assert sum(lens[4:]) <= sum(lens[:4])
+                        assert max(lens[:4]) - min(lens[:4]) <= 1 and max(lens[4:] or [0]) - min(lens[4:] or [0]) <= 1
+                    assert pos == units, (units, ks, wk, pct, rule)
