@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the headline workload (mean of its four GEMMs): FETCH_SIZE + WRITE_SIZE from two
 # `rocprofv3 --pmc` runs of `bench.py --traffic-probe`, each scaled by what the same counter reads for a
 # 256 MiB device copy (x2.000 and x1.000); figures in profiles/gemm_sk_kernel_decode7b_hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28882764
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28742537
 TRAFFIC_PROFILE = "profiles/gemm_sk_kernel_decode7b_hbm_traffic.txt"
 MFMA_F16_PEAK_TFLOPS = 2500.0
 LLAMA7B = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
