@@ -172,7 +172,7 @@ const char* fp6m_strerror(int code)
         case FP6M_ERR_ARG: return "invalid argument";
         case FP6M_ERR_HIP: return "HIP runtime error";
         case FP6M_ERR_NO_GPU_CODE: return "library built without gfx950 kernels";
-        case FP6M_ERR_SCRATCH: return "no scratch for this call: its partial sums do not fit fp6m_mul_static's array (use fp6m_mul), or the device's table of workspace regions is full (fp6m_release_workspace)";
+        case FP6M_ERR_SCRATCH: return "no scratch for this call: its partial sums do not fit fp6m_mul_static's array (fp6m_mul has room for them), or a workspace beyond the built-in regions was first used while its stream was capturing (call fp6m_init_workspace before the capture)";
         default: return "unknown fp6m error";
     }
 }

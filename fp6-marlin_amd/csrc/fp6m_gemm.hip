@@ -25,7 +25,6 @@
 // gemm_sk.h      gemm_sk_kernel (one row: the decode kernel)
 // gemm_m16.h     gemm_m16_kernel (m <= 16)
 // gemm_mb.h      gemm_mb_kernel (16 < m)
-// gemm_wm.h      gemm_wm_kernel (fragments shared by four row tiles; superseded, reachable through the tuning hook)
 // this file      activation gather, per-device scratch, dispatch and the extern "C" entry points
 #include <hip/hip_runtime.h>
 
@@ -39,7 +38,6 @@
 #include "gemm_m16.h"
 #include "gemm_sk.h"
 #include "gemm_mb.h"
-#include "gemm_wm.h"
 
 namespace fp6m {
 
@@ -68,7 +66,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, wm = kUnset, ksplit = kUnset, wn = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset;
+    int mb = kUnset, ksplit = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -470,21 +468,6 @@ void launch_mb(const GemmArgs& a, bool g128, int wk, dim3 grid, hipStream_t stre
     }
 }
 
-void launch_wm(const GemmArgs& a, bool g128, int wn, dim3 grid, hipStream_t stream)
-{
-    if (wn == 2) {
-        if (g128)
-            hipLaunchKernelGGL((gemm_wm_kernel<true, 2>), grid, dim3(512), 0, stream, a);
-        else
-            hipLaunchKernelGGL((gemm_wm_kernel<false, 2>), grid, dim3(512), 0, stream, a);
-    } else {
-        if (g128)
-            hipLaunchKernelGGL((gemm_wm_kernel<true, 1>), grid, dim3(512), 0, stream, a);
-        else
-            hipLaunchKernelGGL((gemm_wm_kernel<false, 1>), grid, dim3(512), 0, stream, a);
-    }
-}
-
 }  // namespace fp6m
 
 extern "C" {
@@ -499,7 +482,7 @@ int fp6m_tuning_set(const char* knob, int value)
         return FP6M_OK;
     }
     const struct { const char* name; int* field; } knobs[] = {
-        {"mb", &g_tuning.mb}, {"wm", &g_tuning.wm}, {"ksplit", &g_tuning.ksplit}, {"wn", &g_tuning.wn},
+        {"mb", &g_tuning.mb}, {"ksplit", &g_tuning.ksplit},
         {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3}, {"young", &g_tuning.young},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
@@ -661,14 +644,6 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     // 27.95 -> 27.4 / 42.3 -> 41.2, 8192 x 10240 at 16 rows 14.3 -> 13.7; 60 % and 85 % within 1 % of it.
     const int young_pct = tune.young != kUnset ? tune.young : 72;
     if (tune.mb != kUnset && prob_m > 16 && (tune.mb == 2 || tune.mb == 4 || tune.mb == 8)) mb = tune.mb;
-    // gemm_wm_kernel (four 64-row tiles share the dequantised fragments of a tile through LDS) was the kernel of launches
-    // of 1024 rows and more until the 128-row tiles of the private-fragment kernel (below) got their dequantisation as
-    // asm: those now measure 1-5 % faster on every large shape (m = 1024: 8192 x 16384 268 vs 272 us, 8192 x 28672
-    // 483 vs 507, 16384 x 16384 504 vs 527, 8192 x 57344 957 vs 1006).  It stays reachable through the tuning hook.
-    const long long weights = (long long)prob_n * prob_k;
-    bool shared_frags = false;
-    if (tune.wm != kUnset) shared_frags = prob_m > 16 && tune.wm != 0;
-    if (row_mix) shared_frags = false;                                // its waves run in lock step on one segment
     // Row mix: the kWaves * ks slices of a tile are dealt to the two segments in proportion to their cost (an FP6
     // step costs about two INT4 steps), at least one each.
     auto deal_slices = [&](int total) {
@@ -679,7 +654,6 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         if (n6 < 1) n6 = 1;
         return (int)(total - n6);
     };
-    if (shared_frags) mb = 4;
     // 128-row tiles (eight blocks per wave, accumulators in the accumulation registers, one wave per SIMD): every
     // dequantised fragment feeds 16 MFMAs instead of 8.  One workgroup per CU is resident, so the launch takes whole
     // rounds of 128 rows per CU; 64-row tiles (two workgroups per CU, or one of eight waves) take 1.13-1.32 x as long for
@@ -689,7 +663,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     // (8192 x 8192: m = 384 74 -> 62 us, m = 512 88 -> 69, m = 768 136 -> 121, m = 1024 177 -> 137; 4096 x 4096 at
     // m = 640 40 -> 36, at m = 512 the rule keeps 64-row tiles: 28 vs 36; 8192 x 5120 at m = 512 69 -> 60, at m = 2048
     // 233 -> 188, at m = 896 it keeps them: 109 vs 117.)
-    if (!shared_frags && !row_mix && tune.mb == kUnset && mb == 4 && prob_m > 64) {
+    if (!row_mix && tune.mb == kUnset && mb == 4 && prob_m > 64) {
         const long long rows8 = prob_m < 128LL * max_par ? prob_m : 128LL * max_par;
         const long long tiles_n = prob_n / kTileN;
         const long long wgs8 = tiles_n * ((rows8 + 127) / 128), wgs4 = tiles_n * ((rows8 + 63) / 64);
@@ -734,37 +708,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         const size_t tile_bytes = (size_t)mb * 16 * kTileN * sizeof(float);
         const long long traffic_cap = (long long)prob_k / (64LL * a.m) > 0 ? (long long)prob_k / (64LL * a.m) : 1;
         const long long env_ks = tune.ksplit != kUnset ? tune.ksplit : 0;
-        if (shared_frags) {
-            gather_pass();
-            // two tiles per workgroup also share the A slabs: pays once the weights are large enough that
-            // halving the grid still fills the chip (measured: 8192 x 16384 and up; one tile per workgroup is
-            // what the tuning knob and the tests still reach)
-            int wn = weights >= (128LL << 20) ? 2 : 1;
-            if (tune.wn != kUnset) wn = tune.wn == 2 ? 2 : 1;
-            const int wk = 2 / wn;
-            a.groups6 = (a.tiles6 + wn - 1) / wn;
-            a.groups4 = (a.tiles - a.tiles6 + wn - 1) / wn;
-            const int groups_m = (mtiles + fp6m::kWmRows - 1) / fp6m::kWmRows;
-            const long long base = (long long)(a.groups6 + a.groups4) * groups_m;
-            long long ks = cus / base;
-            const long long ks_k = units / (wk * 2) > 0 ? units / (wk * 2) : 1;
-            const long long cap = (long long)prob_k / (16LL * rows_per_tile) > 0 ? (long long)prob_k / (16LL * rows_per_tile) : 1;
-            if (ks > ks_k) ks = ks_k;
-            if (ks > cap) ks = cap;
-            if (sms > 0 && ks > sms) ks = sms;
-            if (env_ks >= 1) ks = env_ks;
-            if (ks < 1) ks = 1;
-            if (fixed_scratch && ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > scratch_bytes) return FP6M_ERR_SCRATCH;
-            while (ks > 1 && (size_t)a.tiles * mtiles * ks * tile_bytes > scratch_bytes) ks--;
-            a.ksplit = (int)ks;
-            a.rule[0] = a.rule[1] = make_rule(units, a.ksplit * wk);
-            a.div[0] = a.div[1] = make_div(a.ksplit, (long long)(a.groups6 + a.groups4) * a.ksplit);
-            dim3 grid((unsigned)((a.groups6 + a.groups4) * a.ksplit), (unsigned)groups_m);
-            if (tune.verbose)
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: shared fragments, %d tile(s) x %d k slice(s), row tiles %d ks=%d grid=%ux%u\n",
-                        a.m, prob_n, prob_k, wn, wk, mtiles, a.ksplit, grid.x, grid.y);
-            fp6m::launch_wm(a, g128, wn, grid, st);
-        } else if (mb == 1 && !row_mix && (tune.sk != kUnset ? tune.sk != 0 && a.m <= 4 : a.m == 1) && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24) &&
+        if (mb == 1 && !row_mix && (tune.sk != kUnset ? tune.sk != 0 && a.m <= 4 : a.m == 1) && prob_k / 64 < 65536 && (long long)a.tiles * (prob_k / 64) < (1 << 24) &&
                    (long long)prob_k * prob_n / 2 < (1LL << 32) && (long long)(prob_n / 128) * max_par >= 2 &&
                    (g128 || n4 == 0 || units >= 2)) {
             // (k = 64 with per-column scales stays with the workgroup kernel: an INT4 chunk of that single unit is two

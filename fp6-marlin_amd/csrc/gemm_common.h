@@ -91,9 +91,9 @@ struct GemmArgs {
     int k4, slices4;          // 0 = column mix
     // Division-free bookkeeping, prepared by the host (a 64-bit division costs a wave hundreds of scalar
     // instructions before its first load):
-    SliceRule rule[2];        // k slices of a tile (row mix, shared-fragment kernel): [0] INT4 tiles / INT4 rows, [1] FP6
+    SliceRule rule[2];        // k slices of a tile (row mix): [0] INT4 tiles / INT4 rows, [1] FP6
     WaveRule wrule[2];        // ... (everything else): [0] INT4 tiles, [1] FP6 tiles
-    FastDiv div[2];           // m <= 16: by groups4 / groups6;  m > 16: by ks4 / ks6 (the large-m kernel: [0] by ksplit)
+    FastDiv div[2];           // m <= 16: by groups4 / groups6;  m > 16: by ks4 / ks6
     // weight planes in the gfx950 order (fp6m_repack_gfx950): [tile][k-block][MFMA lane] instead of the reference's
     // [k-block][64-column group][fragment owner]
     int native;

@@ -717,9 +717,8 @@ __device__ __forceinline__ void stream_tile_mbp(const GemmArgs& p, const TileInf
 // Epilogue of the MB kernel: block by block, the four k slices are summed through LDS (wave wk finishes
 // rows wk, wk+4, ... of the block, lane L owns columns 2L, 2L+1); then C is written, or the rows are
 // published and the last-arriving workgroup of the (tile, row tile) gathers all parts in part order.
-// `smem`, `flag` and `valid` belong to the WK waves that share a tile and a row tile (the whole workgroup in
-// gemm_mb_kernel, one of WM groups in gemm_wm_kernel); a group without rows goes through the barriers
-// without touching memory.
+// `smem`, `flag` and `valid` belong to the WK waves that share a tile and a row tile (the whole workgroup); a
+// workgroup without rows goes through the barriers without touching memory.
 template <int MB, int WK = kWaves, int BPR = 1>
 __device__ __forceinline__ void wg_finish_mb(const GemmArgs& p, const TileInfo& ti, int wk, int ks, int slot_base,
                                              f4 (&acc)[MB][8],

@@ -157,7 +157,7 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * Testing / tuning hook: overrides one of the dispatcher's per-shape choices for all later calls in this process.
  * No counterpart in the reference (whose only such knob is the `sms` argument).  knob = "ksplit" (k parts per tile),
  * "wk16" / "wk" (waves per workgroup of the m <= 16 / m > 16 kernel: 4 or 8), "mb" (16-row blocks per wave: 2, 4 or 8),
- * "wm" / "wn" (shared-fragment kernel on/off, its column tiles per workgroup), "pair" (paired activation fetch on/off),
+ * "pair" (paired activation fetch on/off),
  * "sk" (the one-wave decode kernel on for m <= 4 / off), "share" / "share6" (k units per chunk of its work list: both
  * regions / the FP6 region only), "cap" (the waves it aims at), "wgs" (exactly that many waves, one-unit chunks drawn
  * from the counters), "gather" (its own activation gather on / off), "cells" (0: the m <= 16 kernel sums the shared

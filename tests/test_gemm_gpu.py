@@ -220,31 +220,12 @@ def test_partial_tiles_exchanged_through_one_xcd(oracle):
     assert oracle.rel_err(outs[1].cpu().numpy(), c_ref) <= TOL
 
 
-def test_shared_fragment_kernel(oracle):
-    """The kernel that large launches use (four row tiles share a tile's dequantised fragments; one or two
-    column tiles per workgroup), forced onto small problems: ragged row tiles, odd tile counts in both regions,
-    per-column and group scales, one to three k parts."""
-    for wn in (1, 2):
-        e = {"FP6M_WM": 1, "FP6M_WN": wn}
-        run(oracle, 256, 512, 1024, qc=256, ksplit=1, env=e)
-        run(oracle, 256, 512, 1024, qc=256, gs=128, ksplit=1, env=e)
-        run(oracle, 64, 768, 1024, qc=128, ksplit=1, env=e)
-        run(oracle, 100, 1024, 1280, qc=128, gs=128, env=e)
-        run(oracle, 33, 256, 512, qc=128, env=e)
-        run(oracle, 17, 256, 64, qc=-1, env=e)
-        run(oracle, 300, 2048, 2048, qc=256, gs=128, env=e)
-        run(oracle, 300, 2304, 2048, qc=384, gs=128, ksplit=3, env=e)
-        run(oracle, 520, 512, 512, qc=512, ksplit=2, env=e)            # all FP6
-        run(oracle, 1100, 256, 1024, qc=-1, gs=128, max_par=16, env=e)  # second launch of 76 rows
-    run(oracle, 1024, 768, 1024, qc=256, gs=128)                       # default dispatch stays on the other kernel
-
-
 def test_eight_row_blocks_per_wave(oracle):
     """The m > 16 kernel with eight 16-row blocks per wave (128-row tiles, accumulators in the accumulation
     registers), forced onto small problems: ragged row tiles, both regions, both scale modes, k splits through the
     scratch, several launches, and one-hot rows bit for bit."""
     for pair in (1,):                                                   # (eight blocks always fetch A by pairs of steps)
-        e = {"FP6M_MB": 8, "FP6M_WM": 0, "FP6M_PAIR": pair}
+        e = {"FP6M_MB": 8, "FP6M_PAIR": pair}
         for m in (17, 100, 128, 129, 300):
             run(oracle, m, 512, 1024, qc=256, gs=128, env=e)
             run(oracle, m, 512, 1024, qc=256, env=e)
@@ -255,8 +236,8 @@ def test_eight_row_blocks_per_wave(oracle):
         run(oracle, 2100, 256, 1024, qc=-1, gs=128, max_par=16, env=e)  # second launch of 52 rows
         for n, k, qc in [(512, 256, 256), (768, 1024, 256)]:
             for gs in (-1, 128):
-                one_hot_case(oracle, 200, n, k, qc, gs, {"mb": 8, "wm": 0, "pair": pair})
-                one_hot_case(oracle, 130, n, k, qc, gs, {"mb": 8, "wm": 0, "ksplit": 2, "pair": pair})
+                one_hot_case(oracle, 200, n, k, qc, gs, {"mb": 8, "pair": pair})
+                one_hot_case(oracle, 130, n, k, qc, gs, {"mb": 8, "ksplit": 2, "pair": pair})
 
 
 def test_dispatch_picks_128_row_tiles_where_they_fill_the_chip(oracle, capfd):
@@ -410,8 +391,8 @@ def one_hot_case(oracle, m, n, k, qc, gs, knobs=None, max_par=16):
 
 def test_one_hot_rows_return_exact_weight_rows(oracle):
     """A = unit vectors: C must equal rows of the dequantised weight bit for bit (pins layout and scale order) --
-    for the m <= 16 kernel, both loops of the m > 16 kernel, its two-block form and eight-wave form, and the
-    shared-fragment kernel with one and two column tiles, with per-column and with group-128 scales."""
+    for the m <= 16 kernel, both loops of the m > 16 kernel, its two-block form and eight-wave form, with
+    per-column and with group-128 scales."""
     shapes = [(512, 256, 256), (768, 1024, 256), (256, 512, 256), (640, 128, -1)]
     for n, k, qc in shapes:
         for gs in (-1, 128):
@@ -429,9 +410,7 @@ def test_one_hot_rows_return_exact_weight_rows(oracle):
             one_hot_case(oracle, 100, n, k, qc, gs, {"pair": 0})
             one_hot_case(oracle, 40, n, k, qc, gs, {"pair": 1})
             one_hot_case(oracle, 130, n, k, qc, gs, {"ksplit": 2})      # partial tiles through the scratch
-            for wn in (1, 2):                                           # shared-fragment kernel
-                one_hot_case(oracle, 300, n, k, qc, gs, {"wm": 1, "wn": wn})
-            one_hot_case(oracle, 1100, n, k, qc, gs, {"wm": 1, "wn": 1})   # 1024 rows, then a launch of 76
+            one_hot_case(oracle, 300, n, k, qc, gs, {"mb": 4})          # five 64-row tiles
             one_hot_case(oracle, 1100, n, k, qc, gs, {"pair": 1})
 
 
@@ -470,8 +449,8 @@ MSWEEP = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024]
 
 
 def baseline_cases():
-    """(k, n) -> row counts: every shape x M of the benchmark's Llama-2-7B, Llama-2-70B and M-sweep configurations, plus one shape of the two-tile
-    shared-fragment kernel."""
+    """(k, n) -> row counts: every shape x M of the benchmark's Llama-2-7B, Llama-2-70B and M-sweep configurations, plus one
+    launch of 1024 rows on a weight of 128 Mi elements."""
     cases = {}
     for k, n in LLAMA7B:
         cases.setdefault((k, n), set()).update([1, 16])                 # config 1 (M = 1) and its M = 16 bench rows

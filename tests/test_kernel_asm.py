@@ -81,7 +81,7 @@ def test_scalar_operands_of_asm_loads(asm):
 def test_mfma_loops_keep_accumulators_in_place(asm):
     seen = 0
     for name, ins in kernels(asm):
-        if "gemm_mb_kernel" not in name and "gemm_wm_kernel" not in name:
+        if "gemm_mb_kernel" not in name:
             continue
         seen += 1
         meta = asm[asm.index(".name:           " + name) - 400:asm.index(".name:           " + name) + 800]
@@ -97,9 +97,9 @@ def test_mfma_loops_keep_accumulators_in_place(asm):
             continue
         assert not moved, f"{name}: accumulator copies between MFMAs: {moved[:4]}"
     # (group scales or not) x ((MB 2, MB 4, MB 4 with paired A fetches) x (4, 8 k slices) + MB 2 paired with 8 slices +
-    # MB 8 + (one, two tiles per workgroup)), and a second build without the optional paths of those that the
-    # dispatcher picks by itself (6 x 2 less one that would spill)
-    assert seen == 31
+    # MB 8), and a second build without the optional paths of those that the dispatcher picks by itself (6 x 2 less
+    # one that would spill)
+    assert seen == 27
     assert not re.findall(r"\.vgpr_spill_count:\s+[1-9]", asm), "a kernel spills VGPRs"
     # nothing may live in private memory either: a pointer that the compiler keeps on the stack costs the decode loop a
     # scratch load and a full `s_waitcnt vmcnt(0)` per step (seen once with pointers advanced under uniform branches)
@@ -114,7 +114,7 @@ def test_kernel_arguments_are_loaded_in_one_batch(asm):
     argument block itself: four loads, one wait, and no other argument load anywhere."""
     seen = 0
     for name, ins in kernels(asm):
-        if not any(k in name for k in ("gemm_m16_kernel", "gemm_sk_kernel", "gemm_mb_kernel", "gemm_wm_kernel")):
+        if not any(k in name for k in ("gemm_m16_kernel", "gemm_sk_kernel", "gemm_mb_kernel")):
             continue
         seen += 1
         if "gemm_sk_kernel" in name:
@@ -126,4 +126,4 @@ def test_kernel_arguments_are_loaded_in_one_batch(asm):
         # the code of the epilogue may be laid out ahead of the loops: its loads (fused-epilogue pointers) do not count
         late = [(n, l) for n, l in late if not re.search(r"0x(c8|d0|d8)$", l)]
         assert not late, f"{name}: kernel-argument loads after the prologue: {late[:4]}"
-    assert seen == 73            # (the m <= 16 kernel's builds with the partial tiles exchanged inside one XCD are 8 of them)
+    assert seen == 69            # (the m <= 16 kernel's builds with the partial tiles exchanged inside one XCD are 8 of them)

@@ -100,9 +100,8 @@ def test_gemm_on_gfx950_layout_is_bit_identical():
         gpu_case(oracle, m, 512, 512, 256, -1)
     gpu_case(oracle, 16, 2048, 512, 512, -1)                                           # all FP6
     gpu_case(oracle, 16, 2048, 512, -1, 128)                                           # all INT4
-    for wn in (1, 2):                                                                  # the large-m kernel, forced
-        gpu_case(oracle, 300, 1024, 1024, 256, 128, {"FP6M_WM": 1, "FP6M_WN": wn})
-        gpu_case(oracle, 64, 512, 768, 128, -1, {"FP6M_WM": 1, "FP6M_WN": wn})
+    gpu_case(oracle, 300, 1024, 1024, 256, 128, {"FP6M_MB": 8})                        # 128-row tiles, forced
+    gpu_case(oracle, 300, 1024, 1024, 256, 128, {"FP6M_MB": 4})
 
 
 @pytest.mark.gpu
