@@ -66,7 +66,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, ksplit = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset;
+    int mb = kUnset, ksplit = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset, cls = kUnset, cus = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -483,7 +483,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"ksplit", &g_tuning.ksplit},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3}, {"young", &g_tuning.young},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3}, {"young", &g_tuning.young}, {"cls", &g_tuning.cls}, {"cus", &g_tuning.cus},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -593,7 +593,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
         scratch_bytes = kStaticTileBytes;
     }
     if (int rc = workspace_region(dev, workspace, !fixed_scratch, fu.a_cols != nullptr, st, &sc)) return rc;
-    const int cus = sc.cus;
+    const int cus = g_tuning.cus != kUnset && g_tuning.cus > 0 ? g_tuning.cus : sc.cus;   // (the knob: small test problems on a pretended small chip)
     const int xcd_placement = sc.xcd_placement;
     float* const scratch = fixed_scratch ? sc.static_scratch : sc.partials;
 
@@ -616,7 +616,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
     a.slices4 = 0;
     a.xcd_local = 0;
     a.xm4_lo = a.xm4_hi = a.xm6_lo = a.xm6_hi = 0;
-    a.wrule[0] = a.wrule[1] = WaveRule{0, 0, 0, 0};
+    a.wrule[0] = a.wrule[1] = a.wrule_b = WaveRule{0, 0, 0, 0};
+    a.groups4b = 0;
+    a.ks4b = 1;
+    a.div_b = FastDiv{1, 0};
     if (row_mix) {
         // every tile spans all n columns of both segments: INT4 words of rows [0, k4), then the FP6 planes of the rest
         a.b_fp6_2 = a.b_int4 + (size_t)k4 * prob_n / 8;
@@ -959,6 +962,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // workgroups per CU (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle).
             const long long target_wgs = (long long)cus * 3 / 2;
             long long ks = (target_wgs + groups / 2) / groups;
+            long long cls_na = 0, cls_cb = 0;                           // two classes of INT4 tiles (below): tiles of the first, parts of the second
             if (ks > ks_limit(cfg.wk)) ks = ks_limit(cfg.wk);
             if (ks < 1) ks = 1;
             // Second opinion from a small cost model (per-workgroup timelines on MI355X): a wave takes about 0.40 us per
@@ -1004,6 +1008,38 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     cfg.wk = best_wk;
                     ks = best;
                 }
+                // Two classes of INT4 tiles.  A few more tiles than CUs leave the grid above lopsided whatever the split
+                // (6656 x 35328: 274 INT4 tiles, so 22 CUs run two workgroups and end at 29 us where the others end at
+                // 19).  So: as many whole tiles as fill every CU once make the first cus workgroups of the grid (with the
+                // FP6 region's); the tiles left over are cut into parts and dealt, as the later workgroups of the grid,
+                // over the CUs a second time.  Model, from the same timelines: while two four-wave workgroups share a
+                // CU the first runs at 0.73 and the second at 0.52 of the rate one has alone (1.25 together); whoever is
+                // left alone runs at full rate.  Measured (16 rows, us): 6656 x 35328 31.4 -> 26.4, 8192 x 43520
+                // 39.0 -> 33.8 (model: 33.7); with the first class split as well (fewer tiles than CUs) every forced
+                // plan lost 5-30 %, so that is not tried.
+                if (!row_mix && cfg.wn == 1 && sms <= 0 && env_ks < 1 && tune.wk16 == kUnset && a.groups4 > 0 &&
+                    !(tune.cls != kUnset && tune.cls == 0)) {
+                    const double ra = 0.727, rb = 0.523;
+                    const long long c6 = a.groups6 ? ks6_of(1, 4) : 0;
+                    const long long first = cus - a.groups6 * c6;                      // workgroups the first round has left
+                    const long long na = a.groups4 < first ? a.groups4 : first, nb = a.groups4 - na;
+                    if (first >= 1 && nb > 0 && nb <= cus) {                           // (else: one class does it / a third round)
+                        // (the few tiles of the second class may be cut finer than a split of all tiles may: their partial
+                        // tiles are a small part of the traffic, and priced below)
+                        long long cb = cus / nb;
+                        const long long cb_limit = prob_k / 32 / 16 < ks_units(4) ? prob_k / 32 / 16 : ks_units(4);
+                        if (cb > cb_limit) cb = cb_limit;
+                        if (cb < 1) cb = 1;
+                        const double ua = (double)units, ub = (double)((units + cb - 1) / cb);
+                        const double both = ub / rb <= ua / ra ? ua + ub * (1.0 - ra) / rb : ub + ua * (1.0 - rb) / ra;
+                        const double partial_us = ((cb > 1 ? nb * cb : 0) + (c6 > 1 ? a.groups6 * c6 : 0)) * a.m * 0.0005;
+                        const double us = both * unit_steps / 4 * 0.40 + partial_us;
+                        if (tune.cls == 1 || us < 0.96 * model_us(cfg.wk, ks)) {
+                            cls_na = na;
+                            cls_cb = cb;
+                        }
+                    }
+                }
             }
             if (tune.wk16 != kUnset) cfg.wk = tune.wk16 == 8 ? 8 : 4;
             const long long ks_k = ks_units(cfg.wk);
@@ -1017,6 +1053,18 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.ks4 = (int)ks;
             a.ks6 = (int)ks6_of(ks, cfg.wk);
             if (sms > 0 && a.ks6 > sms) a.ks6 = sms;
+            if (cls_na > 0) {
+                const long long c6 = a.groups6 ? ks6_of(1, 4) : 0, nb = a.groups4 - cls_na;
+                const size_t slots = (size_t)(a.groups6 * c6 + cls_na + nb * cls_cb);
+                if (slots * slot_bytes <= scratch_bytes && cls_cb <= kMaxParts && c6 <= kMaxParts) {
+                    cfg.wk = 4;
+                    a.ks4 = 1;
+                    a.ks6 = (int)c6;
+                    a.groups4b = (int)nb;
+                    a.ks4b = (int)cls_cb;
+                    a.groups4 = (int)cls_na;
+                }
+            }
             a.ksplit = a.ks4;
             // Up to four rows, shared tiles meet in cells (one returning atomic per element and workgroup) instead of
             // being published, counted and gathered: one round trip after the loop instead of three (4096 x 4096 at two
@@ -1036,10 +1084,12 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 a.rule[1] = make_rule(units, (a.ks6 > 0 ? a.ks6 : 1) * cfg.wk);
                 a.wrule[0] = make_wave_rule(units, a.ks4, cfg.wk, young_pct);
                 a.wrule[1] = make_wave_rule(units, a.ks6 > 0 ? a.ks6 : 1, cfg.wk, young_pct);
+                a.wrule_b = make_wave_rule(units, a.ks4b, cfg.wk, young_pct);
             }
-            long long wgs = (long long)a.groups6 * a.ks6 + (long long)a.groups4 * a.ks4;
+            long long wgs = (long long)a.groups6 * a.ks6 + (long long)a.groups4 * a.ks4 + (long long)a.groups4b * a.ks4b;
             a.div[0] = make_div(a.groups4, wgs);
             a.div[1] = make_div(a.groups6, wgs);
+            a.div_b = make_div(a.groups4b > 0 ? a.groups4b : 1, wgs);
             // Tiles shared by several workgroups, more than four rows: the workgroups of a tile may be placed on one XCD
             // (xcd_place in gemm_common.h) and exchange their partial tiles through its L2 instead of through memory:
             // the publishing stores are acknowledged 0.2-0.3 us earlier and the gather is 0.1-0.2 us shorter.  The grid
@@ -1052,6 +1102,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             a.xcd_local = 0;
             bool want_local = cfg.wk == 4 && a.ks4 > 1;
             if (tune.xcd != kUnset) want_local = tune.xcd != 0;
+            if (a.groups4b > 0) want_local = false;
             if (want_local && cfg.id == 1 && cfg.wn == 1 && !a.cells && xcd_placement == 1 && (a.ks4 > 1 || a.ks6 > 1) &&
                 a.ks4 <= kMaxLocalParts && a.ks6 <= kMaxLocalParts) {
                 long long most = 0;
@@ -1073,8 +1124,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             }
             dim3 grid((unsigned)wgs, 1);
             if (tune.verbose)
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d grid=%u%s\n", a.m, prob_n,
-                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, grid.x, a.xcd_local ? " (tiles placed per XCD)" : "");
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d (+ %d tiles in %d parts) grid=%u%s\n", a.m, prob_n,
+                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, a.groups4b, a.ks4b, grid.x, a.xcd_local ? " (tiles placed per XCD)" : "");
             launch_m16_any(cfg, a, g128, grid, st);
         } else {
             gather_pass();

@@ -108,6 +108,12 @@ struct GemmArgs {
     // fields, selected by value: an indexed table makes the compiler copy the argument block to scratch memory.)
     int xcd_local;
     uint32_t xm4_lo, xm4_hi, xm6_lo, xm6_hi;
+    // m <= 16, two classes of INT4 tiles: the first groups4 tiles in ks4 parts each (their workgroups, with the FP6
+    // region's, are the first of the grid: one per CU), the other groups4b tiles in ks4b finer parts (the later
+    // workgroups, which share those CUs).  groups4b == 0: one class.
+    int groups4b, ks4b;
+    WaveRule wrule_b;
+    FastDiv div_b;            // by groups4b
 #ifdef FP6M_TIMELINE
     unsigned long long* timeline;   // 8 realtime-clock stamps per workgroup (performance debugging builds only)
 #endif
@@ -157,6 +163,8 @@ __device__ __forceinline__ void preload_args(const GemmArgs& p)
     asm volatile("" : : "s"(p.xcd_local), "s"(p.xm4_lo), "s"(p.xm4_hi), "s"(p.xm6_lo), "s"(p.xm6_hi));
     asm volatile("" : : "s"(p.wrule[0].lo), "s"(p.wrule[0].ly), "s"(p.wrule[0].eo), "s"(p.wrule[0].ey), "s"(p.wrule[1].lo),
                         "s"(p.wrule[1].ly), "s"(p.wrule[1].eo), "s"(p.wrule[1].ey));
+    asm volatile("" : : "s"(p.groups4b), "s"(p.ks4b), "s"(p.wrule_b.lo), "s"(p.wrule_b.ly), "s"(p.wrule_b.eo), "s"(p.wrule_b.ey),
+                        "s"(p.div_b.d), "s"(p.div_b.magic));
 }
 
 // The XCD (accelerator die: 32 CUs with an L2 of their own) this wave runs on.

@@ -537,6 +537,7 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
     const int wn = wave % WN, wk = wave / WN;
     TileInfo ti;
     int group;
+    bool later = false;                                                  // a tile of the second class of INT4 tiles
     if constexpr (LOCAL) {
         const XcdPlace pl = xcd_place(p, blockIdx.x, p.groups6, p.groups4);
         if (!pl.valid) return;                                           // (the grid is padded to a multiple of eight)
@@ -544,20 +545,27 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
         ti.part = pl.part;
         group = pl.group;
     } else {
-        const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+        // (two classes of INT4 tiles: in launch order, so that the workgroups of the second class are the later ones)
+        const int logical = p.groups4b > 0 ? (int)blockIdx.x : xcd_contiguous_id(blockIdx.x, gridDim.x);
         const int wgs6 = p.groups6 * p.ks6;                              // the FP6 region's workgroups come first
         ti.fp6 = logical < wgs6;
-        const int local = ti.fp6 ? logical : logical - wgs6;
-        const int groups = ti.fp6 ? p.groups6 : p.groups4;
-        // (both entries are read at fixed kernarg offsets and selected by value: an index computed here would turn
+        int local = ti.fp6 ? logical : logical - wgs6;
+        const int wgs4 = p.groups4 * p.ks4;
+        later = !ti.fp6 && local >= wgs4;                                // (never with one class)
+        if (later) local -= wgs4;
+        const int groups = ti.fp6 ? p.groups6 : (later ? p.groups4b : p.groups4);
+        // (the entries are read at fixed kernarg offsets and selected by value: an index computed here would turn
         // into a second, dependent scalar load, which measured 0.4 us before the first weight load)
-        const FastDiv gdiv = {ti.fp6 ? p.div[1].d : p.div[0].d, ti.fp6 ? p.div[1].magic : p.div[0].magic};
+        const FastDiv gdiv = {ti.fp6 ? p.div[1].d : (later ? p.div_b.d : p.div[0].d),
+                              ti.fp6 ? p.div[1].magic : (later ? p.div_b.magic : p.div[0].magic)};
         ti.part = fast_div(gdiv, local);                                 // part-major: neighbours share k, adjoin in n
-        group = local - ti.part * groups;
+        group = local - ti.part * groups + (later ? p.groups4 : 0);
     }
-    const int ks = ti.fp6 ? p.ks6 : p.ks4;
-    const WaveRule wrule = {ti.fp6 ? p.wrule[1].lo : p.wrule[0].lo, ti.fp6 ? p.wrule[1].ly : p.wrule[0].ly,
-                            ti.fp6 ? p.wrule[1].eo : p.wrule[0].eo, ti.fp6 ? p.wrule[1].ey : p.wrule[0].ey};
+    const int ks = ti.fp6 ? p.ks6 : (later ? p.ks4b : p.ks4);
+    const WaveRule wrule = {ti.fp6 ? p.wrule[1].lo : (later ? p.wrule_b.lo : p.wrule[0].lo),
+                            ti.fp6 ? p.wrule[1].ly : (later ? p.wrule_b.ly : p.wrule[0].ly),
+                            ti.fp6 ? p.wrule[1].eo : (later ? p.wrule_b.eo : p.wrule[0].eo),
+                            ti.fp6 ? p.wrule[1].ey : (later ? p.wrule_b.ey : p.wrule[0].ey)};
     ti.tcol = group * WN + wn;
     ti.region_n = ti.fp6 ? p.qc : p.n4;
     const bool tile_valid = ti.tcol * kTileN < ti.region_n;
@@ -585,7 +593,9 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
     }
     FP6M_MARK(p, 2);
     // scratch slots: FP6 groups first (groups6 * ks6 slots), then INT4 groups; counters likewise
-    const int slot_base = region6 ? group * p.ks6 : p.groups6 * p.ks6 + group * p.ks4;
+    const int slot_base = region6 ? group * p.ks6
+                                  : (later ? p.groups6 * p.ks6 + p.groups4 * p.ks4 + (group - p.groups4) * p.ks4b
+                                           : p.groups6 * p.ks6 + group * p.ks4);
     int* counter = p.counters + (region6 ? group : p.groups6 + group);
     wg_finish<WN, WK, CELLS, LOCAL>(p, ti, tile_valid, wn, wk, ks, slot_base, counter, acc, !p.k4 && (ti.fp6 || !G128), smem,
                                     kWaveLds, reinterpret_cast<int*>(smem + NW * kWaveLds),

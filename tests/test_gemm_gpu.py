@@ -220,6 +220,27 @@ def test_partial_tiles_exchanged_through_one_xcd(oracle):
     assert oracle.rel_err(outs[1].cpu().numpy(), c_ref) <= TOL
 
 
+def test_two_classes_of_int4_tiles(oracle, capfd):
+    """The m <= 16 kernel with the INT4 tiles in two classes (as many whole tiles as fill the CUs once, the rest in
+    parts on later workgroups), forced onto small problems by pretending a chip of a few CUs: cells (up to four rows)
+    and partial tiles (beyond), both scale modes, with and without an FP6 region, the second class whole or in two
+    parts; and one-hot rows bit for bit.  The second identical call inside run() also checks that counters and cells
+    are left clean."""
+    import re
+    cases = [(8, 1536, 2048, 256), (9, 1536, 2048, 256), (12, 2304, 2048, 256), (16, 3072, 1024, -1), (20, 3072, 1024, -1)]
+    for cus, n, k, qc in cases:
+        e = {"FP6M_CLS": 1, "FP6M_CUS": cus, "FP6M_VERBOSE": 1}
+        for m in (2, 4, 5, 16):
+            for gs in (-1, 128):
+                run(oracle, m, n, k, qc=qc, gs=gs, env=e)
+        out = capfd.readouterr().err
+        second = [int(x) for x in re.findall(r"\(\+ (\d+) tiles in \d+ parts\)", out)]
+        assert len(second) == 16 and all(x > 0 for x in second), out[-3000:]
+        for gs in (-1, 128):
+            for m in (3, 9, 16):
+                one_hot_case(oracle, m, n, k, qc, gs, {"cls": 1, "cus": cus})
+
+
 def test_eight_row_blocks_per_wave(oracle):
     """The m > 16 kernel with eight 16-row blocks per wave (128-row tiles, accumulators in the accumulation
     registers), forced onto small problems: ragged row tiles, both regions, both scale modes, k splits through the

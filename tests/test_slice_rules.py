@@ -281,3 +281,47 @@ def test_wave_slices_tile_the_k_range_and_favour_the_older_waves():
                                 assert sum(lens[4:]) <= sum(lens[:4])
                         assert max(lens[:4]) - min(lens[:4]) <= 1 and max(lens[4:] or [0]) - min(lens[4:] or [0]) <= 1
                     assert pos == units, (units, ks, wk, pct, rule)
+
+
+# ---- two classes of INT4 tiles in the m <= 16 kernel (gemm_m16_kernel's index arithmetic)
+
+def m16_place(b, groups6, ks6, groups4, ks4, groups4b, ks4b):
+    """workgroup b -> (fp6, tile inside its region, part, parts, slot of its partial tile)"""
+    wgs6 = groups6 * ks6
+    fp6 = b < wgs6
+    local = b if fp6 else b - wgs6
+    wgs4 = groups4 * ks4
+    later = (not fp6) and local >= wgs4
+    if later:
+        local -= wgs4
+    groups = groups6 if fp6 else (groups4b if later else groups4)
+    part = local // groups
+    group = local - part * groups + (groups4 if later else 0)
+    ks = ks6 if fp6 else (ks4b if later else ks4)
+    if fp6:
+        slot = group * ks6 + part
+    elif later:
+        slot = groups6 * ks6 + groups4 * ks4 + (group - groups4) * ks4b + part
+    else:
+        slot = groups6 * ks6 + group * ks4 + part
+    return fp6, group, part, ks, slot
+
+
+def test_two_classes_cover_every_tile_part_once():
+    rng = np.random.default_rng(11)
+    cases = [(2, 2, 252, 1, 22, 11), (0, 0, 24, 1, 8, 3), (2, 4, 4, 2, 6, 2), (1, 1, 1, 1, 1, 1), (2, 2, 10, 1, 0, 1)]
+    cases += [tuple(int(v) for v in (rng.integers(0, 4), rng.integers(1, 9), rng.integers(1, 300), rng.integers(1, 6),
+                                     rng.integers(0, 120), rng.integers(1, 14))) for _ in range(60)]
+    for groups6, ks6, groups4, ks4, groups4b, ks4b in cases:
+        if groups6 == 0:
+            ks6 = 0
+        wgs = groups6 * ks6 + groups4 * ks4 + groups4b * ks4b
+        seen, slots = set(), set()
+        for b in range(wgs):
+            fp6, group, part, ks, slot = m16_place(b, groups6, ks6, groups4, ks4, groups4b, ks4b)
+            assert 0 <= part < ks and 0 <= group < (groups6 if fp6 else groups4 + groups4b)
+            assert ks == (ks6 if fp6 else (ks4 if group < groups4 else ks4b))
+            assert (fp6, group, part) not in seen and slot not in slots and 0 <= slot < wgs
+            seen.add((fp6, group, part))
+            slots.add(slot)
+        assert len(seen) == wgs

@@ -73,7 +73,7 @@ def test_static_scratch_entry_refuses_what_does_not_fit():
     with cabi.tuning(ksplit=8):                                          # 66 tile slots x 8 parts x 32 KiB > 12 MiB
         assert call(L.fp6m_mul_static, A, B, C, s, ws, m, n, k, qc, gs) == cabi.ERR_SCRATCH
         assert call(L.fp6m_mul, A, B, C, s, ws, m, n, k, qc, gs) == cabi.OK      # the region-backed entry shrinks the split
-    assert "use fp6m_mul" in cabi.strerror(cabi.ERR_SCRATCH)
+    assert "fp6m_mul has room" in cabi.strerror(cabi.ERR_SCRATCH)
     assert call(L.fp6m_mul_static, A, B, C, s, ws, m, n, k, qc, gs) == cabi.OK    # the dispatcher's own split fits
     torch.cuda.synchronize()
     assert int(ws.abs().sum()) == 0
