@@ -471,7 +471,8 @@ MSWEEP = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024]
 
 def baseline_cases():
     """(k, n) -> row counts: every shape x M of the benchmark's Llama-2-7B, Llama-2-70B and M-sweep configurations, plus one
-    launch of 1024 rows on a weight of 128 Mi elements."""
+    launch of 1024 rows on a weight of 128 Mi elements and one shape that the m <= 16 kernel runs with its INT4 tiles in two
+    classes."""
     cases = {}
     for k, n in LLAMA7B:
         cases.setdefault((k, n), set()).update([1, 16])                 # config 1 (M = 1) and its M = 16 bench rows
@@ -479,6 +480,7 @@ def baseline_cases():
         cases.setdefault((k, n), set()).update([1, 16])                 # config 2
     cases[(8192, 8192)].update(MSWEEP)                                  # config 3
     cases.setdefault((8192, 16384), set()).add(1024)
+    cases.setdefault((6656, 35328), set()).update([4, 16])              # a few more tiles than CUs: INT4 tiles in two classes
     return sorted((kn, sorted(ms)) for kn, ms in cases.items())
 
 
