@@ -73,6 +73,28 @@ def test_scatter_and_gather_are_exact_reorders(oracle, m):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("m", [3, 16])
+def test_fused_epilogue_with_int4_tiles_in_two_classes(oracle, m):
+    """The scatter, bias-free fused path through the m <= 16 kernel's two-class plan (forced by pretending a chip of
+    eight CUs): an exact reorder of the plain call's result, which takes the same plan."""
+    import fp6_marlin
+    k, n, qc, gs = 2048, 1536, 256, 128
+    print(f"case fused two classes m={m}", flush=True)
+    ref, B, s = packed(oracle, k, n, qc, gs)
+    g = torch.Generator().manual_seed(m)
+    A = torch.randn((m, k), generator=g).half().to(dev())
+    c_cols = torch.randperm(n, generator=g).to(torch.int32).to(dev())
+    with fp6_marlin.cabi.tuning(cls=1, cus=8):
+        want = plain(fp6_marlin, A, B, s, n, qc, gs)
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int32, device=dev())
+        C = torch.full((m, n), float("nan"), dtype=torch.half, device=dev())
+        fp6_marlin.mul_fused(A, B, C, s, ws, qc, gs, c_cols=c_cols)
+        torch.cuda.synchronize()
+    assert torch.equal(C[:, c_cols.long()], want)
+    assert int(ws.abs().sum()) == 0
+    assert oracle.rel_err(want.cpu().numpy(), oracle.matmul_ref(A.cpu().numpy(), ref)) <= TOL
+
+
 @pytest.mark.parametrize("k,n,qc,gs", [(4096, 4096, 256, 128), (4096, 4096, 256, -1), (1024, 768, 256, 128), (2048, 512, -1, 128),
                                        (2048, 512, -1, -1), (1024, 384, 384, -1), (11008, 1024, 128, 128), (8192, 2048, 256, -1)])
 def test_one_row_gather_inside_the_decode_kernel(oracle, k, n, qc, gs):
