@@ -448,6 +448,11 @@ void launch_mb_one(const GemmArgs& a, dim3 grid, hipStream_t stream)
     if constexpr (LEAN && !(MB == 4 && WK == 4 && !G128)) {
         if (!needs_extras(a)) kernel = gemm_mb_kernel<G128, MB, D4, D6, WK, PAIR, false>;
     }
+    // (two classes of INT4 tiles: a build of its own of the configurations the dispatcher plans them for)
+    // (64-row tiles with per-column scales are two registers short of a build of this kind: the dispatcher knows)
+    if constexpr (LEAN && PAIR && MB <= 4 && WK == 8 && !(MB == 4 && !G128)) {
+        if (a.groups4b > 0) kernel = gemm_mb_kernel<G128, MB, D4, D6, WK, PAIR, false, true>;
+    }
     hipLaunchKernelGGL(kernel, grid, dim3(64 * WK), 0, stream, a);
 }
 
@@ -1172,6 +1177,35 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             if (env_ks < 1 && !row_mix && a.tiles6 > 0 && units >= 4 * ks * wk && mb != 8 && mtiles <= 2 &&
                 (base + (long long)a.tiles6 * mtiles) * ks <= resident)
                 a.ks6 = 2 * (int)ks;
+            // One row tile and somewhat more tiles than CUs: workgroups of four waves, two to a CU, run both at little more
+            // than half speed, so the CUs that get two set the launch's length at 1.76 x that of a grid that fits
+            // (8192 x 36864 at 32 rows: 288 tiles 60.9 us, 256 tiles 34.6).  Two classes of INT4 tiles instead (as in the
+            // m <= 16 kernel): as many whole tiles as there are CUs, one workgroup per CU with two waves per SIMD, and the
+            // tiles left over in cb >= 2 parts on workgroups that start as those end: 1 + 1 / cb rounds instead of 1.76.
+            a.groups4b = 0;
+            a.ks4b = 1;
+            const long long tiles4 = a.tiles - a.tiles6;
+            if (!row_mix && !needs_extras(a) && tune.pair == kUnset && mb <= 4 && !(mb == 4 && !g128) && mtiles == 1 && mtiles_total == 1 && sms <= 0 && env_ks < 1 && tune.wk == kUnset && ks == 1 && base > cus &&
+                tiles4 > 0 && !(tune.cls != kUnset && tune.cls == 0)) {
+                const int wk_c = 8;
+                const long long c6 = a.tiles6 && units >= 4 * wk_c ? 2 : 1;
+                const long long first = cus - a.tiles6 * c6;
+                const long long na = tiles4 < first ? tiles4 : first, nb = tiles4 - na;
+                if (first >= 1 && nb > 0 && nb <= cus) {
+                    long long cb = cus / nb;
+                    const long long cb_k = units / (wk_c * 2) > 0 ? units / (wk_c * 2) : 1;     // two k units per wave at least
+                    if (cb > cb_k) cb = cb_k;
+                    if (cb > cap) cb = cap;
+                    while (cb > 1 && (size_t)(a.tiles6 * c6 + nb * cb) * tile_bytes > scratch_bytes) cb--;
+                    if (cb >= 2 || (tune.cls == 1 && cb >= 1)) {
+                        wk = wk_c;
+                        a.ks4 = 1;
+                        a.ks6 = (int)c6;
+                        a.groups4b = (int)nb;
+                        a.ks4b = (int)cb;
+                    }
+                }
+            }
             if (row_mix) {
                 a.slices4 = deal_slices(a.ksplit * wk);
                 a.rule[0] = make_rule(k4 / 128, a.slices4);
@@ -1181,14 +1215,16 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 a.rule[1] = make_rule(units, a.ks6 * wk);
                 a.wrule[0] = make_wave_rule(units, a.ks4, wk, young_pct);
                 a.wrule[1] = make_wave_rule(units, a.ks6, wk, young_pct);
+                a.wrule_b = make_wave_rule(units, a.ks4b, wk, young_pct);
             }
-            const long long wgs = (long long)a.tiles6 * a.ks6 + (long long)(a.tiles - a.tiles6) * a.ks4;
+            const long long wgs = (long long)a.tiles6 * a.ks6 + (tiles4 - a.groups4b) * a.ks4 + (long long)a.groups4b * a.ks4b;
             a.div[0] = make_div(a.ks4, wgs);
             a.div[1] = make_div(a.ks6, wgs);
+            a.div_b = make_div(a.ks4b, wgs);
             dim3 grid((unsigned)wgs, (unsigned)mtiles);
             if (tune.verbose)
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks4=%d ks6=%d k slices %d grid=%ux%u\n", a.m, prob_n,
-                        prob_k, mb, mtiles, a.ks4, a.ks6, wk, grid.x, grid.y);
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: MB=%d row tiles %d ks4=%d ks6=%d (+ %d tiles in %d parts) k slices %d grid=%ux%u\n",
+                        a.m, prob_n, prob_k, mb, mtiles, a.ks4, a.ks6, a.groups4b, a.ks4b, wk, grid.x, grid.y);
             // Every launch of 64-row tiles takes the paired loop (33 rows: -5 % .. +5 % over five shapes, 40 rows 0-9 % faster,
             // 64 rows 9-16 %, from 65 rows on 12-20 %; before the FP6 tiles had it too, whose workgroups set a resident
             // grid's length, it paid from 65 rows on only).  The ring loop stays for the tuning hook and for 32-row tiles in

@@ -152,19 +152,44 @@ __device__ __forceinline__ int xcd_contiguous_id(int b, int total)
 // Kernel arguments are fetched with scalar loads that the compiler otherwise issues where each field is first used:
 // three or four dependent round trips (0.2-0.4 us each on a cold kernarg buffer) before a wave's first weight load.
 // Naming the fields in one asm statement at the top makes them one batch behind a single wait.
+// (Only the fields the kernel uses: all of them at once would not fit the scalar registers, and the compiler would
+// fall back to two batches with spills in between.)  LARGE_M: the m > 16 kernel, which has no use for the m <= 16
+// kernel's tile groups, cells and XCD placement.
+template <bool LARGE_M, bool CLASSES = true>
 __device__ __forceinline__ void preload_args(const GemmArgs& p)
 {
-    asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
-                        "s"(p.scratch), "s"(p.counters), "s"(p.cells));
+    if constexpr (LARGE_M && !CLASSES) {
+        // (the build with the row mix and the fused epilogue: the statements its schedule was tuned with)
+        asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
+                            "s"(p.scratch), "s"(p.counters), "s"(p.cells));
+        asm volatile("" : : "s"(p.m), "s"(p.n), "s"(p.k), "s"(p.n4), "s"(p.qc), "s"(p.tiles6), "s"(p.tiles), "s"(p.ksplit),
+                            "s"(p.ks6), "s"(p.ks4), "s"(p.groups6), "s"(p.groups4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
+        asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
+                            "s"(p.div[0].d), "s"(p.div[0].magic), "s"(p.div[1].d), "s"(p.div[1].magic), "s"(p.fused));
+        asm volatile("" : : "s"(p.xcd_local), "s"(p.xm4_lo), "s"(p.xm4_hi), "s"(p.xm6_lo), "s"(p.xm6_hi));
+        asm volatile("" : : "s"(p.wrule[0].lo), "s"(p.wrule[0].ly), "s"(p.wrule[0].eo), "s"(p.wrule[0].ey), "s"(p.wrule[1].lo),
+                            "s"(p.wrule[1].ly), "s"(p.wrule[1].eo), "s"(p.wrule[1].ey));
+        return;
+    }
+    // (The wait for the batch stands in front of the first statement, and the compiler issues the loads that only later
+    // statements name behind it: the first statement therefore names the fields at the far end of the block as well.)
+    if constexpr (CLASSES)
+        asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
+                            "s"(p.scratch), "s"(p.counters), "s"(gridDim.x), "s"(p.groups4b), "s"(p.ks4b), "s"(p.wrule_b.lo),
+                            "s"(p.wrule_b.ly), "s"(p.wrule_b.eo), "s"(p.wrule_b.ey), "s"(p.div_b.d), "s"(p.div_b.magic));
+    else
+        asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
+                            "s"(p.scratch), "s"(p.counters), "s"(gridDim.x));
     asm volatile("" : : "s"(p.m), "s"(p.n), "s"(p.k), "s"(p.n4), "s"(p.qc), "s"(p.tiles6), "s"(p.tiles), "s"(p.ksplit),
-                        "s"(p.ks6), "s"(p.ks4), "s"(p.groups6), "s"(p.groups4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
+                        "s"(p.ks6), "s"(p.ks4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
     asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
                         "s"(p.div[0].d), "s"(p.div[0].magic), "s"(p.div[1].d), "s"(p.div[1].magic), "s"(p.fused));
-    asm volatile("" : : "s"(p.xcd_local), "s"(p.xm4_lo), "s"(p.xm4_hi), "s"(p.xm6_lo), "s"(p.xm6_hi));
     asm volatile("" : : "s"(p.wrule[0].lo), "s"(p.wrule[0].ly), "s"(p.wrule[0].eo), "s"(p.wrule[0].ey), "s"(p.wrule[1].lo),
                         "s"(p.wrule[1].ly), "s"(p.wrule[1].eo), "s"(p.wrule[1].ey));
-    asm volatile("" : : "s"(p.groups4b), "s"(p.ks4b), "s"(p.wrule_b.lo), "s"(p.wrule_b.ly), "s"(p.wrule_b.eo), "s"(p.wrule_b.ey),
-                        "s"(p.div_b.d), "s"(p.div_b.magic));
+    if constexpr (!LARGE_M) {
+        asm volatile("" : : "s"(p.cells), "s"(p.groups6), "s"(p.groups4));
+        asm volatile("" : : "s"(p.xcd_local), "s"(p.xm4_lo), "s"(p.xm4_hi), "s"(p.xm6_lo), "s"(p.xm6_hi));
+    }
 }
 
 // The XCD (accelerator die: 32 CUs with an L2 of their own) this wave runs on.
@@ -298,6 +323,7 @@ struct TileInfo {
     int region_n;            // columns of the region
     int col0;                // first column of the tile in C
     int a_step0;             // k step of A that step 0 of the wave's weight segment multiplies (row mix: k4 / 32)
+    bool later;              // m > 16: an INT4 tile of the second class (ks4b parts, the grid's last workgroups)
 };
 
 // Row mix: slice `sl` of a tile's slices -> its segment (ti.fp6, ti.a_step0) and its steps there.
@@ -341,19 +367,49 @@ __device__ __forceinline__ PlaneGeometry plane_geometry(const Args& p, const Til
     return g;
 }
 
+// A kernel argument as a value the optimiser cannot look through: it otherwise turns a selection among three arguments
+// into a selection among their addresses and one dependent scalar load (0.2-0.4 us in front of the first weight load).
+__device__ __forceinline__ int held(int v)
+{
+    asm volatile("" : "+s"(v));
+    return v;
+}
+__device__ __forceinline__ uint32_t held(uint32_t v)
+{
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
 // The m > 16 kernel's workgroup: blockIdx.x walks the FP6 tiles' (tile, k part) pairs first (ks6 parts each), then the
 // INT4 tiles' (ks4 parts each); blockIdx.y the row tiles.
+template <bool CLASSES = true>
 __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 {
     TileInfo t;
-    const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // (two classes of INT4 tiles: in launch order, so that the workgroups of the second class are the last to start)
+    const int logical = CLASSES && p.groups4b > 0 ? (int)blockIdx.x : xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int wgs6 = p.tiles6 * p.ks6;
     t.fp6 = logical < wgs6;
-    const int local = t.fp6 ? logical : logical - wgs6;
-    // (both entries are read at fixed offsets and selected by value: an index would become a dependent scalar load)
-    const FastDiv kdiv = {t.fp6 ? p.div[1].d : p.div[0].d, t.fp6 ? p.div[1].magic : p.div[0].magic};
-    t.tcol = fast_div(kdiv, local);
-    t.part = local - t.tcol * (t.fp6 ? p.ks6 : p.ks4);
+    int local = t.fp6 ? logical : logical - wgs6;
+    const int first4 = p.tiles - p.tiles6 - p.groups4b;      // INT4 tiles of the first class
+    // (uniform, like everything here; said so explicitly because the compiler otherwise keeps what hangs on it in vector
+    // registers, and the loops' scalar-base loads need their addresses in scalar ones)
+    t.later = CLASSES && p.groups4b > 0 && __builtin_amdgcn_readfirstlane((int)(!t.fp6 && local >= first4 * p.ks4)) != 0;
+    if (t.later) local -= first4 * p.ks4;
+    // (the entries are read at fixed offsets and selected by value: an index would become a dependent scalar load)
+    FastDiv kdiv;
+    int ks;
+    kdiv = FastDiv{t.fp6 ? p.div[1].d : p.div[0].d, t.fp6 ? p.div[1].magic : p.div[0].magic};
+    ks = t.fp6 ? p.ks6 : p.ks4;
+    if constexpr (CLASSES) {
+        const uint32_t db = held(p.div_b.d), mb = held(p.div_b.magic);
+        const int kb = held(p.ks4b);
+        kdiv = FastDiv{t.later ? db : kdiv.d, t.later ? mb : kdiv.magic};
+        ks = t.later ? kb : ks;
+    }
+    const int q = __builtin_amdgcn_readfirstlane(fast_div(kdiv, local));
+    t.part = local - q * ks;
+    t.tcol = q + (t.later ? first4 : 0);
     t.tile = t.fp6 ? t.tcol : p.tiles6 + t.tcol;
     t.mtile = blockIdx.y;
     t.region_n = t.fp6 ? p.qc : p.n4;
@@ -365,12 +421,17 @@ __device__ __forceinline__ TileInfo locate_tile(const GemmArgs& p)
 // k range of one wave in steps of 32 (two k-blocks).  Units of two steps (four with group scales) keep
 // every wave's step count even and group-aligned.
 template <bool G128, int WK = kWaves>
-__device__ __forceinline__ void wave_k_range(const GemmArgs& p, bool fp6, int part, int wave, int& begin, int& end)
+__device__ __forceinline__ void wave_k_range(const GemmArgs& p, bool fp6, bool later, int part, int wave, int& begin, int& end)
 {
     constexpr int unit_steps = G128 ? 4 : 2;
-    // (both entries are read at fixed offsets and selected by value: an index would become a dependent scalar load)
-    const WaveRule rule = {fp6 ? p.wrule[1].lo : p.wrule[0].lo, fp6 ? p.wrule[1].ly : p.wrule[0].ly,
-                           fp6 ? p.wrule[1].eo : p.wrule[0].eo, fp6 ? p.wrule[1].ey : p.wrule[0].ey};
+    // (the entries are read at fixed offsets and selected by value: an index would become a dependent scalar load)
+    WaveRule rule;
+    if (later) {                                           // (uniform; false at compile time where there is one class)
+        rule = WaveRule{held(p.wrule_b.lo), held(p.wrule_b.ly), held(p.wrule_b.eo), held(p.wrule_b.ey)};
+    } else {
+        rule = WaveRule{fp6 ? p.wrule[1].lo : p.wrule[0].lo, fp6 ? p.wrule[1].ly : p.wrule[0].ly,
+                        fp6 ? p.wrule[1].eo : p.wrule[0].eo, fp6 ? p.wrule[1].ey : p.wrule[0].ey};
+    }
     begin = wave_rule_begin(rule, WK, part, wave) * unit_steps;
     end = wave_rule_begin(rule, WK, part, wave + 1) * unit_steps;
 }

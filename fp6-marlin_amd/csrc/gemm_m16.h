@@ -531,7 +531,7 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
         p.bias = nullptr;
         p.residual = nullptr;
     }
-    preload_args(args);
+    preload_args<false>(args);
     FP6M_MARK(p, 0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: addresses stay on the SALU
     const int wn = wave % WN, wk = wave / WN;
@@ -571,6 +571,7 @@ __global__ __launch_bounds__(64 * WN * WK, WK == 8 || AROWS == 16 ? 2 : 3) void 
     const bool tile_valid = ti.tcol * kTileN < ti.region_n;
     ti.tile = ti.fp6 ? ti.tcol : p.tiles6 + ti.tcol;
     ti.mtile = 0;
+    ti.later = later;
     ti.col0 = (ti.fp6 ? p.n4 : 0) + ti.tcol * kTileN;
 
     constexpr int unit_steps = G128 ? 4 : 2;

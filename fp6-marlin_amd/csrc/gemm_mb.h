@@ -908,10 +908,13 @@ constexpr int mb_wave_lds(int mb, int d4, int d6)
 // calls that use none of them (plain fp6m_mul on reference-order words).  Their run-time branches cost the plain path
 // 2-6 % (4096 x 4096 at 64 rows 15.8 -> 14.8 us, 8192 x 8192 at 512 rows 68.4 -> 67.3): the arguments are overwritten
 // with constants and the compiler removes what hangs on them.
-template <bool G128, int MB, int D4, int D6, int WK, bool PAIR, bool EXTRAS = true>
+// CLASSES: the build (of the one for plain calls) that knows two classes of INT4 tiles: the first in ks4 parts each, the
+// other groups4b tiles in ks4b parts on the last workgroups of the grid (see the dispatcher).
+template <bool G128, int MB, int D4, int D6, int WK, bool PAIR, bool EXTRAS = true, bool CLASSES = false>
 __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb_kernel(const GemmArgs args)
 {
     GemmArgs p = args;
+    static_assert(!CLASSES || !EXTRAS, "two classes of INT4 tiles: plain calls only");
     if constexpr (!EXTRAS) {
         p.k4 = 0;
         p.slices4 = 0;
@@ -929,16 +932,34 @@ __global__ __launch_bounds__(64 * WK, (WK == 4 && MB <= 4) ? 2 : 1) void gemm_mb
     static_assert(WK * kWaveLds + 16 <= 160 * 1024, "LDS of one CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[WK * kWaveLds + 16];
 
-    preload_args(args);
+    preload_args<true, CLASSES>(args);
     FP6M_MARK(p, 0);
-    TileInfo ti = locate_tile(p);
+    // (The build with two classes of INT4 tiles takes tile and k range from the argument block itself: selecting among
+    // fields of the copy, which the builds for plain calls modify, makes the compiler keep the copy in private memory.)
+    TileInfo ti;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int step_begin, step_end;
-    wave_k_range<G128, WK>(p, ti.fp6, ti.part, wave, step_begin, step_end);
+    if constexpr (!CLASSES) {
+        ti = locate_tile<false>(p);
+        wave_k_range<G128, WK>(p, ti.fp6, false, ti.part, wave, step_begin, step_end);
+    } else {
+        ti = locate_tile<true>(args);
+        wave_k_range<G128, WK>(args, ti.fp6, ti.later, ti.part, wave, step_begin, step_end);
+        step_begin = __builtin_amdgcn_readfirstlane(step_begin);         // (uniform: see locate_tile)
+        step_end = __builtin_amdgcn_readfirstlane(step_end);
+    }
     // partial-sum slots, row tile by row tile: the FP6 tiles' (tile, part), then the INT4 tiles'
-    const int ks = ti.fp6 ? p.ks6 : p.ks4;
+    const int groups4b = CLASSES ? held(args.groups4b) : 0, ks4b = CLASSES ? held(args.ks4b) : 1;
+    int ks = ti.fp6 ? p.ks6 : (ti.later ? ks4b : p.ks4);
     const int wgs6 = p.tiles6 * p.ks6;
-    const int slot_base = ti.mtile * (wgs6 + (p.tiles - p.tiles6) * p.ks4) + (ti.fp6 ? ti.tcol * p.ks6 : wgs6 + ti.tcol * p.ks4);
+    const int first4 = p.tiles - p.tiles6 - groups4b;                    // INT4 tiles of the first class (all, as a rule)
+    int slot_base = ti.mtile * (wgs6 + first4 * p.ks4 + groups4b * ks4b) +
+                    (ti.fp6 ? ti.tcol * p.ks6
+                            : (ti.later ? wgs6 + first4 * p.ks4 + (ti.tcol - first4) * ks4b : wgs6 + ti.tcol * p.ks4));
+    if constexpr (CLASSES) {                                             // (uniform: into scalar registers before the loops)
+        ks = __builtin_amdgcn_readfirstlane(ks);
+        slot_base = __builtin_amdgcn_readfirstlane(slot_base);
+    }
     if (p.k4) row_mix_slice(p, ti.part * WK + wave, ti, step_begin, step_end);   // (no FP6 column tiles in a row mix)
 
     f4 acc[MB][8];

@@ -166,8 +166,8 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * "gen" (0: the decode kernel's chunks all of one length), "gen2" / "gen3" (per cent: the share of a SIMD that its planner
  * assumes for the waves of the second / third generation, which sets their chunk lengths), "young" (per cent: the k slice
  * of the second wave of every SIMD in eight-wave workgroups relative to the first one's; 100 = equal slices),
- * "cls" (0: the m <= 16 kernel never puts the INT4 tiles in two classes -- whole tiles on the first workgroups, the
- * rest in parts on later ones --, 1: wherever it can), "cus" (tests: plan for a chip of that many CUs),
+ * "cls" (0: the kernels never put the INT4 tiles in two classes -- whole tiles on the first workgroups, the
+ * rest in parts on later ones --, 1: wherever they can), "cus" (tests: plan for a chip of that many CUs),
  * "verbose" (print every launch's configuration to stderr); knob = NULL clears all overrides.  Unknown knob ->
  * FP6M_ERR_ARG.  Not synchronised with GEMM calls running on other threads.  The library reads no environment
  * variables on a call (FP6M_VERBOSE is looked up once at load time).

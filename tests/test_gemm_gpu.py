@@ -241,6 +241,26 @@ def test_two_classes_of_int4_tiles(oracle, capfd):
                 one_hot_case(oracle, m, n, k, qc, gs, {"cls": 1, "cus": cus})
 
 
+def test_two_classes_of_int4_tiles_beyond_sixteen_rows(oracle, capfd):
+    """The m > 16 kernel's plan for one row tile and somewhat more tiles than CUs (as many whole tiles as there are CUs,
+    the rest in parts on the grid's last workgroups), forced onto small problems by pretending a chip of a few CUs:
+    32-row tiles with both scale modes, 64-row tiles with group scales, the second class in one and in two parts, with
+    and without an FP6 region; and one-hot rows bit for bit."""
+    import re
+    cases = [(8, 1536, 2048, 256, 128), (8, 1536, 4096, 256, 128), (16, 3072, 4096, -1, 128), (8, 1536, 2048, 256, -1),
+             (16, 3072, 2048, -1, -1)]
+    for cus, n, k, qc, gs in cases:
+        e = {"FP6M_CLS": 1, "FP6M_CUS": cus, "FP6M_VERBOSE": 1}
+        rows = (17, 32, 40, 64) if gs == 128 else (17, 32)
+        for m in rows:
+            run(oracle, m, n, k, qc=qc, gs=gs, env=e)
+        out = capfd.readouterr().err
+        second = [int(x) for x in re.findall(r"MB=\d row tiles 1 .*\(\+ (\d+) tiles in \d+ parts\)", out)]
+        assert len(second) == 2 * len(rows) and all(x > 0 for x in second), out[-3000:]
+        for m in rows[1::2]:
+            one_hot_case(oracle, m, n, k, qc, gs, {"cls": 1, "cus": cus})
+
+
 def test_eight_row_blocks_per_wave(oracle):
     """The m > 16 kernel with eight 16-row blocks per wave (128-row tiles, accumulators in the accumulation
     registers), forced onto small problems: ragged row tiles, both regions, both scale modes, k splits through the
