@@ -161,7 +161,7 @@ __device__ __forceinline__ void preload_args(const GemmArgs& p)
     if constexpr (LARGE_M && !CLASSES) {
         // (the build with the row mix and the fused epilogue: the statements its schedule was tuned with)
         asm volatile("" : : "s"(p.A), "s"(p.b_int4), "s"(p.b_fp6_2), "s"(p.b_fp6_4), "s"(p.C), "s"(p.s_int4), "s"(p.s_fp6),
-                            "s"(p.scratch), "s"(p.counters), "s"(p.cells));
+                            "s"(p.scratch), "s"(p.counters), "s"(p.cells), "s"(gridDim.x));
         asm volatile("" : : "s"(p.m), "s"(p.n), "s"(p.k), "s"(p.n4), "s"(p.qc), "s"(p.tiles6), "s"(p.tiles), "s"(p.ksplit),
                             "s"(p.ks6), "s"(p.ks4), "s"(p.groups6), "s"(p.groups4), "s"(p.k4), "s"(p.slices4), "s"(p.native));
         asm volatile("" : : "s"(p.rule[0].q), "s"(p.rule[0].first_long), "s"(p.rule[1].q), "s"(p.rule[1].first_long),
