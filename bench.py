@@ -602,6 +602,87 @@ def sweep(args):
         json.dump(rows, fh, indent=1)
 
 
+def timeline(args):
+    """Per-workgroup clock stamps of one GEMM (python fp6-marlin_amd/build.py --timeline builds the instrumented library):
+    where the launch's time goes, and how far apart its workgroups end.  Stamps, microseconds after the first workgroup's
+    start: decode kernel (one wave per workgroup)  start, first weights landed, loop end, rows formed, atomics issued,
+    -, stored / cell cleared, end;  other kernels  start, first weights landed, loop end, slices summed through LDS,
+    partial tile published, counted, gathered and stored (last arrival only), end."""
+    import ctypes
+    import numpy as np
+    import torch
+    path = os.path.join(ROOT, "fp6-marlin_amd", "fp6_marlin", "libfp6m_timeline.so")
+    if not os.path.exists(path):
+        sys.exit("bench.py --timeline: build the instrumented library first (python fp6-marlin_amd/build.py --timeline)")
+    lib = ctypes.CDLL(path)
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.fp6m_mul.argtypes = [vp] * 4 + [ci] * 3 + [vp, ci, vp] + [ci] * 6
+    lib.fp6m_mul.restype = ci
+    lib.fp6m_init.argtypes = [ci]
+    lib.fp6m_tuning_set.argtypes = [ctypes.c_char_p, ci]
+    assert lib.fp6m_init(0) == 0
+    vals = [int(x) for x in args.timeline.split(",")]
+    m, k, n = vals[:3]
+    qc = vals[3] if len(vals) > 3 else 256
+    gs = vals[4] if len(vals) > 4 else 128
+    for kv in (args.knobs or "").split(","):
+        if kv:
+            name, value = kv.split("=")
+            assert lib.fp6m_tuning_set(name.encode(), int(value)) == 0, f"unknown knob {name}"
+    gen = torch.Generator().manual_seed(0)
+    copies = max(2, min(8, int(640e6 // weight_bytes(k, n, qc, gs)) + 1))
+    probs = [Problem(torch, m, k, n, qc, gs, gen, on_device=True) for _ in range(copies)]
+    stamps = torch.zeros(1 << 20, dtype=torch.int64, device="cuda")
+
+    def call(p):
+        rc = lib.fp6m_mul(p.A.data_ptr(), p.B.data_ptr(), p.C.data_ptr(), p.s.data_ptr(), p.m, p.n, p.k, p.ws.data_ptr(), 0,
+                          torch.cuda.current_stream().cuda_stream, -1, -1, -1, 16, p.qc if p.qc else -1, p.gs)
+        assert rc == 0, rc
+
+    t_end = time.perf_counter() + 0.05                     # clocks as in a running loop
+    while time.perf_counter() < t_end:
+        for p in probs:
+            call(p)
+    torch.cuda.synchronize()
+    os.environ["FP6M_TIMELINE_PTR"] = str(stamps.data_ptr())
+    pct = [0, 10, 50, 90, 99, 100]
+    reps = []
+    for rep in range(16):
+        for p in probs[1:]:                                # (other weights in between: nothing of this one is cached)
+            call(p)
+        stamps.zero_()
+        call(probs[0])
+        torch.cuda.synchronize()
+        t = stamps.cpu().numpy().reshape(-1, 8)
+        used = t[:, 0] != 0
+        t = t[used].astype(np.float64)
+        reps.append(((t - t[:, 0].min()) / 100.0, np.nonzero(used)[0]))      # the clock counts 100 MHz
+    names = ["start", "first weights", "loop end", "rows / slices summed", "atomics out / published", "counted",
+             "stored (last arrival)", "end"]
+    out = {"m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "knobs": args.knobs or "", "workgroups": int(len(reps[0][1])),
+           "kernel_us": round(float(np.mean([r[0][:, 7].max() for r in reps])), 2), "percentiles": pct, "stamps_us": {}}
+    for i, name in enumerate(names):
+        if m == 1 and i == 5:
+            continue                                       # (the decode kernel keeps its hardware id there)
+        rows = [np.percentile(r[0][:, i][r[0][:, i] > 0] if i else r[0][:, i], pct) for r in reps if (r[0][:, i] > 0).any() or i == 0]
+        if rows:
+            out["stamps_us"][name] = [round(float(v), 2) for v in np.mean(rows, axis=0)]
+    # by generation: workgroup index / 8 is the index inside an XCD; the first 4 x CUs / 8 one-wave workgroups of an XCD
+    # (CUs / 8 four-wave ones) start on SIMDs (CUs) of their own, the later ones share
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    per_gen = (4 if m == 1 else 1) * cus // 8
+    gens = {}
+    for r, idx in reps:
+        g = (idx >> 3) // per_gen
+        for gi in np.unique(g):
+            sel = g == gi
+            gens.setdefault(int(gi), []).append([sel.sum(), np.median(r[sel, 2]), np.percentile(r[sel, 7], 50), r[sel, 7].max()])
+    out["by_generation"] = {str(gi): {"workgroups": int(np.mean([x[0] for x in v])), "loop_end_median_us": round(float(np.mean([x[1] for x in v])), 2),
+                                      "end_median_us": round(float(np.mean([x[2] for x in v])), 2),
+                                      "end_max_us": round(float(np.mean([x[3] for x in v])), 2)} for gi, v in sorted(gens.items())}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -618,6 +699,9 @@ def main():
                                                           "quant_cols -1 and 256, per-channel scales, time-weighted speed-up over fp16")
     ap.add_argument("--headline-only", action="store_true", help="skip the other regimes' rows of the JSON line")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
+    ap.add_argument("--timeline", type=str, default=None, help="m,k,n[,quant_cols,group_size]: per-workgroup clock stamps of one GEMM "
+                    "(needs fp6-marlin_amd/build.py --timeline)")
+    ap.add_argument("--knobs", type=str, default=None, help="with --timeline: tuning knobs, name=value[,name=value]")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 256 MiB device copy, then one layer of GEMMs")
     args = ap.parse_args()
@@ -626,6 +710,8 @@ def main():
                  "run with --gpus 1")
     if args.traffic_probe:
         traffic_probe()
+    elif args.timeline:
+        timeline(args)
     elif args.models:
         import torch
         import fp6_marlin

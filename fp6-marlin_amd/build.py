@@ -2,10 +2,13 @@
 
     python fp6-marlin_amd/build.py            # C-ABI library + torch extension
     python fp6-marlin_amd/build.py --no-torch # C-ABI library only
+    python fp6-marlin_amd/build.py --timeline # also the instrumented library that `bench.py --timeline` loads
 
 Outputs (next to the Python package, so they travel with the source tree):
     fp6_marlin/libfp6m.so        C ABI of include/fp6m.h: host packers + HIP kernels (hipcc)
     fp6_marlin/_fp6m_torch.so    thin torch extension that unwraps tensors and calls the C ABI (g++)
+    fp6_marlin/libfp6m_timeline.so   (--timeline) the same library with -DFP6M_TIMELINE: every workgroup of the GEMM
+                                 kernels writes eight clock stamps; a measuring tool, never loaded by the package
 """
 import argparse
 import os
@@ -31,11 +34,11 @@ def run(cmd):
     subprocess.check_call(cmd)
 
 
-def build_lib():
+def build_lib(timeline=False):
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    out = os.path.join(PKG, "libfp6m.so")
+    out = os.path.join(PKG, "libfp6m_timeline.so" if timeline else "libfp6m.so")
     srcs = [os.path.join(CSRC, f) for f in ("fp6m_cpu.cpp", "fp6m_gemm.hip", "fp6m_pack.hip")]
-    run([hipcc, *HIP_FLAGS, "-shared", "-pthread", "-o", out, *srcs])
+    run([hipcc, *HIP_FLAGS, *(["-DFP6M_TIMELINE"] if timeline else []), "-shared", "-pthread", "-o", out, *srcs])
     return out
 
 
@@ -60,8 +63,11 @@ def build_torch_ext():
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-torch", action="store_true")
+    ap.add_argument("--timeline", action="store_true", help="also build the instrumented library for bench.py --timeline")
     args = ap.parse_args(argv)
     build_lib()
+    if args.timeline:
+        build_lib(timeline=True)
     if not args.no_torch:
         build_torch_ext()
 
