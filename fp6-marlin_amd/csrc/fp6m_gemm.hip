@@ -66,7 +66,7 @@ thread_local int g_last_hip_error = 0;
 constexpr int kUnset = INT32_MIN;
 const int g_env_verbose = getenv("FP6M_VERBOSE") ? 1 : 0;
 struct Tuning {
-    int mb = kUnset, ksplit = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset, cls = kUnset, cus = kUnset;
+    int mb = kUnset, ksplit = kUnset, wk16 = kUnset, wk = kUnset, pair = kUnset, wgs = kUnset, share = kUnset, share6 = kUnset, sk = kUnset, cap = kUnset, gather = kUnset, cells = kUnset, xcd = kUnset, gen = kUnset, gen2 = kUnset, gen3 = kUnset, young = kUnset, cls = kUnset, cus = kUnset, cap2 = kUnset;
     int verbose = g_env_verbose;
 };
 Tuning g_tuning;
@@ -488,7 +488,7 @@ int fp6m_tuning_set(const char* knob, int value)
     }
     const struct { const char* name; int* field; } knobs[] = {
         {"mb", &g_tuning.mb}, {"ksplit", &g_tuning.ksplit},
-        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3}, {"young", &g_tuning.young}, {"cls", &g_tuning.cls}, {"cus", &g_tuning.cus},
+        {"wk16", &g_tuning.wk16}, {"wk", &g_tuning.wk}, {"pair", &g_tuning.pair}, {"wgs", &g_tuning.wgs}, {"share", &g_tuning.share}, {"share6", &g_tuning.share6}, {"cap", &g_tuning.cap}, {"sk", &g_tuning.sk}, {"gather", &g_tuning.gather}, {"cells", &g_tuning.cells}, {"xcd", &g_tuning.xcd}, {"gen", &g_tuning.gen}, {"gen2", &g_tuning.gen2}, {"gen3", &g_tuning.gen3}, {"young", &g_tuning.young}, {"cls", &g_tuning.cls}, {"cus", &g_tuning.cus}, {"cap2", &g_tuning.cap2},
         {"verbose", &g_tuning.verbose}};
     for (const auto& k : knobs)
         if (!strcmp(knob, k.name)) {
@@ -838,9 +838,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 const long long cap[3] = {gen_size - chunks6, gen_size,
                                           waves_wanted - 2 * gen_size < gen_size ? waves_wanted - 2 * gen_size : gen_size};
                 const long long min_units = g128 ? 1 : 2;
-                auto fit = [&](long long len) {                        // a length whose last chunk of a tile is not too short
+                // (chunks per tile: 32 for the first generation as in the plan above, 48 for the later ones, whose chunks
+                // must come out a third shorter also on the few tiles of a long k: 17664 x 6656 15.6 -> 13.8 us,
+                // 28672 x 5120 18.05 -> 16.5, 21760 x 8192 19.5 -> 19.0; 13824 x 5120 11.0 -> 11.4; 64 measured like 48)
+                const long long later_cap = tune.cap2 != kUnset && tune.cap2 > 0 ? tune.cap2 : 48;
+                auto fit = [&](long long len, int g) {                 // a length whose last chunk of a tile is not too short
+                    const long long most = g == 0 ? 32 : later_cap;
                     if (len < min_units) len = min_units;
-                    if (len * 32 < u4) len = (u4 + 31) / 32;
+                    if (len * most < u4) len = (u4 + most - 1) / most;
                     while (len < u4 && u4 % len != 0 && u4 % len < min_units) len++;
                     return len > u4 ? u4 : len;
                 };
@@ -850,7 +855,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     long long len[3], cpt[3], t[3], left = tiles4;
                     double cost = 0;
                     for (int g = 0; g < 3; g++) {
-                        len[g] = fit(g == 0 ? (u4 + cpt_a - 1) / cpt_a : (long long)((double)len[0] * e[g] + 0.5));
+                        len[g] = fit(g == 0 ? (u4 + cpt_a - 1) / cpt_a : (long long)((double)len[0] * e[g] + 0.5), g);
                         if (g > 0 && len[g] > len[g - 1]) len[g] = len[g - 1];
                         cpt[g] = (u4 + len[g] - 1) / len[g];
                         t[g] = cap[g] / cpt[g] < left ? cap[g] / cpt[g] : left;

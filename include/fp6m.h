@@ -164,7 +164,8 @@ int fp6m_mul_rows(const void* A, int lda, const void* B, void* C, const void* s,
  * tiles of up to four rows through partial tiles, like those of more rows, instead of in the accumulate-and-count cells),
  * "xcd" (the m <= 16 kernel's partial tiles of 5 to 16 rows exchanged inside one XCD: 1 wherever possible, 0 never),
  * "gen" (0: the decode kernel's chunks all of one length), "gen2" / "gen3" (per cent: the share of a SIMD that its planner
- * assumes for the waves of the second / third generation, which sets their chunk lengths), "young" (per cent: the k slice
+ * assumes for the waves of the second / third generation, which sets their chunk lengths), "cap2" (the most chunks per
+ * tile that it gives those generations), "young" (per cent: the k slice
  * of the second wave of every SIMD in eight-wave workgroups relative to the first one's; 100 = equal slices),
  * "cls" (0: the kernels never put the INT4 tiles in two classes -- whole tiles on the first workgroups, the
  * rest in parts on later ones --, 1: wherever they can), "cus" (tests: plan for a chip of that many CUs),
