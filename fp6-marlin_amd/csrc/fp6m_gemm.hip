@@ -805,6 +805,20 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 cpt6 = (u6 + q6 - 1) / q6;
                 chunks4 = tiles4 * cpt4;
                 chunks6 = (long long)a.tiles6 * cpt6;
+                // An FP6 chunk of half an INT4 chunk's rows takes as long as that one; where the bound on a tile's chunks
+                // leaves the FP6 chunks longer, their waves end last (8192 x 3072: 256-row chunks in both regions 7.6 us,
+                // 128-row FP6 chunks 7.0; 14336 x 4096 10.6 -> 9.5; 5120 x 5120 7.25 -> 6.85).  Up to 64 chunks per
+                // tile then, unless the extra waves start another generation of waves (8192 x 8192: 2048 waves
+                // 10.6 us, 2112 11.5).
+                if (a.tiles6 && tiles4 && max_chunks6 < 64 && tune.share6 == kUnset) {
+                    const long long q6p = chunk_units(u6, want6, 2, 64), cpt6p = (u6 + q6p - 1) / q6p;   // (four steps at least)
+                    const long long gen = 4LL * cus, with = chunks4 + a.tiles6 * cpt6p;
+                    if (q6p < q6 && (with + gen - 1) / gen == (chunks4 + chunks6 + gen - 1) / gen) {
+                        q6 = q6p;
+                        cpt6 = cpt6p;
+                        chunks6 = (long long)a.tiles6 * cpt6;
+                    }
+                }
                 if (chunks4 + chunks6 <= waves_wanted || want4 >= u4 || tune.wgs != kUnset || tune.share != kUnset ||
                     env_ks >= 1 || sms > 0)
                     break;
