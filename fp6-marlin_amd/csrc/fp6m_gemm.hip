@@ -1215,7 +1215,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     const long long cb_k = units / (wk_c * 2) > 0 ? units / (wk_c * 2) : 1;     // two k units per wave at least
                     if (cb > cb_k) cb = cb_k;
                     if (cb > cap) cb = cap;
-                    while (cb > 1 && (size_t)(a.tiles6 * c6 + nb * cb) * tile_bytes > scratch_bytes) cb--;
+                    // (partial-tile slots are numbered over all tiles, the whole ones of the first class included)
+                    while (cb > 1 && (size_t)(a.tiles6 * c6 + na + nb * cb) * tile_bytes > scratch_bytes) cb--;
                     if (cb >= 2 || (tune.cls == 1 && cb >= 1)) {
                         wk = wk_c;
                         a.ks4 = 1;
