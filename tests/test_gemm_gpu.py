@@ -501,6 +501,7 @@ def baseline_cases():
     cases[(8192, 8192)].update(MSWEEP)                                  # config 3
     cases.setdefault((8192, 16384), set()).add(1024)
     cases.setdefault((6656, 35328), set()).update([4, 16])              # a few more tiles than CUs: INT4 tiles in two classes
+    cases.setdefault((8192, 36864), set()).update([32, 64])             # the same in the m > 16 kernel (32- and 64-row tiles)
     return sorted((kn, sorted(ms)) for kn, ms in cases.items())
 
 
