@@ -656,7 +656,8 @@ def timeline(args):
         t = stamps.cpu().numpy().reshape(-1, 8)
         used = t[:, 0] != 0
         t = t[used].astype(np.float64)
-        reps.append(((t - t[:, 0].min()) / 100.0, np.nonzero(used)[0]))      # the clock counts 100 MHz
+        raw = stamps.cpu().numpy().reshape(-1, 8)[used]
+        reps.append(((t - t[:, 0].min()) / 100.0, np.nonzero(used)[0], (raw[:, 5] >> 32) & 15))   # the clock counts 100 MHz
     names = ["start", "first weights", "loop end", "rows / slices summed", "atomics out / published", "counted",
              "stored (last arrival)", "end"]
     out = {"m": m, "k": k, "n": n, "quant_cols": qc, "group_size": gs, "knobs": args.knobs or "", "workgroups": int(len(reps[0][1])),
@@ -672,7 +673,7 @@ def timeline(args):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     per_gen = (4 if m == 1 else 1) * cus // 8
     gens = {}
-    for r, idx in reps:
+    for r, idx, _ in reps:
         g = (idx >> 3) // per_gen
         for gi in np.unique(g):
             sel = g == gi
@@ -680,6 +681,14 @@ def timeline(args):
     out["by_generation"] = {str(gi): {"workgroups": int(np.mean([x[0] for x in v])), "loop_end_median_us": round(float(np.mean([x[1] for x in v])), 2),
                                       "end_median_us": round(float(np.mean([x[2] for x in v])), 2),
                                       "end_max_us": round(float(np.mean([x[3] for x in v])), 2)} for gi, v in sorted(gens.items())}
+    if m == 1:
+        # the decode kernel's waves also note the XCD they run on: the dies do not all stream at the same rate
+        xcds = {}
+        for r, _, xcc in reps:
+            for x in np.unique(xcc):
+                xcds.setdefault(int(x), []).append([np.sum(xcc == x), np.median(r[xcc == x, 2]), r[xcc == x, 7].max()])
+        out["by_xcd"] = {str(x): {"waves": int(np.mean([v[0] for v in vs])), "loop_end_median_us": round(float(np.mean([v[1] for v in vs])), 2),
+                                  "end_max_us": round(float(np.mean([v[2] for v in vs])), 2)} for x, vs in sorted(xcds.items())}
     print(json.dumps(out), flush=True)
 
 
