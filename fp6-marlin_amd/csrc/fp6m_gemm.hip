@@ -1217,7 +1217,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     if (cb > cap) cb = cap;
                     // (partial-tile slots are numbered over all tiles, the whole ones of the first class included)
                     while (cb > 1 && (size_t)(a.tiles6 * c6 + na + nb * cb) * tile_bytes > scratch_bytes) cb--;
-                    if (cb >= 2 || (tune.cls == 1 && cb >= 1)) {
+                    // (64-row tiles in two parts only: 4096 x 33280 .. 45056 at 64 rows 2-4 % slower than one class; three or
+                    // more parts, or 32-row tiles in two: 10-39 % faster over 48 shapes)
+                    if (cb >= (mb == 4 ? 3 : 2) || (tune.cls == 1 && cb >= 1)) {
                         wk = wk_c;
                         a.ks4 = 1;
                         a.ks6 = (int)c6;
