@@ -986,6 +986,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // workgroups per CU (more concurrent k fronts cost DRAM efficiency, fewer leave CUs idle).
             const long long target_wgs = (long long)cus * 3 / 2;
             long long ks = (target_wgs + groups / 2) / groups;
+            double cls_gain = 0.0;
             long long cls_na = 0, cls_cb = 0;                           // two classes of INT4 tiles (below): tiles of the first, parts of the second
             if (ks > ks_limit(cfg.wk)) ks = ks_limit(cfg.wk);
             if (ks < 1) ks = 1;
@@ -1034,31 +1035,28 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 }
                 // Two classes of INT4 tiles.  A few more tiles than CUs leave the grid above lopsided whatever the split
                 // (6656 x 35328: 274 INT4 tiles, so 22 CUs run two workgroups and end at 29 us where the others end at
-                // 19).  So: as many whole tiles as fill every CU once make the first cus workgroups of the grid (with the
-                // FP6 region's); the tiles left over are cut into parts and dealt, as the later workgroups of the grid,
-                // over the CUs a second time.  Model, from the same timelines: while two four-wave workgroups share a
-                // CU the first runs at 0.73 and the second at 0.52 of the rate one has alone (1.25 together); whoever is
-                // left alone runs at full rate.  Measured (16 rows, us): 6656 x 35328 31.4 -> 26.4, 8192 x 43520
-                // 39.0 -> 33.8 (model: 33.7); with the first class split as well (fewer tiles than CUs) every forced
-                // plan lost 5-30 %, so that is not tried.
+                // 19: while two four-wave workgroups share a CU the first runs at 0.73 and the second at 0.52 of the
+                // rate one has alone, so the doubled-up CUs take 1.76 x as long).  So: as many whole tiles as fill every
+                // CU once make the first cus workgroups of the grid (with the FP6 region's); the tiles left over are cut
+                // into cb parts and dealt, as the later workgroups of the grid, over the CUs a second time: 1 + 1 / cb
+                // rounds and a second start instead of 1.76.  Taken where  k / 128 * (0.76 - 1 / cb) >= 7.5:  forced both
+                // ways over 56 shapes (k = 2048 .. 14336, 312 .. 424 tiles, 8 and 16 rows) that is where it won (k = 2048
+                // in four parts -7 .. -12 %, k >= 4096 in two or more -5 .. -19 %) and the rest was within -1 .. +4 %.
+                // With the first class split as well (fewer tiles than CUs) every forced plan lost 5-30 %: not tried.
                 if (!row_mix && cfg.wn == 1 && sms <= 0 && env_ks < 1 && tune.wk16 == kUnset && a.groups4 > 0 &&
                     !(tune.cls != kUnset && tune.cls == 0)) {
-                    const double ra = 0.727, rb = 0.523;
                     const long long c6 = a.groups6 ? ks6_of(1, 4) : 0;
                     const long long first = cus - a.groups6 * c6;                      // workgroups the first round has left
                     const long long na = a.groups4 < first ? a.groups4 : first, nb = a.groups4 - na;
                     if (first >= 1 && nb > 0 && nb <= cus) {                           // (else: one class does it / a third round)
                         // (the few tiles of the second class may be cut finer than a split of all tiles may: their partial
-                        // tiles are a small part of the traffic, and priced below)
+                        // tiles are a small part of the traffic)
                         long long cb = cus / nb;
                         const long long cb_limit = prob_k / 32 / 16 < ks_units(4) ? prob_k / 32 / 16 : ks_units(4);
                         if (cb > cb_limit) cb = cb_limit;
                         if (cb < 1) cb = 1;
-                        const double ua = (double)units, ub = (double)((units + cb - 1) / cb);
-                        const double both = ub / rb <= ua / ra ? ua + ub * (1.0 - ra) / rb : ub + ua * (1.0 - rb) / ra;
-                        const double partial_us = ((cb > 1 ? nb * cb : 0) + (c6 > 1 ? a.groups6 * c6 : 0)) * a.m * 0.0005;
-                        const double us = both * unit_steps / 4 * 0.40 + partial_us;
-                        if (tune.cls == 1 || us < 0.96 * model_us(cfg.wk, ks)) {
+                        cls_gain = prob_k / 128.0 * (0.76 - 1.0 / (double)cb);
+                        if (tune.cls == 1 || (cb >= 2 && cls_gain >= 7.5)) {
                             cls_na = na;
                             cls_cb = cb;
                         }
@@ -1148,8 +1146,8 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             }
             dim3 grid((unsigned)wgs, 1);
             if (tune.verbose)
-                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d (+ %d tiles in %d parts) grid=%u%s\n", a.m, prob_n,
-                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, a.groups4b, a.ks4b, grid.x, a.xcd_local ? " (tiles placed per XCD)" : "");
+                fprintf(stderr, "fp6m_mul m=%d n=%d k=%d: cfg %d (%dx%d waves) groups %d+%d ks4=%d ks6=%d (+ %d tiles in %d parts) gain %.1f grid=%u%s\n", a.m, prob_n,
+                        prob_k, cfg.id, cfg.wn, cfg.wk, a.groups6, a.groups4, a.ks4, a.ks6, a.groups4b, a.ks4b, cls_gain, grid.x, a.xcd_local ? " (tiles placed per XCD)" : "");
             launch_m16_any(cfg, a, g128, grid, st);
         } else {
             gather_pass();
