@@ -1210,14 +1210,20 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 const long long na = tiles4 < first ? tiles4 : first, nb = tiles4 - na;
                 if (first >= 1 && nb > 0 && nb <= cus) {
                     long long cb = cus / nb;
-                    const long long cb_k = units / (wk_c * 2) > 0 ? units / (wk_c * 2) : 1;     // two k units per wave at least
+                    const long long cb_k = prob_k / 1024 > 0 ? prob_k / 1024 : 1;               // 128 rows of k per wave at least
                     if (cb > cb_k) cb = cb_k;
                     if (cb > cap) cb = cap;
                     // (partial-tile slots are numbered over all tiles, the whole ones of the first class included)
                     while (cb > 1 && (size_t)(a.tiles6 * c6 + na + nb * cb) * tile_bytes > scratch_bytes) cb--;
-                    // (64-row tiles in two parts only: 4096 x 33280 .. 45056 at 64 rows 2-4 % slower than one class; three or
-                    // more parts, or 32-row tiles in two: 10-39 % faster over 48 shapes)
-                    if (cb >= (mb == 4 ? 3 : 2) || (tune.cls == 1 && cb >= 1)) {
+                    // Taken by the m <= 16 kernel's measure (rounds saved x 128-row units of k), with a bar that follows the
+                    // rows of 32-row tiles: a ragged tile gains less (the one-class grid's four-wave workgroups get
+                    // faster with fewer rows, the eight-wave ones of this plan hardly); 64-row tiles need twice the
+                    // bar.  Fitted to runs against the one-class grid over 236 shapes (17 .. 64 rows x k = 2048 .. 8192 x
+                    // 264 .. 360 tiles, both scale modes): what these bars take gained 0-33 %, what they leave out
+                    // was within -4 .. +8 % when forced.
+                    const double gain = prob_k / 128.0 * (0.76 - 1.0 / (double)cb);
+                    const double bar = mb == 4 ? 16.0 : 7.5 + 0.37 * (32 - a.m);
+                    if ((cb >= 2 && gain >= bar) || (tune.cls == 1 && cb >= 1)) {
                         wk = wk_c;
                         a.ks4 = 1;
                         a.ks6 = (int)c6;
