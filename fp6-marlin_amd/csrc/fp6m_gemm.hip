@@ -973,7 +973,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             auto ks_limit = [&](int wk) {
                 long long c = prob_k / 32 / (4 * wk) > 0 ? prob_k / 32 / (4 * wk) : 1;
                 if (c > ks_units(wk)) c = ks_units(wk);
-                if (c > traffic_cap) c = traffic_cap;
+                // (a grid that leaves CUs idle even so may split twice as far: 2048 x 2048 .. 6144 at 16 rows 7.6-7.8 -> 6.9-7.3 us)
+                const long long cap = groups * 2 * traffic_cap <= cus ? 2 * traffic_cap : traffic_cap;
+                if (c > cap) c = cap;
                 return c;
             };
             // FP6 tiles are split twice as finely as INT4 tiles (their steps move 1.5x the bytes); with FP6 tiles only
@@ -1010,6 +1012,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         // slower both when CUs hosted two of them and when a quarter or more of the CUs stayed idle
                         // (without a k split of the INT4 tiles there is no tail to lose, so fewer busy CUs still pay)
                         if (load > 1.0 || load < (c == 1 ? 0.5 : 0.65)) return 1e9;
+                        // (and their waves keep five k steps: 2048 x 11264 with per-column scales, 2 parts of four steps
+                        // per wave 8.8 us, four waves x 2 parts 8.0; 4096 x 8192 at 8 rows 4 parts 10.0, 3 parts 9.5)
+                        if (c > 1 && prob_k < 160 * 8 * c) return 1e9;
                         t = 0.56;
                     }
                     auto longest = [&](long long slices) { return (double)((units + slices - 1) / slices) * unit_steps; };
@@ -1032,6 +1037,54 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 if (model_us(best_wk, best) < 0.92 * model_us(cfg.wk, ks)) {
                     cfg.wk = best_wk;
                     ks = best;
+                }
+                // Few tiles on a long k (eight or more parts per tile): eight-wave workgroups cover the same slices
+                // with half the partners, or halve the slices, and beyond eight partners the last arrival's gather costs
+                // more than shorter slices gain (0.16-0.27 us per partner).  8192 x 2048 at 8 rows, us by parts: four waves
+                // 8: 10.1, 12: 9.9, 16: 10.9; eight waves 6: 9.45, 8: 9.43, 12: 10.0; at 16 rows four waves x 8 parts 10.8,
+                // eight x 8 9.8; 14336 x 2048 at 16 rows 12.1 (14 parts) -> 11.2; 8192 x 3072 10.8 -> 10.0.
+                bool few_tiles = false;
+                if (!row_mix && ks >= 8 && tune.wk16 == kUnset && env_ks < 1 && sms <= 0) {
+                    const long long fill = cus * 3 / 4 / groups;                       // (8192 x 4096: 6 parts 10.0, 8 parts 10.5)
+                    long long c = fill < 8 ? fill : 8;
+                    if (c > ks_limit(8)) c = ks_limit(8);
+                    if (c >= 4) {
+                        cfg.wk = 8;
+                        ks = c;
+                        few_tiles = true;
+                    }
+                }
+                // Eight-wave workgroups that fit one per CU and leave at most a third of the CUs idle: the finest such split
+                // that leaves every wave five k steps (3072 x 9216 at 16 rows: eight waves x 3 parts, four steps per wave,
+                // 9.7 us; four waves x 3 parts 8.9).  (Forced tables of 4- and 8-wave workgroups x 1 .. 16 parts: 11008 x 5120 at 8 rows
+                // four waves at best 13.2 us (5 parts), eight waves 11.9 (5 parts: 210 workgroups), and 16.5 from 7
+                // parts on, where they no longer fit; 11008 x 8192 at 5 rows 15.6 -> 13.9; 8192 x 5120 at 16 rows
+                // 11.3 -> 10.8, 5120 x 6144 11.5 -> 10.1.)
+                // On a short k (below 6144) four-wave workgroups that fill nine CUs in ten do better still: their waves
+                // keep twice the steps (5120 x 15360 at 16 rows, 2 parts: four waves 12.4 us, eight 13.0; 4096 x 15360
+                // 11.3 vs 12.2; 2048 x 15360 with per-column scales 9.4 -> 8.3; with fewer CUs busy the eight-wave
+                // ones win, 5120 x 11264 at 6 rows 11.2 vs 12.4, and from k = 6656 on they do anyway).
+                if (!row_mix && !few_tiles && ks >= 2 && tune.wk16 == kUnset && env_ks < 1 && sms <= 0) {
+                    auto fit = [&](int wk, long long& c) {
+                        auto wgs_fit = [&](long long cc) { return a.groups4 * cc + a.groups6 * (a.groups6 ? ks6_of(cc, wk) : 0); };
+                        c = ks_limit(wk);
+                        while (c >= 2 && (wgs_fit(c) > cus || prob_k < 160 * wk * c)) c--;   // (five k steps per wave at least)
+                        return c >= 2 ? wgs_fit(c) : 0LL;
+                    };
+                    long long c4 = 0, c8 = 0;
+                    const long long w4 = prob_k < 6144 ? fit(4, c4) : 0, w8 = fit(8, c8);
+                    if (10 * w4 >= 9 * cus) {
+                        cfg.wk = 4;
+                        ks = c4;
+                    } else if (100 * w8 >= 68 * cus) {
+                        cfg.wk = 8;
+                        ks = c8;
+                    } else if (prob_k < 4096 && cfg.wk == 4 && 100 * w4 >= 68 * cus) {
+                        // (a short k with some CUs hosting two workgroups and some one: 2048 x 11264 at 6 rows, per-column
+                        // scales, 4 parts = 360 workgroups 9.0 us, 2 parts = 180 7.7)
+                        const long long now = a.groups4 * ks + a.groups6 * (a.groups6 ? ks6_of(ks, 4) : 0);
+                        if (now > cus && 100 * now < 145 * cus) ks = c4;
+                    }
                 }
                 // Two classes of INT4 tiles.  A few more tiles than CUs leave the grid above lopsided whatever the split
                 // (6656 x 35328: 274 INT4 tiles, so 22 CUs run two workgroups and end at 29 us where the others end at
@@ -1133,8 +1186,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     const long long w = c6 * a.ks6 + c4 * a.ks4;
                     most = w > most ? w : most;
                 }
-                // (no XCD may get more workgroups than its CUs hold at once: two of four waves each)
-                if (most < 8192 && (tune.xcd != kUnset || 8 * most <= 2LL * cus)) {
+                // (no XCD may get more workgroups than its CUs hold at once: two of four waves each; and a grid that fits
+                // one workgroup per CU must still do so on every XCD: 3072 x 4608 at 6 rows in 6 parts, 228 workgroups,
+                // up to 42 on an XCD: 9.1 us against 7.8 in 4 parts)
+                if (most < 8192 && (tune.xcd != kUnset || (8 * most <= 2LL * cus && (wgs > cus || 8 * most <= cus)))) {
                     a.xcd_local = 1;
                     wgs = 8 * most;
                     auto magic32 = [](int d) { return d >= 2 ? (uint32_t)((0x100000000ULL + d - 1) / (unsigned long long)d) : 0u; };
