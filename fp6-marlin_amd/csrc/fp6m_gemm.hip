@@ -1225,12 +1225,28 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // k slices instead of four (same partial-sum traffic, two waves per SIMD) when k is long enough.
             // (Two waves on a SIMD take turns at its one VALU/MFMA port: eight half-length slices last as long as four
             // whole ones, so eight (which hide latency better: 13824 x 5120 at 256 rows 60.6 vs 67.8 us) only pay while
-            // their longest slice, in whole k units, is no more than 0.55 of the longest of four: 5120 x 13824 at 64
-            // rows, 40 units over 16 slices 24.1 us, over 8 slices 21.7.)
-            const long long longest8 = (units + 8 * ks - 1) / (8 * ks), longest4 = (units + 4 * ks - 1) / (4 * ks);
-            int wk = base * ks <= cus && units / 16 >= ks && 20 * longest8 <= 11 * longest4 ? 8 : kWaves;
+            // their longest slice, in whole k units, is no more than 0.58 of the longest of four: 5120 x 13824 at 64
+            // rows, 40 units over 16 slices of up to 3: 24.1 us, over 8 slices of 5: 21.7.)
+            // From forced tables (4 or 8 slices x 1 .. 8 parts, 32 / 64 / 128 rows): a split is no finer than its longest
+            // slice needs (8192 x 6144 at 32 rows: 64 units in 5 parts = 20 slices of up to 4, 16.7 us; in 4 parts = 16
+            // slices of 4, 16.0; as eight-wave workgroups 14.3); one unit per wave is enough for eight (8192 x 2048 at
+            // 32 rows 12.8 -> 12.0); 0.58 rather than 0.55 (14336 x 8192 at 32 rows, 4 against 7 units, 23.0 -> 20.5);
+            // and beyond eight parts the partners' partial tiles cost more than shorter slices gain (14336 x 2048 at
+            // 32 rows: 14 parts of four slices 16.7 us, 8 parts of eight 14.8; at 64 rows 24.0 -> 21.0).
+            auto longest = [&](long long slices) { return (units + slices - 1) / slices; };
+            const bool free_split = env_ks < 1 && sms <= 0 && !row_mix && mb != 8;
+            if (free_split)
+                while (ks > 1 && longest(4 * (ks - 1)) == longest(4 * ks)) ks--;
+            int wk = base * ks <= cus && units / 8 >= ks && 50 * longest(8 * ks) <= 29 * longest(4 * ks) ? 8 : kWaves;
+            if (free_split && tune.wk == kUnset && ks > 8 && base * 8 <= cus && units / 8 >= 8) {
+                wk = 8;
+                ks = 8;
+            }
             if (tune.wk != kUnset) wk = tune.wk == 8 ? 8 : kWaves;
             if (mb == 8) wk = kWaves;                                  // (512 registers per wave: one wave per SIMD)
+            if (free_split && wk == 8)
+                while (ks > 1 && longest(8 * (ks - 1)) == longest(8 * ks)) ks--;
+            a.ksplit = (int)ks;
             // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
             // FP6 tiles' workgroups set the length of the launch (8192 x 8192 at m = 128: 33 us against 29 us with INT4
             // only).  Their k range is cut twice as finely where every slice still gets two units and the grid still
