@@ -1048,7 +1048,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     const long long fill = cus * 3 / 4 / groups;                       // (8192 x 4096: 6 parts 10.0, 8 parts 10.5)
                     long long c = fill < 8 ? fill : 8;
                     if (c > ks_limit(8)) c = ks_limit(8);
-                    if (c >= 4) {
+                    // (eight parts of four waves against fewer of eight: even at 16 rows, 13 % slower at 2 and 4 rows,
+                    // where partners meet in cells: 4096 x 2560 6.7 vs 7.6 us)
+                    if (c >= 4 && (ks > 8 || c == 8 || a.m > 4)) {
                         cfg.wk = 8;
                         ks = c;
                         few_tiles = true;
@@ -1068,7 +1070,9 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     auto fit = [&](int wk, long long& c) {
                         auto wgs_fit = [&](long long cc) { return a.groups4 * cc + a.groups6 * (a.groups6 ? ks6_of(cc, wk) : 0); };
                         c = ks_limit(wk);
-                        while (c >= 2 && (wgs_fit(c) > cus || prob_k < 160 * wk * c)) c--;   // (five k steps per wave at least)
+                        // (five k steps per wave at least; a CU per XCD stays free: a grid of exactly as many workgroups as
+                        // CUs ran 5-11 % slower than the next coarser split, 2048 x 8192 at 4 rows 8.3 vs 7.4 us)
+                        while (c >= 2 && (wgs_fit(c) > cus - cus / 32 || prob_k < 160 * wk * c)) c--;
                         return c >= 2 ? wgs_fit(c) : 0LL;
                     };
                     long long c4 = 0, c8 = 0;
@@ -1085,6 +1089,13 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         const long long now = a.groups4 * ks + a.groups6 * (a.groups6 ? ks6_of(ks, 4) : 0);
                         if (now > cus && 100 * now < 145 * cus) ks = c4;
                     }
+                }
+                // A grid of exactly (or all but) as many workgroups as CUs is slower than the next coarser split (2048 x 8192
+                // at 4 rows: 4 parts = 256 workgroups 8.3 us, 3 parts 7.4; 4096 x 4096: 8 parts 8.3, 6 parts 7.4): one CU
+                // per XCD stays free.
+                if (!row_mix && tune.wk16 == kUnset && env_ks < 1 && sms <= 0) {
+                    auto wgs_of = [&](long long cc) { return a.groups4 * cc + a.groups6 * (a.groups6 ? ks6_of(cc, cfg.wk) : 0); };
+                    while (ks >= 2 && wgs_of(ks) <= cus && wgs_of(ks) > cus - cus / 32) ks--;
                 }
                 // Two classes of INT4 tiles.  A few more tiles than CUs leave the grid above lopsided whatever the split
                 // (6656 x 35328: 274 INT4 tiles, so 22 CUs run two workgroups and end at 29 us where the others end at
