@@ -823,6 +823,19 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     env_ks >= 1 || sms > 0)
                     break;
             }
+            // Chunks of 128 rows (four steps, one more than the fetch side runs ahead) are mostly fill and drain: where they
+            // would come in more than one generation of waves, 256 rows do better as long as those still give two thirds
+            // of the SIMDs a wave (4096 x 6144: 1472 waves of 128 rows 7.1-7.5 us, 736 of 256 rows 6.7; 3072 x 8192
+            // 7.1 -> 6.5; 2048 x 12288 6.8 -> 6.4).
+            if (tiles4 > 0 && q4 * (g128 ? 128 : 64) == 128 && 2 * q4 <= u4 && chunks4 + chunks6 > 4LL * cus && cells_fit &&
+                tune.wgs == kUnset && tune.share == kUnset && env_ks < 1 && sms <= 0 && !(tune.gen != kUnset && tune.gen == 0)) {
+                const long long q2 = 2 * q4, cpt2 = (u4 + q2 - 1) / q2;
+                if (3 * (tiles4 * cpt2 + chunks6) >= 2 * 4LL * cus && (u4 % q2 == 0 || u4 % q2 >= (g128 ? 1 : 2))) {
+                    q4 = q2;
+                    cpt4 = cpt2;
+                    chunks4 = tiles4 * cpt4;
+                }
+            }
             // Waves: one per chunk, up to the number aimed at, which is dealt to the regions by their chunks.
             long long w6 = chunks6, w4 = chunks4;
             if (w4 + w6 > waves_wanted) {
