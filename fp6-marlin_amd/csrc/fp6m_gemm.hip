@@ -773,7 +773,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             long long want6 = 1;
             if (tune.wgs != kUnset) want4 = 1;                         // (tests: few waves, many chunks each)
             const bool cells_fit = (size_t)prob_n * a.m * sizeof(unsigned long long) <= kCellBytes;
-            auto chunk_units = [&](long long units_r, long long want, long long min_units, long long max_chunks) {
+            auto chunk_units = [&](long long units_r, long long want, long long min_units, long long max_chunks, bool fp6_region) {
                 const long long floor_q = (units_r + max_chunks - 1) / max_chunks;
                 long long q = want > floor_q ? want : floor_q;
                 if (q < units_r) {                                     // a divisor of the tile nearby
@@ -786,7 +786,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     if (best) q = best;
                 }
                 if (tune.share != kUnset && tune.share > 0) q = tune.share;
-                if (max_chunks != 32 && tune.share6 != kUnset && tune.share6 > 0) q = tune.share6;
+                if (fp6_region && tune.share6 != kUnset && tune.share6 > 0) q = tune.share6;
                 if (env_ks >= 1) q = (units_r + env_ks - 1) / env_ks;
                 if (sms > 1 && q * sms < units_r) q = (units_r + sms - 1) / sms;
                 if (q < min_units) q = min_units;
@@ -799,8 +799,10 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             long long q4, q6, cpt4, cpt6, chunks4, chunks6;
             for (;; want4++) {                                         // (a last, shorter chunk per tile may push the count over)
                 want6 = g128 ? want4 : (want4 + 1) / 2;
-                q4 = chunk_units(u4, want4, g128 ? 1 : 2, 32);
-                q6 = chunk_units(u6, want6, 1, max_chunks6);
+                // (40 chunks per tile where so few tiles would otherwise leave SIMDs without a wave: 14336 x 2048, 14
+                // INT4 tiles, 28 chunks of 512 rows 8.85 us, 38 of 384 rows 8.2)
+                q4 = chunk_units(u4, want4, g128 ? 1 : 2, tiles4 * 40 <= 3LL * cus ? 40 : 32, false);
+                q6 = chunk_units(u6, want6, 1, max_chunks6, true);
                 cpt4 = (u4 + q4 - 1) / q4;
                 cpt6 = (u6 + q6 - 1) / q6;
                 chunks4 = tiles4 * cpt4;
@@ -811,7 +813,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                 // tile then, unless the extra waves start another generation of waves (8192 x 8192: 2048 waves
                 // 10.6 us, 2112 11.5).
                 if (a.tiles6 && tiles4 && max_chunks6 < 64 && tune.share6 == kUnset) {
-                    const long long q6p = chunk_units(u6, want6, 2, 64), cpt6p = (u6 + q6p - 1) / q6p;   // (four steps at least)
+                    const long long q6p = chunk_units(u6, want6, 2, 64, true), cpt6p = (u6 + q6p - 1) / q6p;   // (four steps at least)
                     const long long gen = 4LL * cus, with = chunks4 + a.tiles6 * cpt6p;
                     if (q6p < q6 && (with + gen - 1) / gen == (chunks4 + chunks6 + gen - 1) / gen) {
                         q6 = q6p;
