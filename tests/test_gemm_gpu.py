@@ -491,8 +491,8 @@ MSWEEP = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024]
 
 def baseline_cases():
     """(k, n) -> row counts: every shape x M of the benchmark's Llama-2-7B, Llama-2-70B and M-sweep configurations, plus one
-    launch of 1024 rows on a weight of 128 Mi elements and one shape that the m <= 16 kernel runs with its INT4 tiles in two
-    classes."""
+    launch of 1024 rows on a weight of 128 Mi elements, shapes that both workgroup kernels run with their INT4 tiles in two
+    classes, and shapes picked for the other branches of the planners."""
     cases = {}
     for k, n in LLAMA7B:
         cases.setdefault((k, n), set()).update([1, 16])                 # config 1 (M = 1) and its M = 16 bench rows
@@ -502,6 +502,14 @@ def baseline_cases():
     cases.setdefault((8192, 16384), set()).add(1024)
     cases.setdefault((6656, 35328), set()).update([4, 16])              # a few more tiles than CUs: INT4 tiles in two classes
     cases.setdefault((8192, 36864), set()).update([32, 64])             # the same in the m > 16 kernel (32- and 64-row tiles)
+    # shapes that take the planners' other branches: few tiles on a long k (eight-wave workgroups, at most eight parts; 40
+    # chunks per tile at one row), splits that fit one workgroup per CU (eight waves, and four on a short k), a split no
+    # finer than its longest slice needs, 256-row chunks at one row
+    cases.setdefault((14336, 2048), set()).update([1, 8, 16, 32, 64])
+    cases.setdefault((11008, 5120), set()).update([8, 48])
+    cases.setdefault((5120, 15360), set()).update([6, 16])
+    cases.setdefault((8192, 6144), set()).update([1, 32, 64])
+    cases.setdefault((4096, 6144), set()).update([1, 4])
     return sorted((kn, sorted(ms)) for kn, ms in cases.items())
 
 
