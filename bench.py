@@ -692,6 +692,79 @@ def timeline(args):
     print(json.dumps(out), flush=True)
 
 
+def regret(args):
+    """The planners against forced plans: for each shape the default call and every forced (waves per workgroup, k parts)
+    plan of the kernel that serves that row count (m = 1: forced uniform chunk lengths), all replayed from HIP graphs over
+    rotated weights; `regret` = default time / best forced time - 1.  --regret KIND[,GROUP_SIZE] with KIND decode (m = 1),
+    m16 (m = 6 and 16) or mb (m = 32, 64, 128); the shapes are k = 2048 .. 11008 x 20 .. 172 column tiles unless --shape
+    names one.  This is how the dispatcher's rules were fitted; on another chip it shows where they no longer hold."""
+    import torch
+    import fp6_marlin
+    from fp6_marlin import cabi
+    kind, _, gs_text = args.regret.partition(",")
+    gs = int(gs_text) if gs_text else 128
+    assert kind in ("decode", "m16", "mb"), "--regret decode|m16|mb[,group_size]"
+    fp6_marlin.init(0)
+    gen = torch.Generator().manual_seed(0)
+    rows = {"decode": [1], "m16": [6, 16], "mb": [32, 64, 128]}[kind]
+    if args.shape:
+        m, k, n = [int(x) for x in args.shape.split(",")[:3]]
+        shapes = [(m, k, n)]
+    else:
+        shapes = [(m, k, t * 128) for m in rows for k in (2048, 3072, 4096, 5120, 8192, 11008)
+                  for t in (20, 32, 44, 60, 72, 88, 104, 120, 172)]
+    parts = (1, 2, 3, 4, 5, 6, 8, 10, 12, 16)
+
+    def plans(m, k):
+        if kind == "decode":
+            units = k // (128 if gs == 128 else 64)
+            return [{"share": q} for q in parts if q <= units]
+        if kind == "m16":
+            return [{"wk16": wk, "ksplit": c} for wk in (4, 8) for c in parts if c <= 8 and k // (32 * wk * c) >= 2]
+        blocks = [2, 4] if m <= 32 else ([4] if m <= 64 else [4, 8])
+        return [{"mb": b, "wk": wk, "ksplit": c} for b in blocks for wk in ((4, 8) if b != 8 else (4,)) for c in parts
+                if c <= 8 and k // (32 * wk * c) >= 2]
+
+    def knobs(plan):
+        cabi.lib.fp6m_tuning_set(None, 0)
+        for name, value in plan.items():
+            assert cabi.lib.fp6m_tuning_set(name.encode(), int(value)) == 0, name
+
+    worst, total, count = 0.0, 0.0, 0
+    for m, k, n in shapes:
+        qc = 256
+        copies = max(2, min(24, int(640e6 // weight_bytes(k, n, qc, gs)) + 1))
+        probs = [Problem(torch, m, k, n, qc, gs, gen, on_device=True) for _ in range(copies)]
+        iters = copies * max(1, 48 // copies)
+        fns = []
+        for plan in [{}] + plans(m, k):
+            knobs(plan)
+            try:
+                probs[0].run(fp6_marlin.mul)
+                torch.cuda.synchronize()
+                fns.append((plan,) + graphed(torch, lambda i: probs[i % copies].run(fp6_marlin.mul), copies, iters))
+            except RuntimeError:                                         # (a forced plan the scratch cannot hold)
+                torch.cuda.synchronize()
+        cabi.lib.fp6m_tuning_set(None, 0)
+        times = {}
+        for _ in range(2):
+            for plan, fn, calls in fns:
+                settle(torch, fn, calls, ms=15)
+                _, ev = time_region(torch, fn, calls)
+                key = json.dumps(plan, sort_keys=True)
+                times[key] = min(times.get(key, 1e9), ev / iters * 1e6)
+        default = times.pop("{}")
+        best = min(times, key=times.get)
+        r = default / times[best] - 1.0
+        worst, total, count = max(worst, r), total + max(r, 0.0), count + 1
+        print(json.dumps({"m": m, "k": k, "n": n, "group_size": gs, "default_us": round(default, 2), "best_forced_us": round(times[best], 2),
+                          "best_forced": json.loads(best), "regret": round(r, 4)}), flush=True)
+        del probs, fns
+        torch.cuda.empty_cache()
+    print(json.dumps({"kind": kind, "group_size": gs, "shapes": count, "mean_regret": round(total / count, 4), "worst_regret": round(worst, 4)}),
+          flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -711,6 +784,8 @@ def main():
     ap.add_argument("--timeline", type=str, default=None, help="m,k,n[,quant_cols,group_size]: per-workgroup clock stamps of one GEMM "
                     "(needs fp6-marlin_amd/build.py --timeline)")
     ap.add_argument("--knobs", type=str, default=None, help="with --timeline: tuning knobs, name=value[,name=value]")
+    ap.add_argument("--regret", type=str, default=None, help="decode|m16|mb[,group_size]: the default plan against every forced plan "
+                    "(with --shape m,k,n: that shape only)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: one 256 MiB device copy, then one layer of GEMMs")
     args = ap.parse_args()
@@ -719,6 +794,8 @@ def main():
                  "run with --gpus 1")
     if args.traffic_probe:
         traffic_probe()
+    elif args.regret:
+        regret(args)
     elif args.timeline:
         timeline(args)
     elif args.models:

@@ -1237,8 +1237,14 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             // of fp32, so the split is also capped by their traffic relative to the weight stream.
             const long long base = (long long)a.tiles * mtiles;
             long long ks = cus / base;
-            const long long ks_k = units / (kWaves * 2) > 0 ? units / (kWaves * 2) : 1;
-            const long long cap = (long long)prob_k / (16LL * rows_per_tile) > 0 ? (long long)prob_k / (16LL * rows_per_tile) : 1;
+            // (two k units per wave at least, one on a short k up to four parts; a grid that leaves half of the CUs idle even
+            // so may split twice as far as the partial tiles' traffic would otherwise allow: 2048 x 2560 .. 7680 at 32 and
+            // 64 rows 10.4 -> 9.2-9.8 us and 13.8 -> 12.7-13.0; eight parts instead of four on k = 4096 cost 6-12 %)
+            long long ks_k = units / (kWaves * 2);
+            if (ks_k < 4) ks_k = units / kWaves < 4 ? units / kWaves : 4;
+            if (ks_k < 1) ks_k = 1;
+            long long cap = (long long)prob_k / (16LL * rows_per_tile) > 0 ? (long long)prob_k / (16LL * rows_per_tile) : 1;
+            if (base * 2 * cap <= cus) cap *= 2;
             if (ks > ks_k) ks = ks_k;
             if (ks > cap) ks = cap;
             if (sms > 0 && ks > sms) ks = sms;
@@ -1263,15 +1269,15 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
             const bool free_split = env_ks < 1 && sms <= 0 && !row_mix && mb != 8;
             if (free_split)
                 while (ks > 1 && longest(4 * (ks - 1)) == longest(4 * ks)) ks--;
-            int wk = base * ks <= cus && units / 8 >= ks && 50 * longest(8 * ks) <= 29 * longest(4 * ks) ? 8 : kWaves;
+            // (32-row tiles are not issue-bound: two waves per SIMD pay up to two thirds, 11008 x 2560 at 32 rows 14.9 -> 13.2)
+            const bool eight_pays = mb == 2 ? 3 * longest(8 * ks) <= 2 * longest(4 * ks) : 50 * longest(8 * ks) <= 29 * longest(4 * ks);
+            int wk = base * ks <= cus && units / 8 >= ks && eight_pays ? 8 : kWaves;
             if (free_split && tune.wk == kUnset && ks > 8 && base * 8 <= cus && units / 8 >= 8) {
                 wk = 8;
                 ks = 8;
             }
             if (tune.wk != kUnset) wk = tune.wk == 8 ? 8 : kWaves;
             if (mb == 8) wk = kWaves;                                  // (512 registers per wave: one wave per SIMD)
-            if (free_split && wk == 8)
-                while (ks > 1 && longest(8 * (ks - 1)) == longest(8 * ks)) ks--;
             a.ksplit = (int)ks;
             // An FP6 step costs more issue slots than an INT4 one, and in a grid that is resident all at once the few
             // FP6 tiles' workgroups set the length of the launch (8192 x 8192 at m = 128: 33 us against 29 us with INT4
