@@ -1102,7 +1102,7 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                         // (a short k with some CUs hosting two workgroups and some one: 2048 x 11264 at 6 rows, per-column
                         // scales, 4 parts = 360 workgroups 9.0 us, 2 parts = 180 7.7)
                         const long long now = a.groups4 * ks + a.groups6 * (a.groups6 ? ks6_of(ks, 4) : 0);
-                        if (now > cus && 100 * now < 145 * cus) ks = c4;
+                        if (now > cus && now < 2LL * cus) ks = c4;           // (2048 x 13312, 424 workgroups: 9.4 us; 212: 7.85)
                     }
                 }
                 // A grid of exactly (or all but) as many workgroups as CUs is slower than the next coarser split (2048 x 8192
