@@ -838,6 +838,35 @@ int mul_common(const void* A, const void* B, void* C, const void* s, int prob_m,
                     chunks4 = tiles4 * cpt4;
                 }
             }
+            // Few tiles and little work (at most a quarter as many INT4 tiles as CUs, 3.5 units per SIMD) in somewhat more
+            // chunks than one generation of waves: the waves beyond the first generation start when those end and are
+            // the launch's tail.  One generation of longer chunks instead, the FP6 chunks at half the INT4 chunks' rows
+            // (best of ten forced lengths against the plan above: 8192 x 5632 1472 waves 9.6 us, 1010 waves 8.4;
+            // 8192 x 7680 10.7 vs 9.6; 8192 x 6144 9.8 vs 9.25; with more work per SIMD generations of different
+            // lengths win, 14336 x 8192 14.2 vs 15.0, and with more tiles too, 4096 x 12288 by up to 6 %).
+            if (tiles4 > 0 && 4 * tiles4 <= cus && 2 * work4 <= 7 * 4LL * cus && chunks4 + chunks6 > 4LL * cus && cells_fit &&
+                tune.wgs == kUnset && tune.share == kUnset && tune.share6 == kUnset && env_ks < 1 && sms <= 0 &&
+                !(tune.gen != kUnset && tune.gen == 0)) {
+                const long long min4 = g128 ? 1 : 2;
+                for (long long q = q4; q <= u4; q++) {
+                    if (q < u4 && u4 % q != 0 && u4 % q < min4) continue;
+                    long long p6 = q * (g128 ? 128 : 64) / 128;                       // FP6 units (64 rows) in half the rows
+                    if (p6 < q6) p6 = q6;
+                    if (p6 > u6) p6 = u6;
+                    while (p6 < u6 && u6 % p6 != 0 && u6 % p6 < 2) p6++;
+                    const long long c4 = tiles4 * ((u4 + q - 1) / q), c6 = a.tiles6 ? a.tiles6 * ((u6 + p6 - 1) / p6) : 0;
+                    if (c4 + c6 > 4LL * cus) continue;
+                    q4 = q;
+                    cpt4 = (u4 + q4 - 1) / q4;
+                    chunks4 = c4;
+                    if (a.tiles6) {
+                        q6 = p6;
+                        cpt6 = (u6 + q6 - 1) / q6;
+                        chunks6 = c6;
+                    }
+                    break;
+                }
+            }
             // Waves: one per chunk, up to the number aimed at, which is dealt to the regions by their chunks.
             long long w6 = chunks6, w4 = chunks4;
             if (w4 + w6 > waves_wanted) {
